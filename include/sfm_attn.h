@@ -1,0 +1,145 @@
+/* sfm_attn.h -- C ABI of the MI355X (gfx950) Monarch / KV-cache attention library.
+ *
+ * Plain pointers and sizes only; every entry point returns 0 on success or a negative
+ * SFM_ERR_* code, never aborts, allocates nothing, keeps no global state besides a
+ * thread-local error string, and enqueues its work on the hipStream_t passed as `stream`
+ * (NULL = the default stream) without synchronising.  All tensor pointers are device
+ * pointers; strides are in ELEMENTS; the innermost (head_dim) axis is contiguous.
+ *
+ * Citations are file:line of the reference (krishagarwal/Self-Forcing) interface each
+ * entry point replaces.
+ */
+#ifndef SFM_ATTN_H
+#define SFM_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SFM_OK               0
+#define SFM_ERR_NULL        -1   /* a required pointer is NULL */
+#define SFM_ERR_DTYPE       -2   /* dtype not one of SFM_BF16 / SFM_F16 / SFM_F32 (or not allowed for the op) */
+#define SFM_ERR_SHAPE       -3   /* sizes inconsistent with the tiling (e.g. tokens not a multiple of b1*b2) */
+#define SFM_ERR_RANGE       -4   /* start/end index out of range or not aligned to a block-frame */
+#define SFM_ERR_STRIDE      -5   /* stride too small / K and V strides differ where they must agree */
+#define SFM_ERR_WORKSPACE   -6   /* workspace NULL, misaligned or too small */
+#define SFM_ERR_ALIGN       -7   /* a tensor pointer is not 16-byte aligned */
+#define SFM_ERR_HIP         -8   /* the HIP runtime refused a launch (see sfm_last_error) */
+#define SFM_ERR_UNSUPPORTED -9   /* combination not implemented */
+
+#define SFM_BF16 0
+#define SFM_F16  1
+#define SFM_F32  2
+
+/* Token tiling of the Monarch op: wan/modules/monarch_attn.py:1696-1703 (_get_rearrange_fns).
+ * Tokens are (frame,row,col) ordered with h rows x w cols per frame.
+ *   b1 = f_tied*h/h_reduce rows per block, b2 = w/w_reduce cols per block,
+ *   block-frames = tokens/(f_tied*h*w) * h_reduce*w_reduce. */
+typedef struct sfm_tiling {
+    int32_t f_tied, h_reduce, w_reduce, h, w;
+} sfm_tiling;
+
+typedef struct sfm_monarch_desc {
+    int32_t dtype;            /* SFM_BF16 | SFM_F16 | SFM_F32 : type of q, k, v, out */
+    int32_t B, H, D;          /* batch, heads, head_dim */
+    int32_t q_tokens;         /* Sq  (multiple of f_tied*h*w) */
+    int32_t kv_tokens;        /* Skv (multiple of f_tied*h*w): the whole cache view / key sequence */
+    sfm_tiling tiling;
+    int32_t kv_block_order;   /* 1: k/v rows are stored in Monarch block order (KV-cache layout,
+                                 monarch_attn.py:1784-1785, 1233-1234); 0: token order like q */
+    int32_t causal_block_frames; /* 0 = every query sees every key; else block-causal in units of
+                                 block-frames (monarch_attn.py:139-141, 804-807), requires Sq == Skv */
+    float   sm_scale;         /* logit scale; the reference default is D^-0.5 (monarch_attn.py:1780-1781) */
+    int64_t q_stride[3];      /* batch, token, head */
+    int64_t k_stride[3];
+    int64_t v_stride[3];      /* must equal k_stride (monarch_attn.py:1261) */
+    int64_t o_stride[3];
+} sfm_monarch_desc;
+
+/* Bytes of device scratch sfm_monarch_fwd needs when it processes `heads_per_pass`
+ * (batch x head) units at a time (0 = library default).  Replaces the per-call torch.empty
+ * scratch of monarch_attn.py:1246-1259. */
+int sfm_monarch_workspace_bytes(const sfm_monarch_desc* desc, int32_t heads_per_pass, size_t* bytes);
+
+/* One-iteration Monarch attention forward.  Replaces _attention_with_cache.forward /
+ * _attention_no_cache.forward and their two Triton kernels: monarch_attn.py:1225-1323,
+ * 1472-1563, 109-253 (_al_cl_y_fwd), 698-842 (_z_fwd).  q and out are in token order.
+ * The number of (batch x head) units per pass is derived from workspace_bytes. */
+int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* Writes new_k/new_v [B, n_new, H, D] (token order) into k_cache/v_cache[:, start_idx:end_idx]
+ * in Monarch block order.  Replaces monarch_attn.py:1784-1785 + 1230-1231.
+ * strides: new_stride for new_k and new_v, cache_stride for both caches. */
+int sfm_kv_cache_write(int32_t dtype, int32_t B, int32_t H, int32_t D, const sfm_tiling* tiling,
+                       const void* new_k, const void* new_v, const int64_t new_stride[3],
+                       void* k_cache, void* v_cache, const int64_t cache_stride[3],
+                       int64_t cache_tokens, int64_t start_idx, int64_t end_idx, void* stream);
+
+/* monarch_attn_with_kv_cache (monarch_attn.py:1778-1796): cache write at [start_idx,end_idx)
+ * followed by sfm_monarch_fwd over the whole cache view (desc->kv_tokens tokens,
+ * desc->kv_block_order must be 1). */
+int sfm_monarch_attn_with_kv_cache(const sfm_monarch_desc* desc, const void* q, void* k_cache, void* v_cache,
+                                   const void* new_k, const void* new_v, const int64_t new_stride[3],
+                                   int64_t start_idx, int64_t end_idx, void* out,
+                                   void* workspace, size_t workspace_bytes, void* stream);
+
+typedef struct sfm_dense_desc {
+    int32_t dtype;            /* SFM_BF16 | SFM_F16 (attn_patch.py:317) | SFM_F32 */
+    int32_t B, H, D;
+    int32_t q_tokens, kv_tokens;
+    float   sm_scale;         /* reference default D^-0.5 (attention.py:179-186, attn_patch.py:417-418) */
+    int64_t q_stride[3];
+    int64_t k_stride[3];
+    int64_t v_stride[3];
+    int64_t o_stride[3];
+} sfm_dense_desc;
+
+/* Dense non-causal softmax attention of q against the first kv_tokens of k/v.  Replaces
+ * attention() (attention.py:141-187) and _attn_fwd (attn_patch.py:20-110).  lse (float32,
+ * [B,H,q_tokens], natural log) may be NULL. */
+int sfm_dense_fwd(const sfm_dense_desc* desc, const void* q, const void* k, const void* v, void* out,
+                  float* lse, void* stream);
+
+/* full_attention_with_kv_cache (attn_patch.py:416-419, 305-351): slice-assign new_k/new_v into
+ * the cache at [start_idx,end_idx) (token order, no permutation), then sfm_dense_fwd. */
+int sfm_full_attention_with_kv_cache(const sfm_dense_desc* desc, const void* q, void* k_cache, void* v_cache,
+                                     const void* new_k, const void* new_v, const int64_t new_stride[3],
+                                     int64_t start_idx, int64_t end_idx, void* out, float* lse, void* stream);
+
+typedef struct sfm_prologue_desc {
+    int32_t dtype;            /* SFM_BF16 | SFM_F16 | SFM_F32 */
+    int32_t B, S, H, D;       /* S new tokens (= F*h*w), model dim C = H*D */
+    int32_t F, h, w;          /* grid of the new tokens */
+    int32_t start_frame;      /* RoPE frame offset (causal_model.py:900-905) */
+    float   eps;              /* RMSNorm epsilon (causal_model.py:773-774) */
+    sfm_tiling tiling;        /* order in which K/V rows are laid into the cache */
+    int64_t x_stride[2];      /* batch, token strides of xq, xk, xv ([B,S,C], C contiguous) */
+    int64_t q_stride[3];      /* q_out [B,S,H,D] */
+    int64_t cache_stride[3];  /* k_cache, v_cache [B,cache_tokens,H,D] */
+    int64_t cache_tokens;
+    int64_t start_idx;        /* K/V rows are written to cache[:, start_idx : start_idx+S] */
+} sfm_prologue_desc;
+
+/* Fused q/k prologue: RMSNorm over the full model dim (model.py:462-478) with weights wq/wk [C],
+ * 3-D RoPE on interleaved pairs (causal_model.py:687-715; angles from the float64 table
+ * `rope_cos_sin` [max_pos, D/2, 2] built as model.py:421-428 + causal_model.py:1350-1357),
+ * q -> q_out (token order), roped k and v -> cache rows in Monarch block order
+ * (monarch_attn.py:1784-1785, 1230-1231; causal_model.py:961-962 when the tiling is the identity). */
+int sfm_qk_prologue(const sfm_prologue_desc* desc, const void* xq, const void* xk, const void* xv,
+                    const void* wq, const void* wk, const double* rope_cos_sin, int32_t rope_max_pos,
+                    void* q_out, void* k_cache, void* v_cache, void* stream);
+
+/* Thread-local description of the last error returned on this thread ("" if none). */
+const char* sfm_last_error(void);
+
+/* ABI version (bumped on any signature change). */
+int sfm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SFM_ATTN_H */

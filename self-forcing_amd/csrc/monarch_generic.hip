@@ -1,0 +1,195 @@
+// Monarch attention forward, shape-generic fp32 path (any dtype in {bf16, fp16, fp32}, any head_dim
+// and block shape that fits LDS).  Same two steps and the same workspace layout as the MFMA path,
+// with Kbar / Y kept in float.  This is the path fp32 tensors take, and the one block shapes
+// outside the MFMA kernels' limits fall back to; it computes exactly
+//   wan/modules/monarch_attn.py:1801-1830 (monarch_attn_ref_op)
+// with all arithmetic in fp32.
+
+#include "sfm_common.hpp"
+
+namespace sfm {
+
+template <typename T> struct Ld;
+template <> struct Ld<float> {
+    static __device__ __forceinline__ float get(const void* p, int64_t i) { return ((const float*)p)[i]; }
+    static __device__ __forceinline__ void put(void* p, int64_t i, float x) { ((float*)p)[i] = x; }
+};
+template <> struct Ld<BF16> {
+    static __device__ __forceinline__ float get(const void* p, int64_t i) { return BF16::to_float(((const uint16_t*)p)[i]); }
+    static __device__ __forceinline__ void put(void* p, int64_t i, float x) { ((uint16_t*)p)[i] = BF16::from_float(x); }
+};
+template <> struct Ld<F16> {
+    static __device__ __forceinline__ float get(const void* p, int64_t i) { return F16::to_float(((const uint16_t*)p)[i]); }
+    static __device__ __forceinline__ void put(void* p, int64_t i, float x) { ((uint16_t*)p)[i] = F16::from_float(x); }
+};
+
+// workgroup = (block row k, kv block-frame f, unit x query block-frame a); 256 threads
+template <typename T>
+__global__ __launch_bounds__(256) void monarch_generic_step1(MonarchArgs p) {
+    extern __shared__ float sm[];
+    const int D = p.D, b2 = p.b2, DP = D + 1;
+    float* Ks = sm;                    // [b2][D+1]
+    float* Vs = Ks + b2 * DP;          // [b2][D+1]
+    float* qs = Vs + b2 * DP;          // [D]
+    float* zs = qs + D;                // [b2]
+
+    const int k = blockIdx.x, f = blockIdx.y;
+    const int ul = blockIdx.z / p.na, a = blockIdx.z % p.na;
+    if (p.causal && (a / p.causal) < (f / p.causal)) return;
+    const int unit = p.unit0 + ul;
+    const int b = unit / p.H, h = unit % p.H;
+    const int tid = threadIdx.x, nt = blockDim.x;
+
+    const int64_t krow0 = p.kmap.row(f, k);
+    for (int e = tid; e < b2 * D; e += nt) {
+        int l = e / D, d = e % D;
+        Ks[l * DP + d] = Ld<T>::get(p.k, (int64_t)b * p.ks[0] + (krow0 + l) * p.ks[1] + (int64_t)h * p.ks[2] + d);
+        Vs[l * DP + d] = Ld<T>::get(p.v, (int64_t)b * p.vs[0] + (krow0 + l) * p.vs[1] + (int64_t)h * p.vs[2] + d);
+    }
+    const int64_t qrow0 = p.qmap.row(a, k);
+    const float sc2 = p.scale * kLog2e;
+    float* kbar = (float*)p.kbar;
+    float* yw = (float*)p.y;
+
+    for (int j = 0; j < b2; ++j) {
+        __syncthreads();
+        for (int d = tid; d < D; d += nt)
+            qs[d] = Ld<T>::get(p.q, (int64_t)b * p.qs[0] + (qrow0 + j) * p.qs[1] + (int64_t)h * p.qs[2] + d);
+        __syncthreads();
+        for (int l = tid; l < b2; l += nt) {
+            float acc = 0.f;
+            for (int d = 0; d < D; ++d) acc += qs[d] * Ks[l * DP + d];
+            zs[l] = acc * sc2;
+        }
+        __syncthreads();
+        float mx = -INFINITY;
+        for (int l = 0; l < b2; ++l) mx = fmaxf(mx, zs[l]);
+        float sum = 0.f, ent = 0.f;
+        for (int l = 0; l < b2; ++l) {
+            float e = exp2f(zs[l] - mx);
+            sum += e;
+            ent += e * zs[l];
+        }
+        const float inv = 1.f / sum;
+        const int64_t blk = (((int64_t)ul * p.na + a) * b2 + j) * p.r_pad + (int64_t)f * p.b1 + k;
+        if (tid == 0) p.cl[blk] = ent * inv - (mx + log2f(sum));
+        for (int d = tid; d < D; d += nt) {
+            float ak = 0.f, av = 0.f;
+            for (int l = 0; l < b2; ++l) {
+                float r = exp2f(zs[l] - mx) * inv;
+                ak += r * Ks[l * DP + d];
+                av += r * Vs[l * DP + d];
+            }
+            kbar[blk * D + d] = ak;
+            yw[blk * D + d] = av;
+        }
+    }
+}
+
+// workgroup = (unit, a, j); loops over the block rows i; 256 threads
+template <typename T>
+__global__ __launch_bounds__(256) void monarch_generic_step2(MonarchArgs p) {
+    extern __shared__ float sm[];
+    const int D = p.D, b2 = p.b2;
+    const int a = blockIdx.x / b2, j = blockIdx.x % b2;
+    const int ul = blockIdx.y;
+    const int unit = p.unit0 + ul;
+    const int b = unit / p.H, h = unit % p.H;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const int f_lim = p.causal ? min(p.nf, (a / p.causal + 1) * p.causal) : p.nf;
+    const int R = f_lim * p.b1;
+
+    float* qs = sm;            // [D]
+    float* zs = qs + D;        // [R]
+    float* red = zs + R;       // [nt]
+
+    const int64_t blk = (((int64_t)ul * p.na + a) * b2 + j) * p.r_pad;
+    const float* kbar = (const float*)p.kbar + blk * D;
+    const float* yw = (const float*)p.y + blk * D;
+    const float* cl = p.cl + blk;
+    const float sc2 = p.scale * kLog2e;
+
+    for (int i = 0; i < p.b1; ++i) {
+        const int64_t tok = p.qmap.row(a, i) + j;
+        __syncthreads();
+        for (int d = tid; d < D; d += nt)
+            qs[d] = Ld<T>::get(p.q, (int64_t)b * p.qs[0] + tok * p.qs[1] + (int64_t)h * p.qs[2] + d);
+        __syncthreads();
+        float mx = -INFINITY;
+        for (int r = tid; r < R; r += nt) {
+            float acc = 0.f;
+            const float* row = kbar + (int64_t)r * D;
+            for (int d = 0; d < D; ++d) acc += qs[d] * row[d];
+            float z = acc * sc2 - cl[r];
+            zs[r] = z;
+            mx = fmaxf(mx, z);
+        }
+        red[tid] = mx;
+        __syncthreads();
+        for (int s = nt / 2; s > 0; s >>= 1) {
+            if (tid < s) red[tid] = fmaxf(red[tid], red[tid + s]);
+            __syncthreads();
+        }
+        mx = red[0];
+        __syncthreads();
+        float sum = 0.f;
+        for (int r = tid; r < R; r += nt) {
+            float e = exp2f(zs[r] - mx);
+            zs[r] = e;
+            sum += e;
+        }
+        red[tid] = sum;
+        __syncthreads();
+        for (int s = nt / 2; s > 0; s >>= 1) {
+            if (tid < s) red[tid] += red[tid + s];
+            __syncthreads();
+        }
+        const float inv = 1.f / red[0];
+        for (int d = tid; d < D; d += nt) {
+            float acc = 0.f;
+            for (int r = 0; r < R; ++r) acc += zs[r] * yw[(int64_t)r * D + d];
+            Ld<T>::put(p.out, (int64_t)b * p.os[0] + tok * p.os[1] + (int64_t)h * p.os[2] + d, acc * inv);
+        }
+    }
+}
+
+static size_t generic_lds1(const MonarchArgs& a) { return sizeof(float) * ((size_t)2 * a.b2 * (a.D + 1) + a.D + a.b2); }
+static size_t generic_lds2(const MonarchArgs& a) { return sizeof(float) * ((size_t)a.D + (size_t)a.nf * a.b1 + 256); }
+
+bool monarch_generic_supported(const MonarchArgs& a) {
+    return generic_lds1(a) <= 160 * 1024 && generic_lds2(a) <= 160 * 1024;
+}
+
+template <typename T>
+static int launch_generic_t(const MonarchArgs& a, int nunits, hipStream_t stream) {
+    const size_t l1 = generic_lds1(a), l2 = generic_lds2(a);
+    hipError_t err = hipSuccess;
+    if (l1 > 64 * 1024)
+        err = hipFuncSetAttribute((const void*)monarch_generic_step1<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)l1);
+    if (err == hipSuccess && l2 > 64 * 1024)
+        err = hipFuncSetAttribute((const void*)monarch_generic_step2<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)l2);
+    if (err != hipSuccess) {
+        set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(err));
+        return SFM_ERR_HIP;
+    }
+    hipLaunchKernelGGL((monarch_generic_step1<T>), dim3(a.b1, a.nf, nunits * a.na), dim3(256), l1, stream, a);
+    hipLaunchKernelGGL((monarch_generic_step2<T>), dim3(a.na * a.b2, nunits), dim3(256), l2, stream, a);
+    err = hipGetLastError();
+    if (err != hipSuccess) {
+        set_error("hip launch failed: %s", hipGetErrorString(err));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream) {
+    if (!monarch_generic_supported(a)) {
+        set_error("block shape b2=%d, rows=%d, D=%d exceeds the LDS budget of the generic path", a.b2, a.nf * a.b1, a.D);
+        return SFM_ERR_UNSUPPORTED;
+    }
+    if (dtype == SFM_F32) return launch_generic_t<float>(a, nunits, stream);
+    if (dtype == SFM_BF16) return launch_generic_t<BF16>(a, nunits, stream);
+    return launch_generic_t<F16>(a, nunits, stream);
+}
+
+}  // namespace sfm

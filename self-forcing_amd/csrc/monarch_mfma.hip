@@ -1,0 +1,522 @@
+// Monarch attention forward on gfx950 MFMA (bf16 / fp16, head_dim 64 or 128, block cols b2 <= 64).
+//
+// Two kernels per pass over a group of (batch x head) units:
+//
+//  step 1 (right factor; replaces _al_cl_y_fwd, wan/modules/monarch_attn.py:109-253)
+//      workgroup = (unit, a-chunk, kv block-frame f, a range of block rows k)
+//      for each k: stage K[f,k,:,:], V[f,k,:,:] in LDS once (row-major K for the logits,
+//      transposed K^T / V^T for the contractions), and for ALL query block-frames of the chunk
+//          S^T[l,(a,j)] = K[f,k,l,:] . Q[a,k,j,:]           (MFMA, wave = 32 (a,j) columns)
+//          R = softmax_l(s S)       cl = sum_l R log2 R      (registers + one cross-half shuffle)
+//          Kbar^T = K^T R^T,  Y^T = V^T R^T                  (MFMA; R^T is fed straight from the
+//                                                             accumulator layout, see perm_row)
+//      rows Kbar[a,j,(f,k),:], Y[a,j,(f,k),:] go to the workspace through an LDS transpose so
+//      that every global store is a full 128-byte line.
+//
+//  step 2 (left factor; replaces _z_fwd, monarch_attn.py:698-842)
+//      wave = (unit, a, j): streams its contiguous Kbar / Y rows once,
+//          S2^T[(f,k), i] = Kbar[(f,k),:] . Q[a,i,j,:]  - cl       online softmax over (f,k)
+//          O^T[d, i]     += Y^T[d,(f,k)] P^T[(f,k), i]
+//      Y^T operands are built in registers from dword loads of 8 rows (no LDS, no transpose pass).
+//
+// The running output stays in fp32 for the whole KV range (the reference rounds it to 16 bit
+// between KV chunks, monarch_attn.py:795,838).
+
+#include "sfm_common.hpp"
+
+namespace sfm {
+
+// ------------------------------------------------------------------------------------------------
+// step 1
+// ------------------------------------------------------------------------------------------------
+template <int D>
+struct S1Lds {
+    static constexpr int kRowPitch = D + 8;    // u16 per row of row-major K   [64][D+8]
+    static constexpr int kTPitch = 72;         // u16 per row of K^T / V^T     [D][64+8]
+    static constexpr int kStagePitch = 72;     // u16 per row of a wave's output stage [32][64+8]
+    static constexpr int kKrow = 0;
+    static constexpr int kKT = kKrow + 64 * kRowPitch;
+    static constexpr int kVT = kKT + D * kTPitch;
+    static constexpr int kStage = kVT + D * kTPitch;
+    static constexpr int kStagePerWave = 32 * kStagePitch;
+    static __host__ __device__ constexpr size_t bytes(int nwaves) { return 2 * (size_t)(kStage + nwaves * kStagePerWave); }
+};
+
+template <class E, int D>
+__global__ __launch_bounds__(512) void monarch_step1_kernel(MonarchArgs p) {
+    using L = S1Lds<D>;
+    constexpr int DS = D / 16;   // contraction steps of the logits
+    constexpr int DT = D / 32;   // 32-row tiles of the transposed outputs
+    constexpr int DP = D / 2;    // dword columns of a K/V row
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+
+    const int tid = threadIdx.x;
+    const int nthreads = blockDim.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int m = lane & 31;
+    const int hf = lane >> 5;
+
+    const int f = blockIdx.y;
+    const int ul = blockIdx.z / p.n_achunks;              // unit within this pass
+    const int a0 = (blockIdx.z % p.n_achunks) * p.a_chunk;
+    const int a_cnt = min(p.a_chunk, p.na - a0);
+    const int unit = p.unit0 + ul;
+    const int b = unit / p.H, h = unit % p.H;
+    const int k0 = blockIdx.x * p.k_per_wg;
+    const int k1 = min(k0 + p.k_per_wg, p.b1);
+    if (p.causal && ((a0 + a_cnt - 1) / p.causal) < (f / p.causal)) return;   // every a of the chunk is masked
+
+    const int b2 = p.b2;
+    const int ncols = a_cnt * b2;
+    const int NT = b2 > 32 ? 2 : 1;                       // 32-row tiles of the key axis l
+    const bool tile_active = wave * 32 < ncols;
+
+    const uint16_t* qg = (const uint16_t*)p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[2];
+    const uint16_t* kg = (const uint16_t*)p.k + (int64_t)b * p.ks[0] + (int64_t)h * p.ks[2];
+    const uint16_t* vg = (const uint16_t*)p.v + (int64_t)b * p.vs[0] + (int64_t)h * p.vs[2];
+
+    // column owned by this lane in the logits/contraction phase
+    const int cg = wave * 32 + m;
+    const bool col_ok = cg < ncols;
+    const int ca = a0 + (col_ok ? cg / b2 : 0);
+    const int cj = col_ok ? cg % b2 : 0;
+
+    // rows this lane stores in the epilogue: 4 rows, r = 8*it + lane/8 of the wave's 32 columns
+    const int R = p.nf * p.b1;
+    int64_t orow[4];
+    bool orow_ok[4];
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        int c = wave * 32 + it * 8 + (lane >> 3);
+        orow_ok[it] = c < ncols;
+        int aa = a0 + (orow_ok[it] ? c / b2 : 0);
+        int jj = orow_ok[it] ? c % b2 : 0;
+        orow[it] = ((((int64_t)ul * p.na + aa) * b2 + jj) * p.r_pad + (int64_t)f * p.b1) * D + (lane & 7) * 8;
+    }
+    const int64_t clbase = (((int64_t)ul * p.na + ca) * b2 + cj) * p.r_pad + (int64_t)f * p.b1;
+
+    // staging tasks: (sh = 2*s + hf', dword column pc); 8 rows perm_row(s, hf', 0..7) each
+    constexpr int kTasks = 8 * DP;
+    constexpr int kMaxTask = 2;                             // host launches >= kTasks/2 threads
+    const int ntask = (kTasks + nthreads - 1) / nthreads;
+    uint32_t pk[kMaxTask][8], pv[kMaxTask][8];
+
+    auto prefetch = [&](int k) {
+        const int64_t krow0 = p.kmap.row(f, k);
+#pragma unroll
+        for (int t = 0; t < kMaxTask; ++t) {
+            int task = tid + t * nthreads;
+            if (t < ntask && task < kTasks) {
+                int pc = task % DP, sh = task / DP;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    int l = perm_row(sh >> 1, sh & 1, e);
+                    uint32_t kk = 0, vv = 0;
+                    if (l < b2) {
+                        kk = *(const uint32_t*)(kg + (krow0 + l) * p.ks[1] + 2 * pc);
+                        vv = *(const uint32_t*)(vg + (krow0 + l) * p.vs[1] + 2 * pc);
+                    }
+                    pk[t][e] = kk;
+                    pv[t][e] = vv;
+                }
+            }
+        }
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int t = 0; t < kMaxTask; ++t) {
+            int task = tid + t * nthreads;
+            if (t < ntask && task < kTasks) {
+                int pc = task % DP, sh = task / DP;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    int l = perm_row(sh >> 1, sh & 1, e);
+                    *(uint32_t*)(lds + L::kKrow + l * L::kRowPitch + 2 * pc) = pk[t][e];
+                }
+                u32x4 lo, hi;
+                lo.x = lo16x2(pk[t][0], pk[t][1]); lo.y = lo16x2(pk[t][2], pk[t][3]);
+                lo.z = lo16x2(pk[t][4], pk[t][5]); lo.w = lo16x2(pk[t][6], pk[t][7]);
+                hi.x = hi16x2(pk[t][0], pk[t][1]); hi.y = hi16x2(pk[t][2], pk[t][3]);
+                hi.z = hi16x2(pk[t][4], pk[t][5]); hi.w = hi16x2(pk[t][6], pk[t][7]);
+                *(u32x4*)(lds + L::kKT + (2 * pc) * L::kTPitch + sh * 8) = lo;
+                *(u32x4*)(lds + L::kKT + (2 * pc + 1) * L::kTPitch + sh * 8) = hi;
+                lo.x = lo16x2(pv[t][0], pv[t][1]); lo.y = lo16x2(pv[t][2], pv[t][3]);
+                lo.z = lo16x2(pv[t][4], pv[t][5]); lo.w = lo16x2(pv[t][6], pv[t][7]);
+                hi.x = hi16x2(pv[t][0], pv[t][1]); hi.y = hi16x2(pv[t][2], pv[t][3]);
+                hi.z = hi16x2(pv[t][4], pv[t][5]); hi.w = hi16x2(pv[t][6], pv[t][7]);
+                *(u32x4*)(lds + L::kVT + (2 * pc) * L::kTPitch + sh * 8) = lo;
+                *(u32x4*)(lds + L::kVT + (2 * pc + 1) * L::kTPitch + sh * 8) = hi;
+            }
+        }
+    };
+
+    uint16_t* stage = lds + L::kStage + wave * L::kStagePerWave;
+    const float sc2 = p.scale * kLog2e;
+
+    if (ntask > kMaxTask) return;   // host launches enough threads (checked there)
+
+    prefetch(k0);
+    for (int k = k0; k < k1; ++k) {
+        __syncthreads();                 // previous iteration finished reading K/V tiles and the stage
+        commit();
+        if (k + 1 < k1) prefetch(k + 1);
+
+        // logits operand: this lane's query row Q[ca, k, cj, :]
+        u32x4 qb[DS];
+        {
+            const uint16_t* qrow = qg + (p.qmap.row(ca, k) + cj) * p.qs[1] + 8 * hf;
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
+        }
+        __syncthreads();                 // K/V tiles visible
+
+        u32x4 pb[4];                     // R^T as B operands, 16 contraction rows per step
+        float inv_l = 0.f, cl2 = 0.f;
+        if (tile_active) {
+            f32x16 s[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[t][v] = 0.f;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (t < NT) {
+                    const uint16_t* arow = lds + L::kKrow + (32 * t + m) * L::kRowPitch + 8 * hf;
+#pragma unroll
+                    for (int ds = 0; ds < DS; ++ds) {
+                        u32x4 a = *(const u32x4*)(arow + 16 * ds);
+                        s[t] = E::mfma32(a, qb[ds], s[t]);
+                    }
+                }
+            }
+            // block softmax over l (rows of S^T): 16*NT values here, the rest in lane ^ 32
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int l = 32 * t + 8 * (v >> 2) + 4 * hf + (v & 3);
+                    float z = (t < NT && l < b2) ? s[t][v] * sc2 : -INFINITY;
+                    s[t][v] = z;
+                    mx = fmaxf(mx, z);
+                }
+            mx = xhalf_max(mx);
+            float sum = 0.f, ent = 0.f;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    float z = s[t][v];
+                    float e = exp2f(z - mx);           // exp2(-inf) = 0 for masked rows
+                    sum += e;
+                    ent += (z == -INFINITY) ? 0.f : e * z;
+                    s[t][v] = e;
+                }
+            sum = xhalf_sum(sum);
+            ent = xhalf_sum(ent);
+            inv_l = 1.f / sum;
+            cl2 = ent * inv_l - (mx + log2f(sum));      // sum_l R log2 R
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                const int t = st >> 1, v0 = 8 * (st & 1);
+                pb[st].x = pack2<E>(s[t][v0 + 0], s[t][v0 + 1]);
+                pb[st].y = pack2<E>(s[t][v0 + 2], s[t][v0 + 3]);
+                pb[st].z = pack2<E>(s[t][v0 + 4], s[t][v0 + 5]);
+                pb[st].w = pack2<E>(s[t][v0 + 6], s[t][v0 + 7]);
+            }
+            if (col_ok && hf == 0) p.cl[clbase + k] = cl2;
+        }
+
+        // contractions with K^T then V^T; each goes out through the wave's LDS stage in two
+        // halves of the head dim (64 columns at a time)
+#pragma unroll
+        for (int which = 0; which < 2; ++which) {
+            const uint16_t* tbase = lds + (which == 0 ? L::kKT : L::kVT);
+            uint16_t* og = (uint16_t*)(which == 0 ? p.kbar : p.y);
+            f32x16 acc[DT];
+            if (tile_active) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
+                    const uint16_t* arow = tbase + (32 * dt + m) * L::kTPitch + 8 * hf;
+#pragma unroll
+                    for (int st = 0; st < 4; ++st) {
+                        if (st < 2 * NT) {
+                            u32x4 a = *(const u32x4*)(arow + 16 * st);
+                            acc[dt] = E::mfma32(a, pb[st], acc[dt]);
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int hd = 0; hd < D / 64; ++hd) {
+                if (tile_active) {
+#pragma unroll
+                    for (int t2 = 0; t2 < 2; ++t2) {
+                        const int dt = 2 * hd + t2;
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            u32x2 w;
+                            w.x = pack2<E>(acc[dt][4 * g + 0] * inv_l, acc[dt][4 * g + 1] * inv_l);
+                            w.y = pack2<E>(acc[dt][4 * g + 2] * inv_l, acc[dt][4 * g + 3] * inv_l);
+                            *(u32x2*)(stage + m * L::kStagePitch + 32 * t2 + 8 * g + 4 * hf) = w;
+                        }
+                    }
+                }
+                __syncthreads();
+                if (tile_active) {
+#pragma unroll
+                    for (int it = 0; it < 4; ++it) {
+                        u32x4 w = *(const u32x4*)(stage + (it * 8 + (lane >> 3)) * L::kStagePitch + (lane & 7) * 8);
+                        if (orow_ok[it]) *(u32x4*)(og + orow[it] + (int64_t)k * D + 64 * hd) = w;
+                    }
+                }
+                __syncthreads();
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// step 2
+// ------------------------------------------------------------------------------------------------
+template <int D>
+struct S2Lds {
+    static constexpr int kPitch = D + 8;             // u16 per row of a wave's [32][D+8] region
+    static constexpr int kPerWave = 32 * kPitch;
+    static __host__ __device__ constexpr size_t bytes() { return 2 * (size_t)(4 * kPerWave); }
+};
+
+template <class E, int D>
+__global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
+    using L = S2Lds<D>;
+    constexpr int DS = D / 16;
+    constexpr int DPn = D / 64;          // 64-wide head-dim spans, each giving an even and an odd 32-row tile
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int m = lane & 31;
+    const int hf = lane >> 5;
+
+    const int b2 = p.b2;
+    const int njg = (b2 + 3) / 4;
+    const int a = blockIdx.x / njg;
+    const int jraw = (blockIdx.x % njg) * 4 + wave;
+    const bool j_ok = jraw < b2;
+    const int j = j_ok ? jraw : b2 - 1;
+    const int ul = blockIdx.y;
+    const int unit = p.unit0 + ul;
+    const int b = unit / p.H, h = unit % p.H;
+    const int i0 = blockIdx.z * 32;
+
+    const int f_lim = p.causal ? min(p.nf, (a / p.causal + 1) * p.causal) : p.nf;
+    const int r_lim = f_lim * p.b1;
+    const int nch = (r_lim + 31) / 32;
+
+    const int64_t blk = (((int64_t)ul * p.na + a) * b2 + j) * p.r_pad;
+    const uint16_t* kb = (const uint16_t*)p.kbar + blk * D;
+    const uint16_t* yb = (const uint16_t*)p.y + blk * D;
+    const float* clp = p.cl + blk;
+
+    uint16_t* wl = lds + wave * L::kPerWave;
+
+    // stage the wave's query rows Q[a, i0 + 0..31, j, :] (zero rows past b1)
+    {
+        const uint16_t* qg = (const uint16_t*)p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[2];
+        constexpr int CH = D / 8;                      // 16-byte chunks per row
+        for (int c = lane; c < 32 * CH; c += 64) {
+            int r = c / CH, ch = c % CH;
+            int i = i0 + r;
+            u32x4 w = {0u, 0u, 0u, 0u};
+            if (i < p.b1) w = *(const u32x4*)(qg + (p.qmap.row(a, i) + j) * p.qs[1] + ch * 8);
+            *(u32x4*)(wl + r * L::kPitch + ch * 8) = w;
+        }
+    }
+    __syncthreads();
+
+    const float sc2 = p.scale * kLog2e;
+    f32x16 oacc[DPn][2];
+#pragma unroll
+    for (int dp = 0; dp < DPn; ++dp)
+#pragma unroll
+        for (int par = 0; par < 2; ++par)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) oacc[dp][par][v] = 0.f;
+    float mrun = -INFINITY, lrun = 0.f;
+
+    u32x4 kcur[DS];
+    f32x4 ccur[4];
+    uint32_t ycur[2][DPn][8];
+
+    auto load_k = [&](int n) {
+        const uint16_t* row = kb + (int64_t)(32 * n + m) * D + 8 * hf;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) kcur[ds] = *(const u32x4*)(row + 16 * ds);
+    };
+    auto load_c = [&](int n) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) ccur[g] = *(const f32x4*)(clp + 32 * n + 8 * g + 4 * hf);
+    };
+    auto load_y = [&](int n) {
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                int r = 32 * n + perm_row(st, hf, e);
+                const uint16_t* row = yb + (int64_t)r * D + 2 * m;
+#pragma unroll
+                for (int dp = 0; dp < DPn; ++dp) {
+                    uint32_t w = *(const uint32_t*)(row + 64 * dp);
+                    ycur[st][dp][e] = r < r_lim ? w : 0u;     // rows past the valid range may hold anything
+                }
+            }
+    };
+
+    // Single-buffered software pipeline: each operand set is re-loaded for chunk n+1 as soon as
+    // chunk n has consumed it, so that about one chunk of Kbar and Y rows is in flight per wave.
+    load_k(0);
+    load_c(0);
+    load_y(0);
+    for (int n = 0; n < nch; ++n) {
+        const int nn = min(n + 1, nch - 1);
+
+        f32x16 s;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            u32x4 qb = *(const u32x4*)(wl + m * L::kPitch + 16 * ds + 8 * hf);
+            s = E::mfma32(kcur[ds], qb, s);
+        }
+        load_k(nn);
+
+        float mx = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            int r = 32 * n + 8 * (v >> 2) + 4 * hf + (v & 3);
+            float z = r < r_lim ? s[v] * sc2 - ccur[v >> 2][v & 3] : -INFINITY;
+            s[v] = z;
+            mx = fmaxf(mx, z);
+        }
+        load_c(nn);
+        mx = xhalf_max(mx);
+        const float mnew = fmaxf(mrun, mx);        // finite: chunk n has at least one valid row
+        const float alpha = exp2f(mrun - mnew);
+        float psum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            float e = exp2f(s[v] - mnew);
+            psum += e;
+            s[v] = e;
+        }
+        lrun = lrun * alpha + psum;
+        mrun = mnew;
+        u32x4 pb[2];
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+            pb[st].x = pack2<E>(s[8 * st + 0], s[8 * st + 1]);
+            pb[st].y = pack2<E>(s[8 * st + 2], s[8 * st + 3]);
+            pb[st].z = pack2<E>(s[8 * st + 4], s[8 * st + 5]);
+            pb[st].w = pack2<E>(s[8 * st + 6], s[8 * st + 7]);
+        }
+
+#pragma unroll
+        for (int dp = 0; dp < DPn; ++dp) {
+#pragma unroll
+            for (int par = 0; par < 2; ++par)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) oacc[dp][par][v] *= alpha;
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                const uint32_t* yy = ycur[st][dp];
+                u32x4 ae, ao;
+                ae.x = lo16x2(yy[0], yy[1]); ae.y = lo16x2(yy[2], yy[3]);
+                ae.z = lo16x2(yy[4], yy[5]); ae.w = lo16x2(yy[6], yy[7]);
+                ao.x = hi16x2(yy[0], yy[1]); ao.y = hi16x2(yy[2], yy[3]);
+                ao.z = hi16x2(yy[4], yy[5]); ao.w = hi16x2(yy[6], yy[7]);
+                oacc[dp][0] = E::mfma32(ae, pb[st], oacc[dp][0]);
+                oacc[dp][1] = E::mfma32(ao, pb[st], oacc[dp][1]);
+            }
+        }
+        load_y(nn);
+    }
+
+    // epilogue: O[i, d] = O^T / l, through the wave's LDS region (the query rows are dead now)
+    const float inv = 1.f / xhalf_sum(lrun);
+    __syncthreads();
+#pragma unroll
+    for (int dp = 0; dp < DPn; ++dp)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            // accumulator row mr = 8g + 4hf + v%4 of tile (dp, par) is head-dim 64dp + 2mr + par
+            u32x4 w;
+            w.x = pack2<E>(oacc[dp][0][4 * g + 0] * inv, oacc[dp][1][4 * g + 0] * inv);
+            w.y = pack2<E>(oacc[dp][0][4 * g + 1] * inv, oacc[dp][1][4 * g + 1] * inv);
+            w.z = pack2<E>(oacc[dp][0][4 * g + 2] * inv, oacc[dp][1][4 * g + 2] * inv);
+            w.w = pack2<E>(oacc[dp][0][4 * g + 3] * inv, oacc[dp][1][4 * g + 3] * inv);
+            *(u32x4*)(wl + m * L::kPitch + 64 * dp + 2 * (8 * g + 4 * hf)) = w;
+        }
+    __syncthreads();
+    {
+        uint16_t* og = (uint16_t*)p.out + (int64_t)b * p.os[0] + (int64_t)h * p.os[2];
+        constexpr int CH = D / 8;
+        for (int c = lane; c < 32 * CH; c += 64) {
+            int r = c / CH, ch = c % CH;
+            int i = i0 + r;
+            if (i < p.b1 && j_ok) {
+                u32x4 w = *(const u32x4*)(wl + r * L::kPitch + ch * 8);
+                *(u32x4*)(og + (p.qmap.row(a, i) + j) * p.os[1] + ch * 8) = w;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host launch
+// ------------------------------------------------------------------------------------------------
+bool monarch_mfma_supported(int dtype, int D, int b2) {
+    return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 >= 1 && b2 <= 64;
+}
+
+template <class E, int D>
+static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream) {
+    const int ncols = a.a_chunk * a.b2;
+    const int ntiles = (ncols + 31) / 32;
+    const int nwaves = ntiles < 4 ? 4 : ntiles;   // at least 4 waves so that K/V staging is <= 2 tasks per thread
+    const int kgroups = (a.b1 + a.k_per_wg - 1) / a.k_per_wg;
+    if (ntiles < 1 || nwaves > 8 || (8 * (D / 2) + nwaves * 64 - 1) / (nwaves * 64) > 2) {
+        set_error("internal: step-1 launch shape (a_chunk=%d, b2=%d)", a.a_chunk, a.b2);
+        return SFM_ERR_UNSUPPORTED;
+    }
+    const size_t lds1 = S1Lds<D>::bytes(nwaves);
+    if (lds1 > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)monarch_step1_kernel<E, D>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1);
+        if (e != hipSuccess) {
+            set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+            return SFM_ERR_HIP;
+        }
+    }
+    dim3 g1(kgroups, a.nf, nunits * a.n_achunks);
+    hipLaunchKernelGGL((monarch_step1_kernel<E, D>), g1, dim3(nwaves * 64), lds1, stream, a);
+    const int njg = (a.b2 + 3) / 4;
+    dim3 g2(a.na * njg, nunits, (a.b1 + 31) / 32);
+    hipLaunchKernelGGL((monarch_step2_kernel<E, D>), g2, dim3(256), S2Lds<D>::bytes(), stream, a);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        set_error("hip launch failed: %s", hipGetErrorString(err));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream) {
+    if (dtype == SFM_BF16) return a.D == 128 ? launch_t<BF16, 128>(a, nunits, stream) : launch_t<BF16, 64>(a, nunits, stream);
+    return a.D == 128 ? launch_t<F16, 128>(a, nunits, stream) : launch_t<F16, 64>(a, nunits, stream);
+}
+
+}  // namespace sfm

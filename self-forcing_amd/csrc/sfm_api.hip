@@ -1,0 +1,454 @@
+// extern "C" entry points: argument validation, workspace accounting, pass scheduling.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "sfm_common.hpp"
+
+namespace sfm {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+int launch_kv_cache_write(int esz, int B, int H, int D, const TokMap& map, int nbf, const void* nk, const void* nv,
+                          const int64_t ns[3], void* kc, void* vc, const int64_t cs[3], int64_t start,
+                          hipStream_t stream);
+int launch_dense(const sfm_dense_desc& d, const void* q, const void* k, const void* v, void* out, float* lse,
+                 hipStream_t stream);
+int launch_prologue(const sfm_prologue_desc& d, const TokMap& map, const void* xq, const void* xk, const void* xv,
+                    const void* wq, const void* wk, const double* rope, void* q_out, void* kc, void* vc,
+                    hipStream_t stream);
+bool monarch_generic_supported(const MonarchArgs& a);
+
+static int elem_size(int dtype) { return dtype == SFM_F32 ? 4 : 2; }
+static bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
+
+static int check_tiling(const sfm_tiling& t) {
+    if (t.f_tied < 1 || t.h_reduce < 1 || t.w_reduce < 1 || t.h < 1 || t.w < 1) {
+        set_error("tiling: f_tied, h_reduce, w_reduce, h, w must be >= 1");
+        return SFM_ERR_SHAPE;
+    }
+    if (t.h % t.h_reduce || t.w % t.w_reduce) {
+        set_error("tiling: h_reduce (%d) must divide h (%d) and w_reduce (%d) must divide w (%d)", t.h_reduce, t.h,
+                  t.w_reduce, t.w);
+        return SFM_ERR_SHAPE;
+    }
+    return SFM_OK;
+}
+
+static TokMap make_map(const sfm_tiling& t, int natural) {
+    TokMap m;
+    m.hh = t.h / t.h_reduce;
+    m.ww = t.w / t.w_reduce;
+    m.b1 = t.f_tied * m.hh;
+    m.b2 = m.ww;
+    m.h = t.h;
+    m.w = t.w;
+    m.f_tied = t.f_tied;
+    m.h_reduce = t.h_reduce;
+    m.w_reduce = t.w_reduce;
+    m.natural = natural;
+    return m;
+}
+
+static int check_strides(const char* name, const int64_t s[3], int64_t tokens, int H, int D, int B, int esz) {
+    if (s[2] < D || s[1] < 1 || s[0] < 0) {
+        set_error("%s: strides (%lld, %lld, %lld) too small for H=%d, D=%d", name, (long long)s[0], (long long)s[1],
+                  (long long)s[2], H, D);
+        return SFM_ERR_STRIDE;
+    }
+    (void)tokens;
+    (void)B;
+    if ((s[0] * esz) % 16 || (s[1] * esz) % 16 || (s[2] * esz) % 16) {
+        set_error("%s: strides must be multiples of 16 bytes", name);
+        return SFM_ERR_STRIDE;
+    }
+    return SFM_OK;
+}
+
+struct MonarchPlan {
+    int na, nf, b1, b2, r_pad, units;
+    bool mfma;
+    size_t per_unit;   // workspace bytes per (batch x head) unit
+};
+
+static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
+    if (!d) {
+        set_error("desc is NULL");
+        return SFM_ERR_NULL;
+    }
+    if (d->dtype != SFM_BF16 && d->dtype != SFM_F16 && d->dtype != SFM_F32) {
+        set_error("unsupported dtype %d", d->dtype);
+        return SFM_ERR_DTYPE;
+    }
+    if (d->B < 1 || d->H < 1 || d->D < 8 || d->D % 8 || d->D > 256) {
+        set_error("B=%d, H=%d, D=%d: need B,H >= 1 and D a multiple of 8 in [8,256]", d->B, d->H, d->D);
+        return SFM_ERR_SHAPE;
+    }
+    int rc = check_tiling(d->tiling);
+    if (rc) return rc;
+    const sfm_tiling& t = d->tiling;
+    const int64_t group = (int64_t)t.f_tied * t.h * t.w;
+    if (d->q_tokens < 1 || d->kv_tokens < 1 || d->q_tokens % group || d->kv_tokens % group) {
+        set_error("q_tokens=%d / kv_tokens=%d must be positive multiples of f_tied*h*w=%lld", d->q_tokens, d->kv_tokens,
+                  (long long)group);
+        return SFM_ERR_SHAPE;
+    }
+    const int per = t.h_reduce * t.w_reduce;
+    pl->na = (int)(d->q_tokens / group) * per;
+    pl->nf = (int)(d->kv_tokens / group) * per;
+    pl->b1 = t.f_tied * (t.h / t.h_reduce);
+    pl->b2 = t.w / t.w_reduce;
+    if (d->causal_block_frames < 0) {
+        set_error("causal_block_frames must be >= 0");
+        return SFM_ERR_SHAPE;
+    }
+    if (d->causal_block_frames > 0) {
+        if (d->q_tokens != d->kv_tokens) {
+            set_error("block-causal Monarch needs kv_tokens == q_tokens");
+            return SFM_ERR_SHAPE;
+        }
+        if (pl->na % d->causal_block_frames) {
+            set_error("causal_block_frames=%d must divide the %d block-frames", d->causal_block_frames, pl->na);
+            return SFM_ERR_SHAPE;
+        }
+    }
+    if (!(d->sm_scale > 0.f) || d->sm_scale != d->sm_scale) {
+        set_error("sm_scale must be a positive number");
+        return SFM_ERR_SHAPE;
+    }
+    const int esz = elem_size(d->dtype);
+    if ((rc = check_strides("q", d->q_stride, d->q_tokens, d->H, d->D, d->B, esz))) return rc;
+    if ((rc = check_strides("k", d->k_stride, d->kv_tokens, d->H, d->D, d->B, esz))) return rc;
+    if ((rc = check_strides("v", d->v_stride, d->kv_tokens, d->H, d->D, d->B, esz))) return rc;
+    if ((rc = check_strides("out", d->o_stride, d->q_tokens, d->H, d->D, d->B, esz))) return rc;
+    if (memcmp(d->k_stride, d->v_stride, sizeof(d->k_stride)) != 0) {
+        set_error("k and v must share strides");
+        return SFM_ERR_STRIDE;
+    }
+    pl->r_pad = (pl->nf * pl->b1 + 31) / 32 * 32;
+    pl->units = d->B * d->H;
+    pl->mfma = monarch_mfma_supported(d->dtype, d->D, pl->b2);
+    const size_t rows = (size_t)pl->na * pl->b2 * pl->r_pad;
+    pl->per_unit = rows * d->D * (pl->mfma ? 2 : 4) * 2 + rows * sizeof(float);
+    pl->per_unit = (pl->per_unit + 255) / 256 * 256;
+    return SFM_OK;
+}
+
+// Default number of units per pass: keep the scratch of one pass well inside the 256 MB
+// last-level cache so that step 2 finds step 1's rows there.
+static int default_units_per_pass(const MonarchPlan& pl) {
+    const size_t budget = (size_t)112 << 20;
+    size_t n = budget / pl.per_unit;
+    if (n < 1) n = 1;
+    if (n > (size_t)pl.units) n = pl.units;
+    return (int)n;
+}
+
+}  // namespace sfm
+
+using namespace sfm;
+
+extern "C" {
+
+int sfm_version(void) { return 1; }
+
+const char* sfm_last_error(void) { return g_err; }
+
+int sfm_monarch_workspace_bytes(const sfm_monarch_desc* desc, int32_t heads_per_pass, size_t* bytes) {
+    if (!bytes) {
+        set_error("bytes is NULL");
+        return SFM_ERR_NULL;
+    }
+    MonarchPlan pl;
+    int rc = plan_monarch(desc, &pl);
+    if (rc) return rc;
+    if (heads_per_pass < 0) {
+        set_error("heads_per_pass must be >= 0");
+        return SFM_ERR_SHAPE;
+    }
+    int upp = heads_per_pass == 0 ? default_units_per_pass(pl) : (heads_per_pass > pl.units ? pl.units : heads_per_pass);
+    *bytes = pl.per_unit * (size_t)upp;
+    return SFM_OK;
+}
+
+int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+    MonarchPlan pl;
+    int rc = plan_monarch(desc, &pl);
+    if (rc) return rc;
+    if (!q || !k || !v || !out) {
+        set_error("q, k, v and out must be non-NULL");
+        return SFM_ERR_NULL;
+    }
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) {
+        set_error("q, k, v and out must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    if (!workspace || (((uintptr_t)workspace) & 255) || workspace_bytes < pl.per_unit) {
+        set_error("workspace must be non-NULL, 256-byte aligned and hold at least %zu bytes (one unit)", pl.per_unit);
+        return SFM_ERR_WORKSPACE;
+    }
+    size_t upp_sz = workspace_bytes / pl.per_unit;
+    const int upp = upp_sz > (size_t)pl.units ? pl.units : (int)upp_sz;
+
+    MonarchArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q; a.k = k; a.v = v; a.out = out;
+    a.B = desc->B; a.H = desc->H; a.D = desc->D;
+    a.na = pl.na; a.nf = pl.nf; a.b1 = pl.b1; a.b2 = pl.b2; a.r_pad = pl.r_pad;
+    a.causal = desc->causal_block_frames;
+    a.scale = desc->sm_scale;
+    a.qmap = make_map(desc->tiling, 1);
+    a.kmap = make_map(desc->tiling, desc->kv_block_order ? 0 : 1);
+    for (int i = 0; i < 3; ++i) {
+        a.qs[i] = desc->q_stride[i]; a.ks[i] = desc->k_stride[i];
+        a.vs[i] = desc->v_stride[i]; a.os[i] = desc->o_stride[i];
+    }
+    const size_t rows = (size_t)pl.na * pl.b2 * pl.r_pad;
+    const size_t mat_bytes = rows * desc->D * (pl.mfma ? 2 : 4);
+    // step 1 takes as many query block-frames per workgroup as fit 256 (a, j) columns
+    int a_max = 256 / pl.b2;
+    if (a_max < 1) a_max = 1;
+    a.n_achunks = (pl.na + a_max - 1) / a_max;
+    a.a_chunk = (pl.na + a.n_achunks - 1) / a.n_achunks;
+    a.n_achunks = (pl.na + a.a_chunk - 1) / a.a_chunk;
+    a.k_per_wg = pl.b1 < 6 ? pl.b1 : 6;
+    for (int u0 = 0; u0 < pl.units; u0 += upp) {
+        const int n = pl.units - u0 < upp ? pl.units - u0 : upp;
+        a.unit0 = u0;
+        // [kbar | y | cl] blocks, each sized for `upp` units
+        a.kbar = workspace;
+        a.y = (char*)workspace + mat_bytes * upp;
+        a.cl = (float*)((char*)workspace + 2 * mat_bytes * upp);
+        rc = pl.mfma ? launch_monarch_mfma(a, desc->dtype, n, (hipStream_t)stream)
+                     : launch_monarch_generic(a, desc->dtype, n, (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    return SFM_OK;
+}
+
+int sfm_kv_cache_write(int32_t dtype, int32_t B, int32_t H, int32_t D, const sfm_tiling* tiling, const void* new_k,
+                       const void* new_v, const int64_t new_stride[3], void* k_cache, void* v_cache,
+                       const int64_t cache_stride[3], int64_t cache_tokens, int64_t start_idx, int64_t end_idx,
+                       void* stream) {
+    if (!tiling || !new_k || !new_v || !new_stride || !k_cache || !v_cache || !cache_stride) {
+        set_error("NULL argument");
+        return SFM_ERR_NULL;
+    }
+    if (dtype != SFM_BF16 && dtype != SFM_F16 && dtype != SFM_F32) {
+        set_error("unsupported dtype %d", dtype);
+        return SFM_ERR_DTYPE;
+    }
+    if (B < 1 || H < 1 || D < 8 || D % 8) {
+        set_error("B=%d, H=%d, D=%d invalid", B, H, D);
+        return SFM_ERR_SHAPE;
+    }
+    int rc = check_tiling(*tiling);
+    if (rc) return rc;
+    const int64_t group = (int64_t)tiling->f_tied * tiling->h * tiling->w;
+    const int64_t n = end_idx - start_idx;
+    if (start_idx < 0 || end_idx > cache_tokens || n < 0) {
+        set_error("start_idx=%lld, end_idx=%lld outside the cache of %lld tokens", (long long)start_idx,
+                  (long long)end_idx, (long long)cache_tokens);
+        return SFM_ERR_RANGE;
+    }
+    if (n % group) {
+        set_error("end_idx - start_idx = %lld is not a multiple of f_tied*h*w = %lld", (long long)n, (long long)group);
+        return SFM_ERR_RANGE;
+    }
+    const int esz = elem_size(dtype);
+    if ((rc = check_strides("new_k/new_v", new_stride, n, H, D, B, esz))) return rc;
+    if ((rc = check_strides("k_cache/v_cache", cache_stride, cache_tokens, H, D, B, esz))) return rc;
+    if (!aligned16(new_k) || !aligned16(new_v) || !aligned16(k_cache) || !aligned16(v_cache)) {
+        set_error("tensors must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    if (n == 0) return SFM_OK;
+    TokMap map = make_map(*tiling, 1);
+    const int nbf = (int)(n / group) * tiling->h_reduce * tiling->w_reduce;
+    return launch_kv_cache_write(esz, B, H, D, map, nbf, new_k, new_v, new_stride, k_cache, v_cache, cache_stride,
+                                 start_idx, (hipStream_t)stream);
+}
+
+int sfm_monarch_attn_with_kv_cache(const sfm_monarch_desc* desc, const void* q, void* k_cache, void* v_cache,
+                                   const void* new_k, const void* new_v, const int64_t new_stride[3],
+                                   int64_t start_idx, int64_t end_idx, void* out, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+    MonarchPlan pl;
+    int rc = plan_monarch(desc, &pl);
+    if (rc) return rc;
+    if (!desc->kv_block_order) {
+        set_error("the KV cache holds rows in Monarch block order: kv_block_order must be 1");
+        return SFM_ERR_UNSUPPORTED;
+    }
+    if (desc->causal_block_frames) {
+        set_error("the KV-cache op takes no causal mask");
+        return SFM_ERR_UNSUPPORTED;
+    }
+    const int64_t blk = (int64_t)pl.b1 * pl.b2;
+    if (start_idx < 0 || end_idx < start_idx || end_idx > desc->kv_tokens) {
+        set_error("start_idx=%lld, end_idx=%lld outside the cache view of %d tokens", (long long)start_idx,
+                  (long long)end_idx, desc->kv_tokens);
+        return SFM_ERR_RANGE;
+    }
+    if (start_idx % blk || end_idx % blk) {
+        set_error("start_idx=%lld / end_idx=%lld must be multiples of b1*b2=%lld", (long long)start_idx,
+                  (long long)end_idx, (long long)blk);
+        return SFM_ERR_RANGE;
+    }
+    // validate everything the forward will check BEFORE the cache is touched
+    if (!q || !k_cache || !v_cache || !out || !new_k || !new_v || !new_stride) {
+        set_error("NULL argument");
+        return SFM_ERR_NULL;
+    }
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out)) {
+        set_error("q, caches and out must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    if (!workspace || (((uintptr_t)workspace) & 255) || workspace_bytes < pl.per_unit) {
+        set_error("workspace must be non-NULL, 256-byte aligned and hold at least %zu bytes (one unit)", pl.per_unit);
+        return SFM_ERR_WORKSPACE;
+    }
+    rc = sfm_kv_cache_write(desc->dtype, desc->B, desc->H, desc->D, &desc->tiling, new_k, new_v, new_stride, k_cache,
+                            v_cache, desc->k_stride, desc->kv_tokens, start_idx, end_idx, stream);
+    if (rc) return rc;
+    return sfm_monarch_fwd(desc, q, k_cache, v_cache, out, workspace, workspace_bytes, stream);
+}
+
+static int check_dense(const sfm_dense_desc* d) {
+    if (!d) {
+        set_error("desc is NULL");
+        return SFM_ERR_NULL;
+    }
+    if (d->dtype != SFM_BF16 && d->dtype != SFM_F16 && d->dtype != SFM_F32) {
+        set_error("unsupported dtype %d", d->dtype);
+        return SFM_ERR_DTYPE;
+    }
+    if (d->B < 1 || d->H < 1 || d->D < 8 || d->D % 8 || d->D > 256 || d->q_tokens < 1 || d->kv_tokens < 1) {
+        set_error("B=%d, H=%d, D=%d, q_tokens=%d, kv_tokens=%d invalid", d->B, d->H, d->D, d->q_tokens, d->kv_tokens);
+        return SFM_ERR_SHAPE;
+    }
+    if (!(d->sm_scale > 0.f)) {
+        set_error("sm_scale must be a positive number");
+        return SFM_ERR_SHAPE;
+    }
+    const int esz = elem_size(d->dtype);
+    int rc;
+    if ((rc = check_strides("q", d->q_stride, d->q_tokens, d->H, d->D, d->B, esz))) return rc;
+    if ((rc = check_strides("k", d->k_stride, d->kv_tokens, d->H, d->D, d->B, esz))) return rc;
+    if ((rc = check_strides("v", d->v_stride, d->kv_tokens, d->H, d->D, d->B, esz))) return rc;
+    if ((rc = check_strides("out", d->o_stride, d->q_tokens, d->H, d->D, d->B, esz))) return rc;
+    return SFM_OK;
+}
+
+int sfm_dense_fwd(const sfm_dense_desc* desc, const void* q, const void* k, const void* v, void* out, float* lse,
+                  void* stream) {
+    int rc = check_dense(desc);
+    if (rc) return rc;
+    if (!q || !k || !v || !out) {
+        set_error("q, k, v and out must be non-NULL");
+        return SFM_ERR_NULL;
+    }
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) {
+        set_error("q, k, v and out must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    return launch_dense(*desc, q, k, v, out, lse, (hipStream_t)stream);
+}
+
+int sfm_full_attention_with_kv_cache(const sfm_dense_desc* desc, const void* q, void* k_cache, void* v_cache,
+                                     const void* new_k, const void* new_v, const int64_t new_stride[3],
+                                     int64_t start_idx, int64_t end_idx, void* out, float* lse, void* stream) {
+    int rc = check_dense(desc);
+    if (rc) return rc;
+    if (!q || !k_cache || !v_cache || !out || !new_k || !new_v || !new_stride) {
+        set_error("NULL argument");
+        return SFM_ERR_NULL;
+    }
+    if (start_idx < 0 || end_idx < start_idx || end_idx > desc->kv_tokens) {
+        set_error("start_idx=%lld, end_idx=%lld outside the cache view of %d tokens", (long long)start_idx,
+                  (long long)end_idx, desc->kv_tokens);
+        return SFM_ERR_RANGE;
+    }
+    if (memcmp(desc->k_stride, desc->v_stride, sizeof(desc->k_stride)) != 0) {
+        set_error("k_cache and v_cache must share strides");
+        return SFM_ERR_STRIDE;
+    }
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out) || !aligned16(new_k) ||
+        !aligned16(new_v)) {
+        set_error("tensors must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    const int64_t n = end_idx - start_idx;
+    if (n > 0) {
+        // token-order slice assignment = the identity tiling with one "frame" of n tokens
+        sfm_tiling ident = {1, 1, 1, 1, (int32_t)n};
+        rc = sfm_kv_cache_write(desc->dtype, desc->B, desc->H, desc->D, &ident, new_k, new_v, new_stride, k_cache,
+                                v_cache, desc->k_stride, desc->kv_tokens, start_idx, end_idx, stream);
+        if (rc) return rc;
+    }
+    return launch_dense(*desc, q, k_cache, v_cache, out, lse, (hipStream_t)stream);
+}
+
+int sfm_qk_prologue(const sfm_prologue_desc* d, const void* xq, const void* xk, const void* xv, const void* wq,
+                    const void* wk, const double* rope_cos_sin, int32_t rope_max_pos, void* q_out, void* k_cache,
+                    void* v_cache, void* stream) {
+    if (!d || !xq || !xk || !xv || !wq || !wk || !rope_cos_sin || !q_out || !k_cache || !v_cache) {
+        set_error("NULL argument");
+        return SFM_ERR_NULL;
+    }
+    if (d->dtype != SFM_BF16 && d->dtype != SFM_F16 && d->dtype != SFM_F32) {
+        set_error("unsupported dtype %d", d->dtype);
+        return SFM_ERR_DTYPE;
+    }
+    if (d->B < 1 || d->H < 1 || d->D < 8 || d->D % 8 || d->S < 1 || d->F < 1 || d->h < 1 || d->w < 1 ||
+        (int64_t)d->F * d->h * d->w != d->S) {
+        set_error("B=%d, S=%d, H=%d, D=%d, grid=(%d,%d,%d): need S == F*h*w and D a multiple of 8", d->B, d->S, d->H,
+                  d->D, d->F, d->h, d->w);
+        return SFM_ERR_SHAPE;
+    }
+    if ((int64_t)d->H * d->D > 8192) {
+        set_error("model dim %d exceeds the 8192 the fused prologue handles", d->H * d->D);
+        return SFM_ERR_UNSUPPORTED;
+    }
+    int rc = check_tiling(d->tiling);
+    if (rc) return rc;
+    if (d->tiling.h != d->h || d->tiling.w != d->w || d->F % d->tiling.f_tied) {
+        set_error("tiling (h=%d, w=%d, f_tied=%d) does not match the grid (%d,%d,%d)", d->tiling.h, d->tiling.w,
+                  d->tiling.f_tied, d->F, d->h, d->w);
+        return SFM_ERR_SHAPE;
+    }
+    if (d->start_frame < 0 || d->start_frame + d->F > rope_max_pos || d->h > rope_max_pos || d->w > rope_max_pos) {
+        set_error("RoPE positions exceed the table of %d rows", rope_max_pos);
+        return SFM_ERR_RANGE;
+    }
+    if (d->start_idx < 0 || d->start_idx + d->S > d->cache_tokens) {
+        set_error("start_idx=%lld + S=%d exceeds the cache of %lld tokens", (long long)d->start_idx, d->S,
+                  (long long)d->cache_tokens);
+        return SFM_ERR_RANGE;
+    }
+    const int esz = elem_size(d->dtype);
+    const int64_t C = (int64_t)d->H * d->D;
+    if (d->x_stride[1] < C || (d->x_stride[0] * esz) % 16 || (d->x_stride[1] * esz) % 16) {
+        set_error("x strides invalid");
+        return SFM_ERR_STRIDE;
+    }
+    if ((rc = check_strides("q_out", d->q_stride, d->S, d->H, d->D, d->B, esz))) return rc;
+    if ((rc = check_strides("k_cache/v_cache", d->cache_stride, d->cache_tokens, d->H, d->D, d->B, esz))) return rc;
+    if (!aligned16(xq) || !aligned16(xk) || !aligned16(xv) || !aligned16(wq) || !aligned16(wk) || !aligned16(q_out) ||
+        !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(rope_cos_sin)) {
+        set_error("tensors must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    TokMap map = make_map(d->tiling, 1);
+    return launch_prologue(*d, map, xq, xk, xv, wq, wk, rope_cos_sin, q_out, k_cache, v_cache, (hipStream_t)stream);
+}
+
+}  // extern "C"

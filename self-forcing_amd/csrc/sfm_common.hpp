@@ -1,0 +1,118 @@
+// Shared device/host helpers for the gfx950 attention kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "sfm_attn.h"
+
+namespace sfm {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// ---------------------------------------------------------------------------------------------
+// 16-bit element traits.  Storage is uint16_t; eight elements travel as one u32x4 (16 bytes).
+//
+// MFMA 32x32x16 operand layout on gfx950 (wave64):
+//   A (32 x 16): lane L supplies row  m = L % 32, k = 8*(L/32) + e, e = 0..7
+//   B (16 x 32): lane L supplies col  n = L % 32, k = 8*(L/32) + e
+//   D (32 x 32): lane L holds col n = L % 32; register v (0..15) holds row
+//                m = 8*(v/4) + 4*(L/32) + v%4
+// ---------------------------------------------------------------------------------------------
+struct BF16 {
+    static constexpr int kDtype = SFM_BF16;
+    static __device__ __forceinline__ float to_float(uint16_t u) { return __uint_as_float(((uint32_t)u) << 16); }
+    static __device__ __forceinline__ uint16_t from_float(float f) {
+        __bf16 b = (__bf16)f;
+        return __builtin_bit_cast(uint16_t, b);
+    }
+    static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+};
+
+struct F16 {
+    static constexpr int kDtype = SFM_F16;
+    static __device__ __forceinline__ float to_float(uint16_t u) { return (float)__builtin_bit_cast(_Float16, u); }
+    static __device__ __forceinline__ uint16_t from_float(float f) {
+        _Float16 b = (_Float16)f;
+        return __builtin_bit_cast(uint16_t, b);
+    }
+    static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+};
+
+template <class E>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+    return (uint32_t)E::from_float(lo) | ((uint32_t)E::from_float(hi) << 16);
+}
+
+// low / high 16-bit halves of two dwords -> one dword
+__device__ __forceinline__ uint32_t lo16x2(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }
+__device__ __forceinline__ uint32_t hi16x2(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
+
+__device__ __forceinline__ float xhalf_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
+__device__ __forceinline__ float xhalf_sum(float x) { return x + __shfl_xor(x, 32); }
+
+// Row of the 16x16-dword-permuted contraction index used when a D tile (rows = contraction
+// index) is fed back as a B operand: element e of lane-half hf in 16-wide step s.
+__device__ __forceinline__ int perm_row(int s, int hf, int e) { return 16 * s + 4 * hf + (e < 4 ? e : e + 4); }
+
+// ---------------------------------------------------------------------------------------------
+// Token index of a Monarch block coordinate (block-frame bf, block row i, block col 0).
+// natural = 0: rows are stored in block order ((bf*b1 + i)*b2 + j), the KV-cache layout.
+// natural = 1: rows are stored in (frame,row,col) token order and
+//     frame = A*f_tied + ft, row = c*hh + ii, col = e*ww + j  with  bf = (A*h_reduce + c)*w_reduce + e,
+//     i = ft*hh + ii.
+// Block columns j are always consecutive tokens.
+// ---------------------------------------------------------------------------------------------
+struct TokMap {
+    int b1, b2, hh, ww, h, w, f_tied, h_reduce, w_reduce, natural;
+    __host__ __device__ __forceinline__ int64_t row(int bf, int i) const {
+        if (!natural) return ((int64_t)bf * b1 + i) * b2;
+        int e = bf % w_reduce;
+        int t = bf / w_reduce;
+        int c = t % h_reduce;
+        int A = t / h_reduce;
+        int ft = i / hh;
+        int ii = i - ft * hh;
+        return ((int64_t)(A * f_tied + ft) * h + (c * hh + ii)) * w + e * ww;
+    }
+};
+
+struct MonarchArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* out;
+    void* kbar;      // [units_per_pass][na][b2][r_pad][D]   16-bit (MFMA path) or float (generic path)
+    void* y;         // same shape
+    float* cl;       // [units_per_pass][na][b2][r_pad]      sum_l R log2 R  (log2 units)
+    int B, H, D, na, nf, b1, b2;
+    int r_pad;       // rows per (a, j) block of the workspace: round_up(nf*b1, 32)
+    int unit0;       // first (b*H + h) unit of this pass
+    int causal;      // block-causal size in block-frames, 0 = none
+    float scale;
+    TokMap qmap, kmap;
+    int64_t qs[3], ks[3], vs[3], os[3];
+    int a_chunk;     // query block-frames per step-1 workgroup
+    int n_achunks;
+    int k_per_wg;    // block rows per step-1 workgroup
+};
+
+int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream);
+int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream);
+bool monarch_mfma_supported(int dtype, int D, int b2);
+
+void set_error(const char* fmt, ...);
+
+}  // namespace sfm

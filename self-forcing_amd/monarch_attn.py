@@ -1,0 +1,122 @@
+"""Monarch attention operators with the reference's call signatures.
+
+    monarch_attn_with_kv_cache  <->  wan/modules/monarch_attn.py:1778-1796
+    monarch_attn                <->  wan/modules/monarch_attn.py:1753-1776
+
+Inputs are [B, S, H, D] CUDA tensors (bf16 / fp16 / fp32, head_dim contiguous) in token order;
+the KV cache holds rows in Monarch block order and is updated in place.  Forward only.
+"""
+import ctypes as C
+
+import torch
+
+from . import lib as _l
+
+_DT = {torch.bfloat16: _l.SFM_BF16, torch.float16: _l.SFM_F16, torch.float32: _l.SFM_F32}
+
+
+def _check4(name, t, dtype=None, device=None):
+    if not isinstance(t, torch.Tensor) or t.dim() != 4:
+        raise ValueError(f"{name} must be a [B, S, H, D] tensor")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU")
+    if t.stride(3) != 1:
+        raise ValueError(f"{name}: head_dim must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise ValueError(f"{name}: dtype {t.dtype} differs from q's {dtype}")
+    if device is not None and t.device != device:
+        raise ValueError(f"{name}: device {t.device} differs from q's {device}")
+
+
+def _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, kv_block_order, causal_block_frames):
+    if q.dtype not in _DT:
+        raise ValueError(f"unsupported dtype {q.dtype}")
+    d = _l.MonarchDesc()
+    d.dtype = _DT[q.dtype]
+    d.B, d.q_tokens, d.H, d.D = q.shape
+    d.kv_tokens = k.shape[1]
+    d.tiling = _l.Tiling(f_tied, h_reduce, w_reduce, h, w)
+    d.kv_block_order = kv_block_order
+    d.causal_block_frames = causal_block_frames
+    d.sm_scale = float(sm_scale)
+    d.q_stride = _l.strides3(q)
+    d.k_stride = _l.strides3(k)
+    d.v_stride = _l.strides3(v)
+    d.o_stride = _l.strides3(out)
+    return d
+
+
+def monarch_workspace_bytes(desc, heads_per_pass=0):
+    n = C.c_size_t(0)
+    _l.check(_l.load().sfm_monarch_workspace_bytes(C.byref(desc), heads_per_pass, C.byref(n)))
+    return n.value
+
+
+def _stream(t):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, f_tied, h_reduce, w_reduce, h, w,
+                               sm_scale=None, num_iters=1, grad_only_new_kv=False, heads_per_pass=0):
+    """Writes new_k/new_v into k_cache/v_cache[:, start_idx:end_idx] (block order, in place) and
+    returns one-iteration Monarch attention of q against the whole cache view."""
+    if num_iters != 1:
+        raise NotImplementedError("num_iters > 1 (the reference's pure-torch refinement) is not built")
+    if torch.is_grad_enabled() and (q.requires_grad or new_k.requires_grad or new_v.requires_grad):
+        raise NotImplementedError("forward only: call under torch.no_grad()")
+    _check4("q", q)
+    for name, t in (("k_cache", k_cache), ("v_cache", v_cache), ("new_k", new_k), ("new_v", new_v)):
+        _check4(name, t, q.dtype, q.device)
+    if k_cache.shape != v_cache.shape or new_k.shape != new_v.shape:
+        raise ValueError("k/v shapes differ")
+    if new_k.stride() != new_v.stride():
+        new_v = new_v.contiguous()
+        new_k = new_k.contiguous()
+    if new_k.shape[1] != end_idx - start_idx:
+        raise ValueError(f"new_k holds {new_k.shape[1]} tokens but end_idx - start_idx = {end_idx - start_idx}")
+    if sm_scale is None:
+        sm_scale = q.shape[-1] ** -0.5
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    d = _desc(q, k_cache, v_cache, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1, 0)
+    nbytes = monarch_workspace_bytes(d, heads_per_pass)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        _l.check(_l.load().sfm_monarch_attn_with_kv_cache(
+            C.byref(d), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), new_k.data_ptr(), new_v.data_ptr(),
+            _l.strides3(new_k), start_idx, end_idx, out.data_ptr(), ws.data_ptr(), nbytes, _stream(q)))
+    return out
+
+
+def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block_causal_size=None, num_iters=1,
+                 heads_per_pass=0):
+    """One-iteration Monarch attention without a cache; `block_causal_size` (tokens) masks
+    block-frames of later causal blocks."""
+    if num_iters != 1:
+        raise NotImplementedError("num_iters > 1 (the reference's pure-torch refinement) is not built")
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        raise NotImplementedError("forward only: call under torch.no_grad()")
+    _check4("q", q)
+    _check4("k", k, q.dtype, q.device)
+    _check4("v", v, q.dtype, q.device)
+    if k.stride() != v.stride():
+        k, v = k.contiguous(), v.contiguous()
+    if sm_scale is None:
+        sm_scale = q.shape[-1] ** -0.5
+    cbf = 0
+    if block_causal_size is not None:
+        per_block = f_tied * (h // h_reduce) * (w // w_reduce)
+        if q.shape[1] % block_causal_size:
+            raise ValueError(f"block_causal_size ({block_causal_size}) must divide sequence length ({q.shape[1]})")
+        if k.shape[1] != q.shape[1]:
+            raise ValueError("causal attention needs kv length equal to q length")
+        if block_causal_size % per_block:
+            raise ValueError("block_causal_size must align with Monarch block sizes")
+        cbf = block_causal_size // per_block
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    d = _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 0, cbf)
+    nbytes = monarch_workspace_bytes(d, heads_per_pass)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        _l.check(_l.load().sfm_monarch_fwd(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                           ws.data_ptr(), nbytes, _stream(q)))
+    return out
