@@ -71,6 +71,12 @@ int sfm_monarch_workspace_bytes(const sfm_monarch_desc* desc, int32_t heads_per_
 int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
                     void* workspace, size_t workspace_bytes, void* stream);
 
+/* Measurement variant of sfm_monarch_fwd: brackets the two kernels of every pass with hipEvents recorded on
+ * `stream`, WAITS for them, and returns the summed kernel durations in milliseconds.  No counterpart in the
+ * reference (its pipeline times whole chunks with torch.cuda.Event, pipeline/causal_inference.py:105-115). */
+int sfm_monarch_fwd_timed(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
+                          void* workspace, size_t workspace_bytes, void* stream, float* step1_ms, float* step2_ms);
+
 /* Writes new_k/new_v [B, n_new, H, D] (token order) into k_cache/v_cache[:, start_idx:end_idx]
  * in Monarch block order.  Replaces monarch_attn.py:1784-1785 + 1230-1231.
  * strides: new_stride for new_k and new_v, cache_stride for both caches. */

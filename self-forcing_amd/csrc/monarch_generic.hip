@@ -161,7 +161,7 @@ bool monarch_generic_supported(const MonarchArgs& a) {
 }
 
 template <typename T>
-static int launch_generic_t(const MonarchArgs& a, int nunits, hipStream_t stream) {
+static int launch_generic_t(const MonarchArgs& a, int nunits, hipStream_t stream, const StepEvents* ev) {
     const size_t l1 = generic_lds1(a), l2 = generic_lds2(a);
     hipError_t err = hipSuccess;
     if (l1 > 64 * 1024)
@@ -172,8 +172,11 @@ static int launch_generic_t(const MonarchArgs& a, int nunits, hipStream_t stream
         set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(err));
         return SFM_ERR_HIP;
     }
+    if (ev) (void)hipEventRecord(ev->ev[0], stream);
     hipLaunchKernelGGL((monarch_generic_step1<T>), dim3(a.b1, a.nf, nunits * a.na), dim3(256), l1, stream, a);
+    if (ev) (void)hipEventRecord(ev->ev[1], stream);
     hipLaunchKernelGGL((monarch_generic_step2<T>), dim3(a.na * a.b2, nunits), dim3(256), l2, stream, a);
+    if (ev) (void)hipEventRecord(ev->ev[2], stream);
     err = hipGetLastError();
     if (err != hipSuccess) {
         set_error("hip launch failed: %s", hipGetErrorString(err));
@@ -182,14 +185,14 @@ static int launch_generic_t(const MonarchArgs& a, int nunits, hipStream_t stream
     return SFM_OK;
 }
 
-int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream) {
+int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev) {
     if (!monarch_generic_supported(a)) {
         set_error("block shape b2=%d, rows=%d, D=%d exceeds the LDS budget of the generic path", a.b2, a.nf * a.b1, a.D);
         return SFM_ERR_UNSUPPORTED;
     }
-    if (dtype == SFM_F32) return launch_generic_t<float>(a, nunits, stream);
-    if (dtype == SFM_BF16) return launch_generic_t<BF16>(a, nunits, stream);
-    return launch_generic_t<F16>(a, nunits, stream);
+    if (dtype == SFM_F32) return launch_generic_t<float>(a, nunits, stream, ev);
+    if (dtype == SFM_BF16) return launch_generic_t<BF16>(a, nunits, stream, ev);
+    return launch_generic_t<F16>(a, nunits, stream, ev);
 }
 
 }  // namespace sfm

@@ -483,7 +483,7 @@ bool monarch_mfma_supported(int dtype, int D, int b2) {
 }
 
 template <class E, int D>
-static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream) {
+static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const StepEvents* ev) {
     const int ncols = a.a_chunk * a.b2;
     const int ntiles = (ncols + 31) / 32;
     const int nwaves = ntiles < 4 ? 4 : ntiles;   // at least 4 waves so that K/V staging is <= 2 tasks per thread
@@ -502,10 +502,13 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream) {
         }
     }
     dim3 g1(kgroups, a.nf, nunits * a.n_achunks);
+    if (ev) (void)hipEventRecord(ev->ev[0], stream);
     hipLaunchKernelGGL((monarch_step1_kernel<E, D>), g1, dim3(nwaves * 64), lds1, stream, a);
+    if (ev) (void)hipEventRecord(ev->ev[1], stream);
     const int njg = (a.b2 + 3) / 4;
     dim3 g2(a.na * njg, nunits, (a.b1 + 31) / 32);
     hipLaunchKernelGGL((monarch_step2_kernel<E, D>), g2, dim3(256), S2Lds<D>::bytes(), stream, a);
+    if (ev) (void)hipEventRecord(ev->ev[2], stream);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) {
         set_error("hip launch failed: %s", hipGetErrorString(err));
@@ -514,9 +517,10 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream) {
     return SFM_OK;
 }
 
-int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream) {
-    if (dtype == SFM_BF16) return a.D == 128 ? launch_t<BF16, 128>(a, nunits, stream) : launch_t<BF16, 64>(a, nunits, stream);
-    return a.D == 128 ? launch_t<F16, 128>(a, nunits, stream) : launch_t<F16, 64>(a, nunits, stream);
+int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev) {
+    if (dtype == SFM_BF16)
+        return a.D == 128 ? launch_t<BF16, 128>(a, nunits, stream, ev) : launch_t<BF16, 64>(a, nunits, stream, ev);
+    return a.D == 128 ? launch_t<F16, 128>(a, nunits, stream, ev) : launch_t<F16, 64>(a, nunits, stream, ev);
 }
 
 }  // namespace sfm

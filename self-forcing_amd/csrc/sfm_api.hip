@@ -178,8 +178,8 @@ int sfm_monarch_workspace_bytes(const sfm_monarch_desc* desc, int32_t heads_per_
     return SFM_OK;
 }
 
-int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
-                    void* workspace, size_t workspace_bytes, void* stream) {
+static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
+                            void* workspace, size_t workspace_bytes, void* stream, float* step_ms) {
     MonarchPlan pl;
     int rc = plan_monarch(desc, &pl);
     if (rc) return rc;
@@ -227,11 +227,50 @@ int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, 
         a.kbar = workspace;
         a.y = (char*)workspace + mat_bytes * upp;
         a.cl = (float*)((char*)workspace + 2 * mat_bytes * upp);
-        rc = pl.mfma ? launch_monarch_mfma(a, desc->dtype, n, (hipStream_t)stream)
-                     : launch_monarch_generic(a, desc->dtype, n, (hipStream_t)stream);
+        StepEvents se;
+        if (step_ms) {
+            for (int i = 0; i < 3; ++i)
+                if (hipEventCreate(&se.ev[i]) != hipSuccess) {
+                    set_error("hipEventCreate failed");
+                    return SFM_ERR_HIP;
+                }
+        }
+        rc = pl.mfma ? launch_monarch_mfma(a, desc->dtype, n, (hipStream_t)stream, step_ms ? &se : nullptr)
+                     : launch_monarch_generic(a, desc->dtype, n, (hipStream_t)stream, step_ms ? &se : nullptr);
+        if (step_ms) {
+            float t1 = 0.f, t2 = 0.f;
+            hipError_t e = rc ? hipSuccess : hipEventSynchronize(se.ev[2]);
+            if (!rc && e == hipSuccess) e = hipEventElapsedTime(&t1, se.ev[0], se.ev[1]);
+            if (!rc && e == hipSuccess) e = hipEventElapsedTime(&t2, se.ev[1], se.ev[2]);
+            for (int i = 0; i < 3; ++i) (void)hipEventDestroy(se.ev[i]);
+            if (!rc && e != hipSuccess) {
+                set_error("event timing failed: %s", hipGetErrorString(e));
+                return SFM_ERR_HIP;
+            }
+            step_ms[0] += t1;
+            step_ms[1] += t2;
+        }
         if (rc) return rc;
     }
     return SFM_OK;
+}
+
+int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+    return monarch_fwd_impl(desc, q, k, v, out, workspace, workspace_bytes, stream, nullptr);
+}
+
+int sfm_monarch_fwd_timed(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
+                          void* workspace, size_t workspace_bytes, void* stream, float* step1_ms, float* step2_ms) {
+    if (!step1_ms || !step2_ms) {
+        set_error("step1_ms / step2_ms are NULL");
+        return SFM_ERR_NULL;
+    }
+    float ms[2] = {0.f, 0.f};
+    int rc = monarch_fwd_impl(desc, q, k, v, out, workspace, workspace_bytes, stream, ms);
+    *step1_ms = ms[0];
+    *step2_ms = ms[1];
+    return rc;
 }
 
 int sfm_kv_cache_write(int32_t dtype, int32_t B, int32_t H, int32_t D, const sfm_tiling* tiling, const void* new_k,

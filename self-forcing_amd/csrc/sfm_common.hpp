@@ -109,8 +109,13 @@ struct MonarchArgs {
     int k_per_wg;    // block rows per step-1 workgroup
 };
 
-int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream);
-int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream);
+// Optional timing hooks: ev[0] is recorded before step 1, ev[1] between the steps, ev[2] after step 2.
+struct StepEvents {
+    hipEvent_t ev[3];
+};
+
+int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev);
+int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev);
 bool monarch_mfma_supported(int dtype, int D, int b2);
 
 void set_error(const char* fmt, ...);

@@ -18,7 +18,7 @@ ERR_NAMES = {
 
 # every symbol include/sfm_attn.h declares
 SYMBOLS = [
-    "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
+    "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_last_error", "sfm_version",
 ]
 
@@ -72,6 +72,8 @@ def load():
     lib.sfm_last_error.restype = C.c_char_p
     lib.sfm_monarch_workspace_bytes.argtypes = [C.POINTER(MonarchDesc), C.c_int32, C.POINTER(C.c_size_t)]
     lib.sfm_monarch_fwd.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, C.c_size_t, P]
+    lib.sfm_monarch_fwd_timed.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, C.c_size_t, P,
+                                          C.POINTER(C.c_float), C.POINTER(C.c_float)]
     lib.sfm_kv_cache_write.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(Tiling), P, P, S3, P, P,
                                        S3, I64, I64, I64, P]
     lib.sfm_monarch_attn_with_kv_cache.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, S3, I64, I64, P, P,

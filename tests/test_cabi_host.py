@@ -1,0 +1,156 @@
+"""CPU-only checks of the C-ABI boundary: the library loads, exports every symbol the header
+declares, and rejects bad arguments with error codes before touching any device."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from self_forcing_amd import lib as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sfm_attn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sfm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = L.load()
+    names = _declared_symbols()
+    assert len(names) >= 9 and set(names) == set(L.SYMBOLS)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.sfm_version() == 1
+
+
+def test_struct_sizes_match_header_layout():
+    # int32 x 6, tiling (5 x int32), 2 x int32, float, pad to 8, 12 x int64
+    assert C.sizeof(L.Tiling) == 20
+    assert C.sizeof(L.MonarchDesc) == 56 + 12 * 8
+    assert C.sizeof(L.DenseDesc) == 32 + 12 * 8
+    assert C.sizeof(L.PrologueDesc) == 64 + 8 * 8 + 16
+
+
+def _desc(**kw):
+    d = L.MonarchDesc()
+    d.dtype, d.B, d.H, d.D = L.SFM_BF16, 1, 2, 128
+    d.q_tokens, d.kv_tokens = 3 * 30 * 52, 21 * 30 * 52
+    d.tiling = L.Tiling(1, 1, 1, 30, 52)
+    d.kv_block_order, d.causal_block_frames, d.sm_scale = 1, 0, 128 ** -0.5
+    for name in ("q_stride", "k_stride", "v_stride", "o_stride"):
+        toks = d.kv_tokens if name[0] in "kv" else d.q_tokens
+        setattr(d, name, (C.c_int64 * 3)(toks * 256, 256, 128))
+    for k, v in kw.items():
+        setattr(d, k, v)
+    return d
+
+
+def _ws(d, hpp=0):
+    n = C.c_size_t(0)
+    rc = L.load().sfm_monarch_workspace_bytes(C.byref(d), hpp, C.byref(n))
+    return rc, n.value
+
+
+def test_workspace_bytes_accounting():
+    rc, n1 = _ws(_desc(), 1)
+    assert rc == 0
+    # per unit: 2 matrices of a*b2*r_pad rows x D bf16 + one fp32 per row, r_pad = round_up(21*30, 32)
+    rows = 3 * 52 * 640
+    assert n1 == rows * 128 * 2 * 2 + rows * 4
+    rc, n2 = _ws(_desc(), 2)
+    assert rc == 0 and n2 == 2 * n1
+    rc, nall = _ws(_desc(), 99)
+    assert rc == 0 and nall == 2 * n1          # clamped to B*H units
+    # fp32 tensors take the generic path, which keeps its scratch rows in float
+    rc, nf32 = _ws(_desc(dtype=L.SFM_F32), 1)
+    assert rc == 0 and nf32 == rows * 128 * 4 * 2 + rows * 4
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(dtype=7), -2),
+    (dict(D=100), -3),
+    (dict(q_tokens=1000), -3),
+    (dict(kv_tokens=30 * 52 + 1), -3),
+    (dict(tiling=L.Tiling(1, 4, 1, 30, 52)), -3),
+    (dict(tiling=L.Tiling(0, 1, 1, 30, 52)), -3),
+    (dict(sm_scale=0.0), -3),
+    (dict(causal_block_frames=3), -3),                 # needs q_tokens == kv_tokens
+    (dict(q_stride=(C.c_int64 * 3)(0, 256, 64)), -5),  # head stride < D
+    (dict(v_stride=(C.c_int64 * 3)(1 << 20, 512, 128)), -5),   # differs from k_stride
+    (dict(k_stride=(C.c_int64 * 3)(1 << 20, 257, 128), v_stride=(C.c_int64 * 3)(1 << 20, 257, 128)), -5),
+])
+def test_monarch_desc_validation(kw, code):
+    rc, _ = _ws(_desc(**kw))
+    assert rc == code
+    assert L.load().sfm_last_error() != b""
+
+
+def test_monarch_fwd_pointer_and_workspace_checks():
+    lib = L.load()
+    d = _desc()
+    _, need = _ws(d, 1)
+    fake = 0x10000
+    assert lib.sfm_monarch_fwd(C.byref(d), None, fake, fake, fake, fake, need, None) == -1
+    assert lib.sfm_monarch_fwd(C.byref(d), fake + 2, fake, fake, fake, fake, need, None) == -7
+    assert lib.sfm_monarch_fwd(C.byref(d), fake, fake, fake, fake, None, need, None) == -6
+    assert lib.sfm_monarch_fwd(C.byref(d), fake, fake, fake, fake, fake + 16, need, None) == -6
+    assert lib.sfm_monarch_fwd(C.byref(d), fake, fake, fake, fake, fake, need - 1, None) == -6
+    assert lib.sfm_monarch_fwd(None, fake, fake, fake, fake, fake, need, None) == -1
+
+
+def test_kv_cache_op_range_checks_happen_before_any_write():
+    lib = L.load()
+    d = _desc()
+    _, need = _ws(d, 1)
+    fake = 0x10000
+    ns = (C.c_int64 * 3)(4680 * 256, 256, 128)
+    blk = 30 * 52
+    call = lambda s, e, **kw: lib.sfm_monarch_attn_with_kv_cache(
+        C.byref(_desc(**kw)), fake, fake, fake, fake, fake, ns, s, e, fake, fake, need, None)
+    assert call(18 * blk + 1, 21 * blk) == -4          # not aligned to a block-frame
+    assert call(18 * blk, 22 * blk) == -4              # past the end of the view
+    assert call(-blk, 2 * blk) == -4
+    assert call(3 * blk, 2 * blk) == -4
+    assert call(18 * blk, 21 * blk, kv_block_order=0) == -9
+
+
+def test_dense_and_prologue_validation():
+    lib = L.load()
+    fake = 0x10000
+    d = L.DenseDesc()
+    d.dtype, d.B, d.H, d.D, d.q_tokens, d.kv_tokens, d.sm_scale = L.SFM_BF16, 1, 2, 128, 10, 20, 0.1
+    for name in ("q_stride", "k_stride", "v_stride", "o_stride"):
+        setattr(d, name, (C.c_int64 * 3)(20 * 256, 256, 128))
+    assert lib.sfm_dense_fwd(C.byref(d), fake, fake, None, fake, None, None) == -1
+    d.D = 12
+    assert lib.sfm_dense_fwd(C.byref(d), fake, fake, fake, fake, None, None) == -3
+    d.D = 128
+    ns = (C.c_int64 * 3)(5 * 256, 256, 128)
+    assert lib.sfm_full_attention_with_kv_cache(C.byref(d), fake, fake, fake, fake, fake, ns, 18, 23, fake, None, None) == -4
+
+    p = L.PrologueDesc()
+    p.dtype, p.B, p.S, p.H, p.D = L.SFM_BF16, 1, 24, 2, 128
+    p.F, p.h, p.w, p.start_frame, p.eps = 1, 4, 6, 0, 1e-6
+    p.tiling = L.Tiling(1, 1, 1, 4, 6)
+    p.x_stride = (C.c_int64 * 2)(24 * 256, 256)
+    p.q_stride = (C.c_int64 * 3)(24 * 256, 256, 128)
+    p.cache_stride = (C.c_int64 * 3)(48 * 256, 256, 128)
+    p.cache_tokens, p.start_idx = 48, 24
+    args = [fake] * 6
+    assert lib.sfm_qk_prologue(C.byref(p), *args, 1024, fake, fake, None, None) == -1
+    p.start_idx = 30
+    assert lib.sfm_qk_prologue(C.byref(p), *args, 1024, fake, fake, fake, None) == -4
+    p.start_idx, p.start_frame = 24, 1024
+    assert lib.sfm_qk_prologue(C.byref(p), *args, 1024, fake, fake, fake, None) == -4
+    p.start_frame, p.S = 0, 25
+    assert lib.sfm_qk_prologue(C.byref(p), *args, 1024, fake, fake, fake, None) == -3
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(L, "_lib", None)
+    monkeypatch.setattr(L, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no fallback"):
+        L.load()

@@ -1,0 +1,189 @@
+"""GPU parity of the Monarch attention kernels against the CPU oracle, through the C ABI.
+
+Tolerances: fp32 path <= 1e-5 max-abs; 16-bit paths the reference's atol = rtol = 1e-2 (bf16) /
+1e-3 (fp16) against the fp32 oracle, and max-abs < 2e-2 with per-head cosine > 0.999."""
+import pytest
+import torch
+
+import self_forcing_amd as sfa
+from gpu_util import assert_close_16bit, max_abs, per_head_cosine, randn
+from oracle import blocks, dense, monarch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+mattn = sfa.monarch_attn
+
+
+def _tokens(F, h, w):
+    return F * h * w
+
+
+def test_c1_plumbing_fp32():
+    """B=1, H=2, D=64, 3 frames of 8x8 tokens, q,k,v ~ N(0,1) drawn in this order from seed 0."""
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(1, 192, 2, 64, generator=g) for _ in range(3))
+    ref = monarch.monarch_attn(q, k, v, 1, 1, 1, 8, 8, sm_scale=0.125)
+    out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, 8, 8, sm_scale=0.125)
+    assert max_abs(out, ref) < 1e-5
+    # same case through the KV-cache entry point: cache holds frames 0-1, frame 2 arrives
+    kc, vc = torch.zeros(1, 192, 2, 64, device=DEV), torch.zeros(1, 192, 2, 64, device=DEV)
+    kc[:, :128], vc[:, :128] = k[:, :128].to(DEV), v[:, :128].to(DEV)
+    out2 = mattn.monarch_attn_with_kv_cache(q.to(DEV), kc, vc, k[:, 128:].to(DEV), v[:, 128:].to(DEV), 128, 192,
+                                            1, 1, 1, 8, 8, sm_scale=0.125)
+    assert max_abs(out2, ref) < 1e-5
+    assert torch.equal(kc.cpu(), k) and torch.equal(vc.cpu(), v)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,D,a,f,b1,b2", [
+    (1, 1, 128, 1, 1, 2, 8),          # single wave tile, one row tile of keys
+    (1, 2, 128, 3, 4, 6, 52),         # the 52-column block of the 480p grid
+    (2, 2, 64, 2, 3, 5, 20),          # head_dim 64, ragged everything
+    (1, 2, 128, 6, 6, 15, 52),        # reduce2xh-like: two query chunks per step-1 workgroup group
+    (1, 1, 128, 2, 3, 40, 33),        # more than 32 block rows: two query-row tiles in step 2
+    (1, 3, 64, 5, 2, 3, 64),          # full 64-wide key tile
+    (1, 1, 128, 9, 2, 4, 32),         # 9 x 32 = 288 columns: query block-frames split across workgroups
+])
+def test_mfma_path_small_shapes(dtype, B, H, D, a, f, b1, b2):
+    q, k, v = (randn((B, n * b1 * b2, H, D), 10 + i, dtype) for i, n in enumerate((a, f, f)))
+    ref = monarch.monarch_attn(q, k, v, 1, 1, 1, b1, b2, dtype=torch.float32)
+    out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, b1, b2)
+    assert_close_16bit(out, ref, dtype)
+
+
+@pytest.mark.parametrize("heads_per_pass", [1, 2, 5])
+def test_head_passes_give_identical_results(heads_per_pass):
+    q, k, v = (randn((1, n * 6 * 20, 5, 128), 20 + i, torch.bfloat16).to(DEV) for i, n in enumerate((2, 3, 3)))
+    full = mattn.monarch_attn(q, k, v, 1, 1, 1, 6, 20, heads_per_pass=5)
+    part = mattn.monarch_attn(q, k, v, 1, 1, 1, 6, 20, heads_per_pass=heads_per_pass)
+    assert torch.equal(full, part)
+
+
+@pytest.mark.parametrize("f_tied,h_reduce,w_reduce", [(1, 1, 1), (1, 2, 1), (3, 1, 1), (1, 2, 2), (3, 3, 4), (1, 6, 13)])
+def test_kv_cache_op_tilings(f_tied, h_reduce, w_reduce):
+    """Every tiling: output vs oracle and the cache contents (block order) bit for bit."""
+    h, w, H, D = 6, 52, 2, 128
+    dtype = torch.bfloat16
+    nq, nc = 3 * h * w, 9 * h * w
+    q, nk, nv = (randn((1, nq, H, D), 30 + i, dtype) for i in range(3))
+    kc, vc = randn((1, nc, H, D), 33, dtype), randn((1, nc, H, D), 34, dtype)
+    kc_o, vc_o = kc.clone(), vc.clone()
+    ref = monarch.monarch_attn_with_kv_cache(q, kc_o, vc_o, nk, nv, nc - nq, nc, f_tied, h_reduce, w_reduce, h, w,
+                                             dtype=torch.float32)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    out = mattn.monarch_attn_with_kv_cache(q.to(DEV), kd, vd, nk.to(DEV), nv.to(DEV), nc - nq, nc, f_tied, h_reduce,
+                                           w_reduce, h, w)
+    assert torch.equal(kd.cpu(), kc_o) and torch.equal(vd.cpu(), vc_o)
+    assert_close_16bit(out, ref, dtype)
+
+
+def test_kv_cache_view_with_batch_stride_and_prefix():
+    """B=2, the op sees kv_cache[:, :local_end] of a longer allocation (batch stride = full cache)."""
+    h, w, H, D = 4, 20, 2, 64
+    dtype = torch.float16
+    blk = h * w
+    full_k, full_v = randn((2, 8 * blk, H, D), 40, dtype).to(DEV), randn((2, 8 * blk, H, D), 41, dtype).to(DEV)
+    sentinel_k = full_k[:, 5 * blk:].clone()
+    q, nk, nv = (randn((2, 2 * blk, H, D), 42 + i, dtype) for i in range(3))
+    kc_o, vc_o = full_k[:, :5 * blk].cpu().clone(), full_v[:, :5 * blk].cpu().clone()
+    ref = monarch.monarch_attn_with_kv_cache(q, kc_o, vc_o, nk, nv, 3 * blk, 5 * blk, 1, 1, 1, h, w, dtype=torch.float32)
+    out = mattn.monarch_attn_with_kv_cache(q.to(DEV), full_k[:, :5 * blk], full_v[:, :5 * blk], nk.to(DEV), nv.to(DEV),
+                                           3 * blk, 5 * blk, 1, 1, 1, h, w)
+    assert_close_16bit(out, ref, dtype)
+    assert torch.equal(full_k[:, :5 * blk].cpu(), kc_o)
+    assert torch.equal(full_k[:, 5 * blk:], sentinel_k)          # nothing written past the view
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_block_causal_no_cache(dtype):
+    h, w, H, D, F = 3, 20, 2, 64, 6
+    q, k, v = (randn((1, F * h * w, H, D), 50 + i, dtype) for i in range(3))
+    for bcs in (h * w, 3 * h * w):
+        ref = monarch.monarch_attn_causal_chunked(q, k, v, 1, 1, 1, h, w, bcs, dtype=torch.float32)
+        out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, h, w, block_causal_size=bcs)
+        if dtype == torch.float32:
+            assert max_abs(out, ref) < 1e-5
+        else:
+            assert_close_16bit(out, ref, dtype, atol_scale=2.0)      # the reference's causal bar is 2e-2
+
+
+def test_generic_path_wide_blocks():
+    """b2 = 80 (the 720p grid) is outside the MFMA kernels and runs the fp32 generic kernels."""
+    q, k, v = (randn((1, n * 3 * 80, 2, 128), 60 + i, torch.bfloat16) for i, n in enumerate((2, 3, 3)))
+    ref = monarch.monarch_attn(q, k, v, 1, 1, 1, 3, 80, dtype=torch.float32)
+    out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, 3, 80)
+    assert_close_16bit(out, ref, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B", [1, 2])
+def test_reference_kv_cache_test_shape(dtype, B):
+    """The reference's own harness shape (monarch_attn.py:1981-1984): A=3, F=21, 30x52, H=12, D=128, new_f=3.
+    The oracle is evaluated on 3 of the 12 heads to keep the CPU side to seconds."""
+    A, F, b1, b2, H, D, new_f = 3, 21, 30, 52, 12, 128, 3
+    q = randn((B, A * b1 * b2, H, D), 70, dtype)
+    kc, vc = randn((B, F * b1 * b2, H, D), 71, dtype), randn((B, F * b1 * b2, H, D), 72, dtype)
+    nk, nv = randn((B, new_f * b1 * b2, H, D), 73, dtype), randn((B, new_f * b1 * b2, H, D), 74, dtype)
+    start, end = (F - new_f) * b1 * b2, F * b1 * b2
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    out = mattn.monarch_attn_with_kv_cache(q.to(DEV), kd, vd, nk.to(DEV), nv.to(DEV), start, end, 1, 1, 1, b1, b2,
+                                           D ** -0.5)
+    heads = [0, 5, 11]
+    kc[:, start:end], vc[:, start:end] = nk, nv
+    assert torch.equal(kd.cpu(), kc) and torch.equal(vd.cpu(), vc)
+    ref = monarch.monarch_attn(q[:, :, heads], kc[:, :, heads], vc[:, :, heads], 1, 1, 1, b1, b2, dtype=torch.float32)
+    assert_close_16bit(out[:, :, heads], ref, dtype)
+
+
+@pytest.mark.parametrize("frames", [3, 6, 9, 12, 15, 18, 21])
+def test_kv_length_sweep(frames):
+    """Cache grows by one chunk per generated chunk: f in {3, ..., 21} at the 30 x 52 block."""
+    b1, b2, H, D = 30, 52, 2, 128
+    q = randn((1, 3 * b1 * b2, H, D), 80, torch.bfloat16)
+    k, v = randn((1, frames * b1 * b2, H, D), 81, torch.bfloat16), randn((1, frames * b1 * b2, H, D), 82, torch.bfloat16)
+    ref = monarch.monarch_attn(q[:, :, :1], k[:, :, :1], v[:, :, :1], 1, 1, 1, b1, b2, dtype=torch.float32)
+    out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, b1, b2)
+    assert_close_16bit(out[:, :, :1], ref, torch.bfloat16)
+
+
+def test_full_size_properties_c2():
+    """Size-independent facts at the full C2 shape (H=12, 4680 queries vs 32760 keys):
+    constant V gives constant output; permuting KV block-frames changes nothing (up to rounding)."""
+    b1, b2, H, D = 30, 52, 12, 128
+    q = randn((1, 3 * b1 * b2, H, D), 90, torch.bfloat16).to(DEV)
+    k = randn((1, 21 * b1 * b2, H, D), 91, torch.bfloat16).to(DEV)
+    v = randn((1, 21 * b1 * b2, H, D), 92, torch.bfloat16).to(DEV)
+    const = torch.full_like(v, 1.5)
+    out = mattn.monarch_attn(q, k, const, 1, 1, 1, b1, b2)
+    assert (out.float() - 1.5).abs().max().item() <= 2 ** -6     # one bf16 ulp at 1.5
+    base = mattn.monarch_attn(q, k, v, 1, 1, 1, b1, b2)
+    perm = torch.randperm(21, generator=torch.Generator().manual_seed(1))
+    kp = k.view(1, 21, b1 * b2, H, D)[:, perm].reshape(k.shape)
+    vp = v.view(1, 21, b1 * b2, H, D)[:, perm].reshape(v.shape)
+    other = mattn.monarch_attn(q, kp, vp, 1, 1, 1, b1, b2)
+    assert max_abs(base, other) < 4e-3
+    assert per_head_cosine(base, other) > 0.9999
+
+
+def test_monarch_vs_dense_is_reported_not_asserted(capsys):
+    """Monarch is an approximation of dense attention; the gap on random inputs is printed."""
+    b1, b2, H, D = 30, 52, 2, 128
+    q, k, v = (randn((1, n * b1 * b2, H, D), 95 + i, torch.bfloat16).to(DEV) for i, n in enumerate((3, 6, 6)))
+    m = mattn.monarch_attn(q, k, v, 1, 1, 1, b1, b2)
+    d = sfa.attention.attention(q, k, v)
+    print(f"monarch vs dense: max-abs {max_abs(m, d):.3e}, per-head cosine {per_head_cosine(m, d):.4f}")
+
+
+def test_host_argument_errors():
+    q = randn((1, 60, 2, 64), 1, torch.bfloat16).to(DEV)
+    kc = randn((1, 120, 2, 64), 2, torch.bfloat16).to(DEV)
+    with pytest.raises(ValueError):
+        mattn.monarch_attn_with_kv_cache(q, kc, kc.clone(), q, q, 50, 110, 1, 1, 1, 3, 20)   # start not block aligned
+    with pytest.raises(ValueError):
+        mattn.monarch_attn_with_kv_cache(q, kc, kc.clone(), q, q, 60, 120, 1, 1, 1, 4, 20)   # 60 tokens != k * 80
+    with pytest.raises(ValueError):
+        mattn.monarch_attn(q.cpu(), kc, kc, 1, 1, 1, 3, 20)
+    with pytest.raises(ValueError):
+        mattn.monarch_attn(q, kc, kc, 1, 1, 1, 3, 20, block_causal_size=60)                  # needs Skv == Sq
+    with pytest.raises(NotImplementedError):
+        mattn.monarch_attn(q, kc, kc, 1, 1, 1, 3, 20, num_iters=4)
