@@ -108,10 +108,10 @@ __global__ __launch_bounds__(256) void dense_fwd_kernel(sfm_dense_desc p, const 
 
     prefetch(0);
     for (int tile = 0; tile < ntile; ++tile) {
-        __syncthreads();
+        lds_barrier();                   // everyone is done reading the previous tile
         commit();
         if (tile + 1 < ntile) prefetch(64 * (tile + 1));
-        __syncthreads();
+        lds_barrier();                   // tile visible; the prefetch stays in flight
 
         f32x16 s[2];
 #pragma unroll

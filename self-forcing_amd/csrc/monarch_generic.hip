@@ -71,7 +71,7 @@ __global__ __launch_bounds__(256) void monarch_generic_step1(MonarchArgs p) {
             ent += e * zs[l];
         }
         const float inv = 1.f / sum;
-        const int64_t blk = (((int64_t)ul * p.na + a) * b2 + j) * p.r_pad + (int64_t)f * p.b1 + k;
+        const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj + (int64_t)(f * p.b1 + k) * p.ws_row;
         if (tid == 0) p.cl[blk] = ent * inv - (mx + log2f(sum));
         for (int d = tid; d < D; d += nt) {
             float ak = 0.f, av = 0.f;
@@ -103,7 +103,8 @@ __global__ __launch_bounds__(256) void monarch_generic_step2(MonarchArgs p) {
     float* zs = qs + D;        // [R]
     float* red = zs + R;       // [nt]
 
-    const int64_t blk = (((int64_t)ul * p.na + a) * b2 + j) * p.r_pad;
+    const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj;
+    const int64_t rs = p.ws_row;
     const float* kbar = (const float*)p.kbar + blk * D;
     const float* yw = (const float*)p.y + blk * D;
     const float* cl = p.cl + blk;
@@ -118,9 +119,9 @@ __global__ __launch_bounds__(256) void monarch_generic_step2(MonarchArgs p) {
         float mx = -INFINITY;
         for (int r = tid; r < R; r += nt) {
             float acc = 0.f;
-            const float* row = kbar + (int64_t)r * D;
+            const float* row = kbar + (int64_t)r * rs * D;
             for (int d = 0; d < D; ++d) acc += qs[d] * row[d];
-            float z = acc * sc2 - cl[r];
+            float z = acc * sc2 - cl[r * rs];
             zs[r] = z;
             mx = fmaxf(mx, z);
         }
@@ -147,7 +148,7 @@ __global__ __launch_bounds__(256) void monarch_generic_step2(MonarchArgs p) {
         const float inv = 1.f / red[0];
         for (int d = tid; d < D; d += nt) {
             float acc = 0.f;
-            for (int r = 0; r < R; ++r) acc += zs[r] * yw[(int64_t)r * D + d];
+            for (int r = 0; r < R; ++r) acc += zs[r] * yw[(int64_t)r * rs * D + d];
             Ld<T>::put(p.out, (int64_t)b * p.os[0] + tok * p.os[1] + (int64_t)h * p.os[2] + d, acc * inv);
         }
     }

@@ -33,48 +33,74 @@ template <int D>
 struct S1Lds {
     static constexpr int kRowPitch = D + 8;    // u16 per row of row-major K   [64][D+8]
     static constexpr int kTPitch = 72;         // u16 per row of K^T / V^T     [D][64+8]
-    static constexpr int kStagePitch = 72;     // u16 per row of a wave's output stage [32][64+8]
-    static constexpr int kKrow = 0;
-    static constexpr int kKT = kKrow + 64 * kRowPitch;
-    static constexpr int kVT = kKT + D * kTPitch;
-    static constexpr int kStage = kVT + D * kTPitch;
+    static constexpr int kStagePitch = 40;     // u16 per row of a wave's output stage [32][32+8]
     static constexpr int kStagePerWave = 32 * kStagePitch;
-    static __host__ __device__ constexpr size_t bytes(int nwaves) { return 2 * (size_t)(kStage + nwaves * kStagePerWave); }
+    // The stages share their LDS with the row-major K tile: that tile is dead once every wave has its
+    // logits, and the stages are dead before the next tile is committed.
+    static __host__ __device__ constexpr int union_elems(int nwaves) {
+        return 64 * kRowPitch > nwaves * kStagePerWave ? 64 * kRowPitch : nwaves * kStagePerWave;
+    }
+    static __host__ __device__ constexpr size_t bytes(int nwaves) { return 2 * (size_t)(union_elems(nwaves) + 2 * D * kTPitch); }
 };
 
 template <class E, int D>
-__global__ __launch_bounds__(512) void monarch_step1_kernel(MonarchArgs p) {
+__global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) void monarch_step1_kernel(MonarchArgs p) {
     using L = S1Lds<D>;
     constexpr int DS = D / 16;   // contraction steps of the logits
-    constexpr int DT = D / 32;   // 32-row tiles of the transposed outputs
     constexpr int DP = D / 2;    // dword columns of a K/V row
-    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds_all[];
 
-    const int tid = threadIdx.x;
-    const int nthreads = blockDim.x;
+    // A workgroup is `p.s1_groups` independent wave groups that share nothing but the barriers: group g
+    // works on kv block-frame f0 + g, f0 + g + groups, ... with its own LDS tiles.  Two groups of 5 waves
+    // put 3,3,2,2 waves on the four SIMDs, which one group of 5 cannot (waves go to SIMDs round-robin).
+    const int nthreads = blockDim.x / p.s1_groups;        // threads of one group
+    const int grp = threadIdx.x / nthreads;
+    const int tid = threadIdx.x - grp * nthreads;
+    const int nwaves = nthreads >> 6;
     const int wave = tid >> 6;
     const int lane = tid & 63;
     const int m = lane & 31;
     const int hf = lane >> 5;
 
-    const int f = blockIdx.y;
-    const int ul = blockIdx.z / p.n_achunks;              // unit within this pass
-    const int a0 = (blockIdx.z % p.n_achunks) * p.a_chunk;
+    uint16_t* const lds = lds_all + grp * (L::bytes(nwaves) / 2);
+    uint16_t* const lds_krow = lds;                                  // [64][D+8], aliased by the stages
+    uint16_t* const lds_kt = lds + L::union_elems(nwaves);           // [D][72]
+    uint16_t* const lds_vt = lds_kt + D * L::kTPitch;                // [D][72]
+    uint16_t* const stage = lds + wave * L::kStagePerWave;           // [32][40], private to the wave
+
+    // Workgroup = (unit, a-chunk, key block row k, range of kv block-frames f).  The query rows
+    // Q[a, k, :, :] of the chunk depend on k only, so they are loaded once and stay in registers for
+    // every f of the range.  Workgroups are handed to the 8 XCDs round-robin (id % 8); give each XCD a
+    // contiguous range of the logical order.
+    const int per_xcd = gridDim.x >> 3;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= p.s1_total) return;
+    const int nfs = (p.nf + p.f_per_wg - 1) / p.f_per_wg;
+    const int fs = logical % nfs;
+    const int kz = logical / nfs;
+    const int k = kz % p.b1;
+    const int z = kz / p.b1;
+    const int ul = z / p.n_achunks;                       // unit within this pass
+    const int a0 = (z % p.n_achunks) * p.a_chunk;
     const int a_cnt = min(p.a_chunk, p.na - a0);
     const int unit = p.unit0 + ul;
     const int b = unit / p.H, h = unit % p.H;
-    const int k0 = blockIdx.x * p.k_per_wg;
-    const int k1 = min(k0 + p.k_per_wg, p.b1);
-    if (p.causal && ((a0 + a_cnt - 1) / p.causal) < (f / p.causal)) return;   // every a of the chunk is masked
+    const int f0 = fs * p.f_per_wg;
+    int f1 = min(f0 + p.f_per_wg, p.nf);
+    if (p.causal) f1 = min(f1, ((a0 + a_cnt - 1) / p.causal + 1) * p.causal);   // later block-frames are masked for every a
+    if (f0 >= f1) return;
 
     const int b2 = p.b2;
     const int ncols = a_cnt * b2;
     const int NT = b2 > 32 ? 2 : 1;                       // 32-row tiles of the key axis l
-    const bool tile_active = wave * 32 < ncols;
+    const bool tile_ok = wave * 32 < ncols;
 
+    // Uniform 64-bit bases; everything that varies per lane is a 32-bit element offset from them
+    // (the host checks that each tensor and the scratch of one pass stay below 2^31 elements).
     const uint16_t* qg = (const uint16_t*)p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[2];
     const uint16_t* kg = (const uint16_t*)p.k + (int64_t)b * p.ks[0] + (int64_t)h * p.ks[2];
     const uint16_t* vg = (const uint16_t*)p.v + (int64_t)b * p.vs[0] + (int64_t)h * p.vs[2];
+    const uint32_t qs1 = (uint32_t)p.qs[1], ks1 = (uint32_t)p.ks[1];
 
     // column owned by this lane in the logits/contraction phase
     const int cg = wave * 32 + m;
@@ -82,97 +108,109 @@ __global__ __launch_bounds__(512) void monarch_step1_kernel(MonarchArgs p) {
     const int ca = a0 + (col_ok ? cg / b2 : 0);
     const int cj = col_ok ? cg % b2 : 0;
 
-    // rows this lane stores in the epilogue: 4 rows, r = 8*it + lane/8 of the wave's 32 columns
-    const int R = p.nf * p.b1;
-    int64_t orow[4];
-    bool orow_ok[4];
+    // logits operand (B): this lane's query row Q[ca, k, cj, 16 ds + 8 hf + 0..7]
+    u32x4 qb[DS];
+    {
+        const uint16_t* qrow = qg + ((uint32_t)(p.qmap.row(ca, k) + cj) * qs1 + 8 * hf);
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-        int c = wave * 32 + it * 8 + (lane >> 3);
-        orow_ok[it] = c < ncols;
-        int aa = a0 + (orow_ok[it] ? c / b2 : 0);
-        int jj = orow_ok[it] ? c % b2 : 0;
-        orow[it] = ((((int64_t)ul * p.na + aa) * b2 + jj) * p.r_pad + (int64_t)f * p.b1) * D + (lane & 7) * 8;
+        for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
     }
-    const int64_t clbase = (((int64_t)ul * p.na + ca) * b2 + cj) * p.r_pad + (int64_t)f * p.b1;
 
-    // staging tasks: (sh = 2*s + hf', dword column pc); 8 rows perm_row(s, hf', 0..7) each
+    // rows this lane stores in the epilogue: 2 rows, c = 16*it + lane/4 of the wave's 32 columns,
+    // 16 bytes (lane%4) of each 64-byte piece.  BYTE offsets from the (uniform) scratch row of (f, k).
+    uint32_t orow[2];                                     // ~0u = no row
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        int c = wave * 32 + it * 16 + (lane >> 2);
+        bool ok = c < ncols;
+        int aa = a0 + (ok ? c / b2 : 0);
+        int jj = ok ? c % b2 : 0;
+        uint32_t o = ((uint32_t)(aa * b2 + jj) * p.ws_aj * D + (lane & 3) * 8) * 2;
+        orow[it] = ok ? o : ~0u;
+    }
+    const uint32_t cloff = (uint32_t)(ca * b2 + cj) * p.ws_aj * 4;     // byte offset into cl, same convention
+    const uint32_t ubase = (uint32_t)ul * p.ws_unit + (uint32_t)k * p.ws_row;   // scratch row of (unit, k), f = 0
+    const uint32_t fstep = (uint32_t)p.b1 * p.ws_row;     // scratch rows between consecutive f
+
+    // staging tasks: (sh = 2*s + hf', dword column pc); 8 rows perm_row(s, hf', 0..7) each.  With
+    // D = 128 the 64 lanes of a wave share sh, which makes the row-validity tests scalar branches.
     constexpr int kTasks = 8 * DP;
     constexpr int kMaxTask = 2;                             // host launches >= kTasks/2 threads
     const int ntask = (kTasks + nthreads - 1) / nthreads;
+    if (ntask > kMaxTask) return;                           // (checked on the host as well)
     uint32_t pk[kMaxTask][8], pv[kMaxTask][8];
+    int tsh[kMaxTask];                                      // sh of the task, 8 = none
+    uint32_t tcol[kMaxTask];                                // byte offset of dword column pc
+#pragma unroll
+    for (int t = 0; t < kMaxTask; ++t) {
+        int task = tid + t * nthreads;
+        bool ok = t < ntask && task < kTasks;
+        int sh = ok ? task / DP : 8;
+        if (DP == 64) sh = __builtin_amdgcn_readfirstlane(sh);
+        tsh[t] = sh;
+        tcol[t] = (uint32_t)(task % DP) * 4;
+    }
 
-    auto prefetch = [&](int k) {
-        const int64_t krow0 = p.kmap.row(f, k);
+    auto prefetch = [&](int f) {
+        const uint32_t krow0 = (uint32_t)p.kmap.row(f, k);            // uniform
 #pragma unroll
         for (int t = 0; t < kMaxTask; ++t) {
-            int task = tid + t * nthreads;
-            if (t < ntask && task < kTasks) {
-                int pc = task % DP, sh = task / DP;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    int l = perm_row(sh >> 1, sh & 1, e);
-                    uint32_t kk = 0, vv = 0;
-                    if (l < b2) {
-                        kk = *(const uint32_t*)(kg + (krow0 + l) * p.ks[1] + 2 * pc);
-                        vv = *(const uint32_t*)(vg + (krow0 + l) * p.vs[1] + 2 * pc);
-                    }
-                    pk[t][e] = kk;
-                    pv[t][e] = vv;
+            for (int e = 0; e < 8; ++e) {
+                const int l = perm_row(tsh[t] >> 1, tsh[t] & 1, e);
+                uint32_t kk = 0, vv = 0;
+                if (tsh[t] < 8 && l < b2) {
+                    const size_t rowb = (size_t)((krow0 + (uint32_t)l) * ks1) * 2;
+                    kk = *(const uint32_t*)((const char*)kg + rowb + tcol[t]);
+                    vv = *(const uint32_t*)((const char*)vg + rowb + tcol[t]);
                 }
+                pk[t][e] = kk;
+                pv[t][e] = vv;
             }
         }
     };
     auto commit = [&]() {
 #pragma unroll
         for (int t = 0; t < kMaxTask; ++t) {
-            int task = tid + t * nthreads;
-            if (t < ntask && task < kTasks) {
-                int pc = task % DP, sh = task / DP;
+            if (tsh[t] < 8) {
+                const int pc = tcol[t] >> 2, sh = tsh[t];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     int l = perm_row(sh >> 1, sh & 1, e);
-                    *(uint32_t*)(lds + L::kKrow + l * L::kRowPitch + 2 * pc) = pk[t][e];
+                    *(uint32_t*)(lds_krow + l * L::kRowPitch + 2 * pc) = pk[t][e];
                 }
                 u32x4 lo, hi;
                 lo.x = lo16x2(pk[t][0], pk[t][1]); lo.y = lo16x2(pk[t][2], pk[t][3]);
                 lo.z = lo16x2(pk[t][4], pk[t][5]); lo.w = lo16x2(pk[t][6], pk[t][7]);
                 hi.x = hi16x2(pk[t][0], pk[t][1]); hi.y = hi16x2(pk[t][2], pk[t][3]);
                 hi.z = hi16x2(pk[t][4], pk[t][5]); hi.w = hi16x2(pk[t][6], pk[t][7]);
-                *(u32x4*)(lds + L::kKT + (2 * pc) * L::kTPitch + sh * 8) = lo;
-                *(u32x4*)(lds + L::kKT + (2 * pc + 1) * L::kTPitch + sh * 8) = hi;
+                *(u32x4*)(lds_kt + (2 * pc) * L::kTPitch + sh * 8) = lo;
+                *(u32x4*)(lds_kt + (2 * pc + 1) * L::kTPitch + sh * 8) = hi;
                 lo.x = lo16x2(pv[t][0], pv[t][1]); lo.y = lo16x2(pv[t][2], pv[t][3]);
                 lo.z = lo16x2(pv[t][4], pv[t][5]); lo.w = lo16x2(pv[t][6], pv[t][7]);
                 hi.x = hi16x2(pv[t][0], pv[t][1]); hi.y = hi16x2(pv[t][2], pv[t][3]);
                 hi.z = hi16x2(pv[t][4], pv[t][5]); hi.w = hi16x2(pv[t][6], pv[t][7]);
-                *(u32x4*)(lds + L::kVT + (2 * pc) * L::kTPitch + sh * 8) = lo;
-                *(u32x4*)(lds + L::kVT + (2 * pc + 1) * L::kTPitch + sh * 8) = hi;
+                *(u32x4*)(lds_vt + (2 * pc) * L::kTPitch + sh * 8) = lo;
+                *(u32x4*)(lds_vt + (2 * pc + 1) * L::kTPitch + sh * 8) = hi;
             }
         }
     };
 
-    uint16_t* stage = lds + L::kStage + wave * L::kStagePerWave;
     const float sc2 = p.scale * kLog2e;
 
-    if (ntask > kMaxTask) return;   // host launches enough threads (checked there)
-
-    prefetch(k0);
-    for (int k = k0; k < k1; ++k) {
-        __syncthreads();                 // previous iteration finished reading K/V tiles and the stage
-        commit();
-        if (k + 1 < k1) prefetch(k + 1);
-
-        // logits operand: this lane's query row Q[ca, k, cj, :]
-        u32x4 qb[DS];
-        {
-            const uint16_t* qrow = qg + (p.qmap.row(ca, k) + cj) * p.qs[1] + 8 * hf;
-#pragma unroll
-            for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
-        }
-        __syncthreads();                 // K/V tiles visible
+    const int G = p.s1_groups;
+    if (f0 + grp < f1) prefetch(f0 + grp);
+    for (int fb = f0; fb < f1; fb += G) {
+        const int f = fb + grp;
+        const bool has_f = f < f1;       // a group may run out of block-frames one round early; it still joins the barriers
+        lds_barrier();                   // previous iteration finished reading the tiles and the stages
+        if (has_f) commit();
+        if (f + G < f1) prefetch(f + G);
+        lds_barrier();                   // K/V tiles visible
 
         u32x4 pb[4];                     // R^T as B operands, 16 contraction rows per step
-        float inv_l = 0.f, cl2 = 0.f;
+        float inv_l = 0.f;
+        const bool tile_active = has_f && tile_ok;
         if (tile_active) {
             f32x16 s[2];
 #pragma unroll
@@ -182,7 +220,7 @@ __global__ __launch_bounds__(512) void monarch_step1_kernel(MonarchArgs p) {
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 if (t < NT) {
-                    const uint16_t* arow = lds + L::kKrow + (32 * t + m) * L::kRowPitch + 8 * hf;
+                    const uint16_t* arow = lds_krow + (32 * t + m) * L::kRowPitch + 8 * hf;
 #pragma unroll
                     for (int ds = 0; ds < DS; ++ds) {
                         u32x4 a = *(const u32x4*)(arow + 16 * ds);
@@ -197,9 +235,9 @@ __global__ __launch_bounds__(512) void monarch_step1_kernel(MonarchArgs p) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     int l = 32 * t + 8 * (v >> 2) + 4 * hf + (v & 3);
-                    float z = (t < NT && l < b2) ? s[t][v] * sc2 : -INFINITY;
-                    s[t][v] = z;
-                    mx = fmaxf(mx, z);
+                    float zz = (t < NT && l < b2) ? s[t][v] * sc2 : kMaskLogit;
+                    s[t][v] = zz;
+                    mx = fmaxf(mx, zz);
                 }
             mx = xhalf_max(mx);
             float sum = 0.f, ent = 0.f;
@@ -207,73 +245,66 @@ __global__ __launch_bounds__(512) void monarch_step1_kernel(MonarchArgs p) {
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    float z = s[t][v];
-                    float e = exp2f(z - mx);           // exp2(-inf) = 0 for masked rows
+                    float zz = s[t][v];
+                    float e = fast_exp2(zz - mx);        // exactly 0 for masked rows
                     sum += e;
-                    ent += (z == -INFINITY) ? 0.f : e * z;
+                    ent += e * zz;
                     s[t][v] = e;
                 }
             sum = xhalf_sum(sum);
             ent = xhalf_sum(ent);
             inv_l = 1.f / sum;
-            cl2 = ent * inv_l - (mx + log2f(sum));      // sum_l R log2 R
+            // R = e / sum is rounded to 16 bit once, as the reference's right factor is
 #pragma unroll
             for (int st = 0; st < 4; ++st) {
                 const int t = st >> 1, v0 = 8 * (st & 1);
-                pb[st].x = pack2<E>(s[t][v0 + 0], s[t][v0 + 1]);
-                pb[st].y = pack2<E>(s[t][v0 + 2], s[t][v0 + 3]);
-                pb[st].z = pack2<E>(s[t][v0 + 4], s[t][v0 + 5]);
-                pb[st].w = pack2<E>(s[t][v0 + 6], s[t][v0 + 7]);
+                pb[st].x = pack2<E>(s[t][v0 + 0] * inv_l, s[t][v0 + 1] * inv_l);
+                pb[st].y = pack2<E>(s[t][v0 + 2] * inv_l, s[t][v0 + 3] * inv_l);
+                pb[st].z = pack2<E>(s[t][v0 + 4] * inv_l, s[t][v0 + 5] * inv_l);
+                pb[st].w = pack2<E>(s[t][v0 + 6] * inv_l, s[t][v0 + 7] * inv_l);
             }
-            if (col_ok && hf == 0) p.cl[clbase + k] = cl2;
+            if (col_ok && hf == 0)                 // sum_l R log2 R
+                *(float*)((char*)p.cl + (size_t)(ubase + (uint32_t)f * fstep) * 4 + cloff) = ent * inv_l - (mx + log2f(sum));
         }
+        lds_barrier();                   // every wave has its logits: the row-major K tile may be overwritten
 
-        // contractions with K^T then V^T; each goes out through the wave's LDS stage in two
-        // halves of the head dim (64 columns at a time)
+        // contractions with K^T then V^T, 32 head-dim columns at a time; each 32 x 32 piece goes out
+        // through the wave's LDS stage so that a row's 64 bytes are stored by 4 adjacent lanes
 #pragma unroll
         for (int which = 0; which < 2; ++which) {
-            const uint16_t* tbase = lds + (which == 0 ? L::kKT : L::kVT);
-            uint16_t* og = (uint16_t*)(which == 0 ? p.kbar : p.y);
-            f32x16 acc[DT];
-            if (tile_active) {
+            const uint16_t* tbase = which == 0 ? lds_kt : lds_vt;
+            char* og = (char*)(which == 0 ? p.kbar : p.y) + (size_t)(ubase + (uint32_t)f * fstep) * (D * 2);
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
+            for (int dt = 0; dt < D / 32; ++dt) {
+                if (tile_active) {
+                    f32x16 acc;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
+                    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
                     const uint16_t* arow = tbase + (32 * dt + m) * L::kTPitch + 8 * hf;
 #pragma unroll
                     for (int st = 0; st < 4; ++st) {
                         if (st < 2 * NT) {
                             u32x4 a = *(const u32x4*)(arow + 16 * st);
-                            acc[dt] = E::mfma32(a, pb[st], acc[dt]);
+                            acc = E::mfma32(a, pb[st], acc);
                         }
                     }
-                }
-            }
 #pragma unroll
-            for (int hd = 0; hd < D / 64; ++hd) {
-                if (tile_active) {
-#pragma unroll
-                    for (int t2 = 0; t2 < 2; ++t2) {
-                        const int dt = 2 * hd + t2;
-#pragma unroll
-                        for (int g = 0; g < 4; ++g) {
-                            u32x2 w;
-                            w.x = pack2<E>(acc[dt][4 * g + 0] * inv_l, acc[dt][4 * g + 1] * inv_l);
-                            w.y = pack2<E>(acc[dt][4 * g + 2] * inv_l, acc[dt][4 * g + 3] * inv_l);
-                            *(u32x2*)(stage + m * L::kStagePitch + 32 * t2 + 8 * g + 4 * hf) = w;
-                        }
+                    for (int g = 0; g < 4; ++g) {
+                        u32x2 w;
+                        w.x = pack2<E>(acc[4 * g + 0], acc[4 * g + 1]);
+                        w.y = pack2<E>(acc[4 * g + 2], acc[4 * g + 3]);
+                        *(u32x2*)(stage + m * L::kStagePitch + 8 * g + 4 * hf) = w;
                     }
                 }
-                __syncthreads();
+                lds_wave_sync();             // the stage is private to the wave
                 if (tile_active) {
 #pragma unroll
-                    for (int it = 0; it < 4; ++it) {
-                        u32x4 w = *(const u32x4*)(stage + (it * 8 + (lane >> 3)) * L::kStagePitch + (lane & 7) * 8);
-                        if (orow_ok[it]) *(u32x4*)(og + orow[it] + (int64_t)k * D + 64 * hd) = w;
+                    for (int it = 0; it < 2; ++it) {
+                        u32x4 w = *(const u32x4*)(stage + (it * 16 + (lane >> 2)) * L::kStagePitch + (lane & 3) * 8);
+                        if (orow[it] != ~0u) *(u32x4*)(og + orow[it] + 64 * dt) = w;
                     }
                 }
-                __syncthreads();
+                lds_wave_sync();
             }
         }
     }
@@ -317,10 +348,11 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
     const int r_lim = f_lim * p.b1;
     const int nch = (r_lim + 31) / 32;
 
-    const int64_t blk = (((int64_t)ul * p.na + a) * b2 + j) * p.r_pad;
+    const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj;   // in rows
     const uint16_t* kb = (const uint16_t*)p.kbar + blk * D;
     const uint16_t* yb = (const uint16_t*)p.y + blk * D;
     const float* clp = p.cl + blk;
+    constexpr uint32_t rstride = D;                 // rows of one (a, j) are consecutive (ws_row == 1)
 
     uint16_t* wl = lds + wave * L::kPerWave;
 
@@ -353,7 +385,7 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
     uint32_t ycur[2][DPn][8];
 
     auto load_k = [&](int n) {
-        const uint16_t* row = kb + (int64_t)(32 * n + m) * D + 8 * hf;
+        const uint16_t* row = kb + (uint32_t)(32 * n + m) * rstride + 8 * hf;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) kcur[ds] = *(const u32x4*)(row + 16 * ds);
     };
@@ -367,7 +399,7 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 int r = 32 * n + perm_row(st, hf, e);
-                const uint16_t* row = yb + (int64_t)r * D + 2 * m;
+                const uint16_t* row = yb + (uint32_t)r * rstride + 2 * m;
 #pragma unroll
                 for (int dp = 0; dp < DPn; ++dp) {
                     uint32_t w = *(const uint32_t*)(row + 64 * dp);
@@ -487,12 +519,13 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const 
     const int ncols = a.a_chunk * a.b2;
     const int ntiles = (ncols + 31) / 32;
     const int nwaves = ntiles < 4 ? 4 : ntiles;   // at least 4 waves so that K/V staging is <= 2 tasks per thread
-    const int kgroups = (a.b1 + a.k_per_wg - 1) / a.k_per_wg;
+    const int nfs = (a.nf + a.f_per_wg - 1) / a.f_per_wg;
     if (ntiles < 1 || nwaves > 8 || (8 * (D / 2) + nwaves * 64 - 1) / (nwaves * 64) > 2) {
         set_error("internal: step-1 launch shape (a_chunk=%d, b2=%d)", a.a_chunk, a.b2);
         return SFM_ERR_UNSUPPORTED;
     }
-    const size_t lds1 = S1Lds<D>::bytes(nwaves);
+    const int groups = nwaves <= 5 ? 2 : 1;             // wave groups per workgroup (<= 10 waves in all)
+    const size_t lds1 = S1Lds<D>::bytes(nwaves) * groups;
     if (lds1 > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)monarch_step1_kernel<E, D>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1);
@@ -501,9 +534,12 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const 
             return SFM_ERR_HIP;
         }
     }
-    dim3 g1(kgroups, a.nf, nunits * a.n_achunks);
+    MonarchArgs a1 = a;
+    a1.s1_total = nfs * a.b1 * nunits * a.n_achunks;
+    a1.s1_groups = groups;
+    dim3 g1((a1.s1_total + 7) / 8 * 8);
     if (ev) (void)hipEventRecord(ev->ev[0], stream);
-    hipLaunchKernelGGL((monarch_step1_kernel<E, D>), g1, dim3(nwaves * 64), lds1, stream, a);
+    hipLaunchKernelGGL((monarch_step1_kernel<E, D>), g1, dim3(nwaves * 64 * groups), lds1, stream, a1);
     if (ev) (void)hipEventRecord(ev->ev[1], stream);
     const int njg = (a.b2 + 3) / 4;
     dim3 g2(a.na * njg, nunits, (a.b1 + 31) / 32);

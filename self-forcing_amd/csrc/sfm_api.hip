@@ -1,6 +1,7 @@
 // extern "C" entry points: argument validation, workspace accounting, pass scheduling.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "sfm_common.hpp"
@@ -63,8 +64,12 @@ static int check_strides(const char* name, const int64_t s[3], int64_t tokens, i
                   (long long)s[2], H, D);
         return SFM_ERR_STRIDE;
     }
-    (void)tokens;
     (void)B;
+    // kernels address a (batch, head) slice with 32-bit element offsets
+    if ((tokens + 1) * s[1] >= ((int64_t)1 << 31)) {
+        set_error("%s: tokens * token-stride must stay below 2^31 elements", name);
+        return SFM_ERR_STRIDE;
+    }
     if ((s[0] * esz) % 16 || (s[1] * esz) % 16 || (s[2] * esz) % 16) {
         set_error("%s: strides must be multiples of 16 bytes", name);
         return SFM_ERR_STRIDE;
@@ -141,10 +146,10 @@ static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
     return SFM_OK;
 }
 
-// Default number of units per pass: keep the scratch of one pass well inside the 256 MB
-// last-level cache so that step 2 finds step 1's rows there.
+// Default number of units per pass: all of them while the scratch stays under 4 GiB (one launch pair
+// fills the chip best; smaller passes only pay when the scratch would not fit).
 static int default_units_per_pass(const MonarchPlan& pl) {
-    const size_t budget = (size_t)112 << 20;
+    const size_t budget = (size_t)3 << 30;        // keeps 32-bit element offsets into each scratch matrix
     size_t n = budget / pl.per_unit;
     if (n < 1) n = 1;
     if (n > (size_t)pl.units) n = pl.units;
@@ -196,6 +201,11 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
         return SFM_ERR_WORKSPACE;
     }
     size_t upp_sz = workspace_bytes / pl.per_unit;
+    if (upp_sz * pl.per_unit > ((size_t)3 << 30)) upp_sz = ((size_t)3 << 30) / pl.per_unit;   // 32-bit offsets
+    if (upp_sz < 1) {
+        set_error("one (batch, head) unit needs %zu bytes of scratch, more than the 3 GiB a pass may use", pl.per_unit);
+        return SFM_ERR_UNSUPPORTED;
+    }
     const int upp = upp_sz > (size_t)pl.units ? pl.units : (int)upp_sz;
 
     MonarchArgs a;
@@ -213,13 +223,22 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
     }
     const size_t rows = (size_t)pl.na * pl.b2 * pl.r_pad;
     const size_t mat_bytes = rows * desc->D * (pl.mfma ? 2 : 4);
+    a.ws_unit = (uint32_t)rows;
+    // (a, j)-major scratch: the rows one step-2 wave streams are consecutive.  (An r-major layout, in
+    // which the rows a step-1 workgroup writes are consecutive instead, measured the same for step 1.)
+    a.ws_aj = (uint32_t)pl.r_pad;
+    a.ws_row = 1;
     // step 1 takes as many query block-frames per workgroup as fit 256 (a, j) columns
     int a_max = 256 / pl.b2;
     if (a_max < 1) a_max = 1;
     a.n_achunks = (pl.na + a_max - 1) / a_max;
     a.a_chunk = (pl.na + a.n_achunks - 1) / a.n_achunks;
     a.n_achunks = (pl.na + a.a_chunk - 1) / a.a_chunk;
-    a.k_per_wg = pl.b1 < 6 ? pl.b1 : 6;
+    a.f_per_wg = pl.nf < 7 ? pl.nf : 7;
+    if (const char* e = getenv("SFM_F_PER_WG")) {          // tuning override: kv block-frames per step-1 workgroup
+        int v = atoi(e);
+        if (v >= 1) a.f_per_wg = v < pl.nf ? v : pl.nf;
+    }
     for (int u0 = 0; u0 < pl.units; u0 += upp) {
         const int n = pl.units - u0 < upp ? pl.units - u0 : upp;
         a.unit0 = u0;

@@ -14,6 +14,9 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -34,6 +37,11 @@ struct BF16 {
         __bf16 b = (__bf16)f;
         return __builtin_bit_cast(uint16_t, b);
     }
+    // two floats -> one dword of two round-to-nearest-even elements (a single packed convert)
+    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+        f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+    }
     static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
     }
@@ -46,6 +54,10 @@ struct F16 {
         _Float16 b = (_Float16)f;
         return __builtin_bit_cast(uint16_t, b);
     }
+    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+        f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+    }
     static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
     }
@@ -53,15 +65,30 @@ struct F16 {
 
 template <class E>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
-    return (uint32_t)E::from_float(lo) | ((uint32_t)E::from_float(hi) << 16);
+    return E::pack(lo, hi);
 }
 
 // low / high 16-bit halves of two dwords -> one dword
 __device__ __forceinline__ uint32_t lo16x2(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }
 __device__ __forceinline__ uint32_t hi16x2(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
 
+// v_exp_f32 without the denormal-range fix-up of exp2f(): arguments here are <= 0 and results that
+// underflow may flush to zero.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Logit value given to masked positions: finite, so that 0 * mask stays 0 in entropy sums, and far
+// enough below any real logit that exp2(mask - max) underflows to exactly 0.
+constexpr float kMaskLogit = -1.0e30f;
+
 __device__ __forceinline__ float xhalf_max(float x) { return fmaxf(x, __shfl_xor(x, 32)); }
 __device__ __forceinline__ float xhalf_sum(float x) { return x + __shfl_xor(x, 32); }
+
+// Workgroup barrier that orders LDS traffic only: waits for this wave's LDS operations, then s_barrier.
+// Unlike __syncthreads() it does not drain outstanding global loads/stores, so register prefetches and
+// streaming stores stay in flight across it.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// Orders a wave's own LDS writes before its later LDS reads (wave-private staging buffers).
+__device__ __forceinline__ void lds_wave_sync() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
 // Row of the 16x16-dword-permuted contraction index used when a D tile (rows = contraction
 // index) is fed back as a B operand: element e of lane-half hf in 16-wide step s.
@@ -87,6 +114,12 @@ struct TokMap {
         int ii = i - ft * hh;
         return ((int64_t)(A * f_tied + ft) * h + (c * hh + ii)) * w + e * ww;
     }
+    // row(bf, i) - row(bf, 0): the same for every block-frame
+    __host__ __device__ __forceinline__ int row_delta(int i) const {
+        if (!natural) return i * b2;
+        int ft = i / hh;
+        return (ft * h + (i - ft * hh)) * w;
+    }
 };
 
 struct MonarchArgs {
@@ -99,6 +132,8 @@ struct MonarchArgs {
     float* cl;       // [units_per_pass][na][b2][r_pad]      sum_l R log2 R  (log2 units)
     int B, H, D, na, nf, b1, b2;
     int r_pad;       // rows per (a, j) block of the workspace: round_up(nf*b1, 32)
+    // scratch row index of (unit ul, a, j, r) = ul*ws_unit + (a*b2 + j)*ws_aj + r*ws_row
+    uint32_t ws_unit, ws_aj, ws_row;
     int unit0;       // first (b*H + h) unit of this pass
     int causal;      // block-causal size in block-frames, 0 = none
     float scale;
@@ -106,7 +141,9 @@ struct MonarchArgs {
     int64_t qs[3], ks[3], vs[3], os[3];
     int a_chunk;     // query block-frames per step-1 workgroup
     int n_achunks;
-    int k_per_wg;    // block rows per step-1 workgroup
+    int f_per_wg;    // kv block-frames per step-1 workgroup
+    int s1_groups;   // wave groups per step-1 workgroup
+    int s1_total;    // step-1 workgroups that have work (the grid is padded to a multiple of 8)
 };
 
 // Optional timing hooks: ev[0] is recorded before step 1, ev[1] between the steps, ev[2] after step 2.
