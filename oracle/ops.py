@@ -1,0 +1,37 @@
+"""Oracle (test infrastructure): attention operators for causal_model built on the CPU oracle: lets a test run the
+product's own module code with reference attention, on the CPU, to compare against the HIP run."""
+import torch
+
+from oracle import blocks, dense, monarch, prologue
+
+
+class OracleOps:
+    def __init__(self, compute_dtype=torch.float32):
+        self.compute_dtype = compute_dtype
+        self.calls = []
+
+    def rope_table(self, head_dim, device):
+        return None
+
+    def qk_prologue(self, xq, xk, xv, wq, wk, num_heads, grid, start_frame, rope, k_cache, v_cache, start_idx,
+                    f_tied=1, h_reduce=1, w_reduce=1, eps=1e-6):
+        q, k, v = prologue.qk_prologue(xq, xk, xv, wq, wk, num_heads, grid, start_frame, eps)
+        B, S, H, D = q.shape
+        _, h, w = grid
+        k_cache[:, start_idx:start_idx + S] = blocks.to_blocks(k, f_tied, h_reduce, w_reduce, h, w).reshape(B, S, H, D)
+        v_cache[:, start_idx:start_idx + S] = blocks.to_blocks(v, f_tied, h_reduce, w_reduce, h, w).reshape(B, S, H, D)
+        self.calls.append(("prologue", start_frame, start_idx, (f_tied, h_reduce, w_reduce)))
+        return q
+
+    def monarch_cached(self, q, k_view, v_view, f_tied, h_reduce, w_reduce, h, w):
+        B, _, H, D = q.shape
+        qb = blocks.to_blocks(q, f_tied, h_reduce, w_reduce, h, w)
+        b1, b2 = qb.shape[2], qb.shape[3]
+        out = monarch.monarch_1iter(qb, k_view.reshape(B, -1, b1, b2, H, D), v_view.reshape(B, -1, b1, b2, H, D),
+                                    D ** -0.5, dtype=self.compute_dtype)
+        self.calls.append(("monarch", k_view.shape[1]))
+        return blocks.from_blocks(out, f_tied, h_reduce, w_reduce, h, w).to(q.dtype)
+
+    def dense(self, q, k, v):
+        self.calls.append(("dense", k.shape[1]))
+        return dense.attention(q, k, v, dtype=self.compute_dtype).to(q.dtype)

@@ -7,7 +7,8 @@ reference's module names:
     monarch_attn.monarch_attn_with_kv_cache / monarch_attn.monarch_attn
     attention.attention / attention.full_attention_with_kv_cache
     prologue.qk_prologue / prologue.rope_table
+    causal_model.CausalWanModel (+ self-attention, block, head), pipeline.CausalInferencePipeline
 """
-from . import lib, monarch_attn, attention, prologue  # noqa: F401
+from . import lib, monarch_attn, attention, prologue, causal_model, pipeline  # noqa: F401
 
-__all__ = ["lib", "monarch_attn", "attention", "prologue"]
+__all__ = ["lib", "monarch_attn", "attention", "prologue", "causal_model", "pipeline"]

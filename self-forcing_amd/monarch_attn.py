@@ -88,9 +88,11 @@ def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end
 
 
 def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block_causal_size=None, num_iters=1,
-                 heads_per_pass=0):
-    """One-iteration Monarch attention without a cache; `block_causal_size` (tokens) masks
-    block-frames of later causal blocks."""
+                 heads_per_pass=0, kv_block_order=False):
+    """One-iteration Monarch attention without a cache write; `block_causal_size` (tokens) masks
+    block-frames of later causal blocks.  `kv_block_order=True` (no counterpart in the reference) says
+    that k, v are a KV-cache view whose rows are already in Monarch block order, e.g. after
+    prologue.qk_prologue wrote them."""
     if num_iters != 1:
         raise NotImplementedError("num_iters > 1 (the reference's pure-torch refinement) is not built")
     if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
@@ -113,7 +115,7 @@ def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block
             raise ValueError("block_causal_size must align with Monarch block sizes")
         cbf = block_causal_size // per_block
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    d = _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 0, cbf)
+    d = _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1 if kv_block_order else 0, cbf)
     nbytes = monarch_workspace_bytes(d, heads_per_pass)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):

@@ -1,0 +1,191 @@
+"""Few-step autoregressive rollout around the causal DiT: scheduler, x0 conversion, KV-cache ownership.
+
+Counterpart of
+    FlowMatchScheduler            utils/scheduler.py:106-176
+    WanDiffusionWrapper           utils/wan_wrapper.py:117-143, 172-196, 221-292
+    CausalInferencePipeline       pipeline/causal_inference.py:13-50, 51-322
+Text encoder and VAE are outside this build: `inference` takes prompt embeddings and returns latents.
+"""
+import time
+
+import torch
+import torch.nn as nn
+
+from .causal_model import FRAME_HEIGHT, FRAME_WIDTH, CausalWanModel
+
+
+class FlowMatchScheduler:
+    """sigma ladder with shift; float32 like the reference's torch.linspace tables."""
+
+    def __init__(self, num_inference_steps=1000, num_train_timesteps=1000, shift=5.0, sigma_max=1.0, sigma_min=0.0,
+                 extra_one_step=True):
+        self.num_train_timesteps, self.shift = num_train_timesteps, shift
+        self.sigma_max, self.sigma_min, self.extra_one_step = sigma_max, sigma_min, extra_one_step
+        self.set_timesteps(num_inference_steps)
+
+    def set_timesteps(self, num_inference_steps):
+        if self.extra_one_step:
+            sig = torch.linspace(self.sigma_max, self.sigma_min, num_inference_steps + 1)[:-1]
+        else:
+            sig = torch.linspace(self.sigma_max, self.sigma_min, num_inference_steps)
+        self.sigmas = self.shift * sig / (1 + (self.shift - 1) * sig)
+        self.timesteps = self.sigmas * self.num_train_timesteps
+
+    def _sigma(self, timestep, device):
+        self.sigmas, self.timesteps = self.sigmas.to(device), self.timesteps.to(device)
+        idx = torch.argmin((self.timesteps.unsqueeze(0) - timestep.unsqueeze(1)).abs(), dim=1)
+        return self.sigmas[idx].reshape(-1, 1, 1, 1)
+
+    def add_noise(self, original_samples, noise, timestep):
+        """(1 - sigma_t) x0 + sigma_t noise on [B*T, C, H, W] with timestep [B*T]."""
+        sigma = self._sigma(timestep.flatten(), noise.device)
+        return ((1 - sigma) * original_samples + sigma * noise).type_as(noise)
+
+
+class WanDiffusionWrapper(nn.Module):
+    """Wraps the DiT: latents [B, F, C, H, W] in, (flow_pred, x0_pred) out."""
+
+    def __init__(self, model, timestep_shift=5.0):
+        super().__init__()
+        self.model = model
+        self.scheduler = FlowMatchScheduler(shift=timestep_shift, sigma_min=0.0, extra_one_step=True)
+
+    def get_scheduler(self):
+        return self.scheduler
+
+    def _convert_flow_pred_to_x0(self, flow_pred, xt, timestep):
+        """x0 = x_t - sigma_t * flow in float64 (wan_wrapper.py:172-196)."""
+        dt = flow_pred.dtype
+        sig = self.scheduler.sigmas.double().to(flow_pred.device)
+        ts = self.scheduler.timesteps.double().to(flow_pred.device)
+        idx = torch.argmin((ts.unsqueeze(0) - timestep.double().unsqueeze(1)).abs(), dim=1)
+        return (xt.double() - sig[idx].reshape(-1, 1, 1, 1) * flow_pred.double()).to(dt)
+
+    @torch.no_grad()
+    def forward(self, noisy_image_or_video, conditional_dict, timestep, kv_cache=None, crossattn_cache=None,
+                current_start=None):
+        flow = self.model(noisy_image_or_video.permute(0, 2, 1, 3, 4), t=timestep,
+                          context=conditional_dict["prompt_embeds"], kv_cache=kv_cache,
+                          crossattn_cache=crossattn_cache, current_start=current_start).permute(0, 2, 1, 3, 4)
+        x0 = self._convert_flow_pred_to_x0(flow.flatten(0, 1), noisy_image_or_video.flatten(0, 1),
+                                           timestep.flatten(0, 1)).unflatten(0, flow.shape[:2])
+        return flow, x0
+
+
+class CausalInferencePipeline(nn.Module):
+    """Chunk loop x denoising loop with per-layer KV caches (pipeline/causal_inference.py:182-254).
+
+    denoising_step_list (1000, 750, 500, 250) is warped through the shifted sigma table when
+    warp_denoising_step is set (`:33-35`); after the last step of a chunk the clean chunk is run once more
+    at t = context_noise so that the cache holds K/V of the clean frames (`:236-245`).  The reference draws
+    the re-noising randoms from a hard-coded seed list for eval consistency; here `seeds` is a parameter
+    (any iterable of ints, cycled) and defaults to 0, 1, 2, ..."""
+
+    def __init__(self, generator, denoising_step_list=(1000, 750, 500, 250), warp_denoising_step=True,
+                 num_frame_per_block=3, context_noise=0, local_attn_size=-1, frame_hw=(FRAME_HEIGHT, FRAME_WIDTH),
+                 num_cache_frames=21, seeds=None):
+        super().__init__()
+        self.generator = generator
+        self.scheduler = generator.get_scheduler()
+        steps = torch.tensor(denoising_step_list, dtype=torch.long)
+        if warp_denoising_step:
+            ts = torch.cat((self.scheduler.timesteps.cpu(), torch.tensor([0], dtype=torch.float32)))
+            steps = ts[1000 - steps]
+        self.denoising_step_list = steps
+        self.num_frame_per_block = num_frame_per_block
+        self.context_noise = context_noise
+        self.local_attn_size = local_attn_size
+        self.frame_seq_length = frame_hw[0] * frame_hw[1]
+        self.num_cache_frames = num_cache_frames
+        self.kv_cache1 = None
+        self.crossattn_cache = None
+        self.seeds = list(seeds) if seeds is not None else None
+        self._seed_count = 0
+        self.last_chunk_ms = []
+
+    def _initialize_kv_cache(self, batch_size, dtype, device):
+        m = self.generator.model
+        frames = self.local_attn_size if self.local_attn_size != -1 else self.num_cache_frames
+        size = frames * self.frame_seq_length
+        self.kv_cache1 = [{
+            "k": torch.zeros([batch_size, size, m.num_heads, m.dim // m.num_heads], dtype=dtype, device=device),
+            "v": torch.zeros([batch_size, size, m.num_heads, m.dim // m.num_heads], dtype=dtype, device=device),
+            "global_end_index": torch.tensor([0], dtype=torch.long, device=device),
+            "local_end_index": torch.tensor([0], dtype=torch.long, device=device),
+            "_global_end": 0, "_local_end": 0,
+        } for _ in range(m.num_layers)]
+
+    def _initialize_crossattn_cache(self):
+        self.crossattn_cache = [{"k": None, "v": None, "is_init": False} for _ in range(self.generator.model.num_layers)]
+
+    def _reset_caches(self, device):
+        for c in self.crossattn_cache:
+            c["is_init"] = False
+        for c in self.kv_cache1:       # only the counters are reset, not the K/V storage (`:129-138`)
+            c["global_end_index"] = torch.tensor([0], dtype=torch.long, device=device)
+            c["local_end_index"] = torch.tensor([0], dtype=torch.long, device=device)
+            c["_global_end"] = c["_local_end"] = 0
+
+    def _next_seed(self):
+        if self.seeds is None:
+            s = self._seed_count
+        else:
+            s = self.seeds[self._seed_count % len(self.seeds)]
+        self._seed_count += 1
+        return s
+
+    @torch.no_grad()
+    def inference(self, noise, prompt_embeds, profile=False):
+        """noise [B, F, C, H, W]; prompt_embeds [B, L_text, text_dim].  Returns latents [B, F, C, H, W]."""
+        B, num_frames, C, H, W = noise.shape
+        assert num_frames % self.num_frame_per_block == 0
+        num_blocks = num_frames // self.num_frame_per_block
+        cond = {"prompt_embeds": prompt_embeds}
+        output = torch.zeros_like(noise)
+        if self.kv_cache1 is None or self.kv_cache1[0]["k"].shape[0] != B:
+            self._initialize_kv_cache(B, noise.dtype, noise.device)
+            self._initialize_crossattn_cache()
+        else:
+            self._reset_caches(noise.device)
+        self.last_chunk_ms = []
+        start_frame = 0
+        for _ in range(num_blocks):
+            nf = self.num_frame_per_block
+            if profile:
+                torch.cuda.synchronize(noise.device)
+                t0 = time.perf_counter()
+            noisy = noise[:, start_frame:start_frame + nf]
+            cur = start_frame * self.frame_seq_length
+            for index, cur_t in enumerate(self.denoising_step_list):
+                timestep = torch.ones([B, nf], device=noise.device, dtype=torch.int64) * cur_t
+                _, denoised = self.generator(noisy, cond, timestep, self.kv_cache1, self.crossattn_cache, cur)
+                if index < len(self.denoising_step_list) - 1:
+                    next_t = self.denoising_step_list[index + 1]
+                    # drawn on the host so that the same seeds give the same video on any device
+                    g = torch.Generator().manual_seed(self._next_seed())
+                    flat = denoised.flatten(0, 1)
+                    eps = torch.randn(flat.shape, generator=g, dtype=torch.float32).to(flat.device, flat.dtype)
+                    noisy = self.scheduler.add_noise(
+                        flat, eps, next_t * torch.ones([B * nf], device=noise.device, dtype=torch.long)
+                    ).unflatten(0, denoised.shape[:2])
+            output[:, start_frame:start_frame + nf] = denoised
+            ctx_t = torch.ones([B, nf], device=noise.device, dtype=torch.int64) * self.context_noise
+            self.generator(denoised, cond, ctx_t, self.kv_cache1, self.crossattn_cache, cur)
+            if profile:
+                torch.cuda.synchronize(noise.device)
+                self.last_chunk_ms.append((time.perf_counter() - t0) * 1e3)
+            start_frame += nf
+        return output
+
+
+def build_generator(size="1.3B", dtype=torch.bfloat16, device="cuda:0", seed=0, zero_head=False, timestep_shift=5.0,
+                    **model_overrides):
+    """Random-init causal Wan generator of a named size (reference init, optionally with a non-zero head)."""
+    from .causal_model import WAN_CONFIGS
+    cfg = dict(WAN_CONFIGS[size]) if size in WAN_CONFIGS else {}
+    cfg.update(model_overrides)
+    torch.manual_seed(seed)
+    model = CausalWanModel(**cfg)
+    model.init_weights(zero_head=zero_head)
+    model = model.to(dtype=dtype, device=device).eval()
+    return WanDiffusionWrapper(model, timestep_shift=timestep_shift)

@@ -1,0 +1,115 @@
+"""Host logic of the causal DiT and the rollout pipeline, run on the CPU with oracle attention operators:
+cache index state machine, dispatch flags, shapes, scheduler, determinism."""
+import numpy as np
+import pytest
+import torch
+
+import self_forcing_amd as sfa
+from oracle import cache as ocache, sched as osched
+from oracle.ops import OracleOps
+
+cm, pl = sfa.causal_model, sfa.pipeline
+TINY = dict(dim=64, ffn_dim=128, num_heads=2, num_layers=2, text_dim=32, text_len=8, frame_hw=(2, 3), total_seq_len=6 * 6)
+
+
+def _tiny(ops, seed=0, **flags):
+    torch.manual_seed(seed)
+    m = cm.CausalWanModel(ops=ops, attention_flags=flags, **TINY)
+    m.init_weights(zero_head=False)
+    return pl.WanDiffusionWrapper(m.float().eval())
+
+
+def test_scheduler_matches_closed_form():
+    s = pl.FlowMatchScheduler(shift=5.0)
+    sig, ts = osched.sigma_table(shift=5.0)
+    assert np.allclose(s.sigmas.numpy(), sig, atol=1e-6) and np.allclose(s.timesteps.numpy(), ts, atol=1e-3)
+    x0, eps = torch.randn(2, 3, 4, 4), torch.randn(2, 3, 4, 4)
+    t = torch.tensor([625.0, 1000.0])
+    got = s.add_noise(x0, eps, t)
+    for i, tt in enumerate((625.0, 1000.0)):
+        sg = osched.sigma_of(tt)
+        assert torch.allclose(got[i], (1 - sg) * x0[i] + sg * eps[i], atol=1e-5)
+
+
+def test_flow_to_x0_conversion():
+    gen = _tiny(OracleOps())
+    flow, xt = torch.randn(3, 16, 4, 6), torch.randn(3, 16, 4, 6)
+    t = torch.tensor([1000.0, 937.5, 625.0])
+    x0 = gen._convert_flow_pred_to_x0(flow, xt, t)
+    for i, tt in enumerate(t.tolist()):
+        assert torch.allclose(x0[i], xt[i] - osched.sigma_of(tt) * flow[i], atol=1e-5)
+
+
+def test_cache_step_matches_oracle_state_machine():
+    for local_attn, sink, max_attn in ((-1, 0, 36), (4, 1, 24), (3, 0, 18)):
+        cache_len = 36 if local_attn == -1 else local_attn * 6
+        kv = {"k": torch.zeros(1, cache_len, 1, 8), "global_end_index": torch.tensor([0]), "local_end_index": torch.tensor([0])}
+        st = ocache.KVCacheState(cache_len, max_attn, 6, local_attn, sink)
+        for cur in (0, 0, 12, 12, 24, 24, 24):
+            roll, cs, ls, le, ce = cm.cache_step(kv, cur, 12, 6, local_attn, sink, max_attn)
+            cm.cache_commit(kv, ce, le)
+            o = st.step(cur, 12)
+            assert roll == (o.roll_src, o.roll_dst, o.roll_len) or (roll[2] == 0 and o.roll_len == 0)
+            assert (cs, ls, le) == (o.cache_start, o.write_start, o.write_end)
+            assert int(kv["global_end_index"]) == st.global_end and int(kv["local_end_index"]) == st.local_end
+
+
+def test_pipeline_rollout_dispatch_and_cache_trace():
+    ops = OracleOps()
+    gen = _tiny(ops, use_framewise=True)
+    pipe = pl.CausalInferencePipeline(gen, frame_hw=(2, 3), num_cache_frames=6)
+    noise = torch.randn(1, 6, 16, 4, 6)
+    ctx = torch.randn(1, 5, 32)
+    out = pipe.inference(noise, ctx)
+    assert out.shape == noise.shape and torch.isfinite(out).all() and out.abs().sum() > 0
+    assert [round(float(t), 2) for t in pipe.denoising_step_list] == [1000.0, 937.5, 833.33, 625.0]
+    # 2 chunks x (4 + 1) passes x 2 layers, Monarch over 3 then 6 cached frames
+    mon = [c for c in ops.calls if c[0] == "monarch"]
+    assert len(mon) == 20 and [c[1] for c in mon] == [18] * 10 + [36] * 10
+    pro = [c for c in ops.calls if c[0] == "prologue"]
+    assert [c[1] for c in pro] == [0] * 10 + [3] * 10 and [c[2] for c in pro] == [0] * 10 + [18] * 10
+    # cross-attention K/V computed once per layer, then served from the cache
+    assert all(c["is_init"] for c in pipe.crossattn_cache)
+    assert sum(1 for c in ops.calls if c[0] == "dense") == 20
+    assert pipe.kv_cache1[0]["_global_end"] == 36 and int(pipe.kv_cache1[0]["local_end_index"]) == 36
+    # a second video resets the counters and gives the same result with the same seeds
+    pipe._seed_count = 0
+    out2 = pipe.inference(noise, ctx)
+    assert torch.equal(out, out2)
+
+
+def test_dense_init_and_disable_flags():
+    ops = OracleOps()
+    pipe = pl.CausalInferencePipeline(_tiny(ops, use_framewise=True, use_dense_init=True), frame_hw=(2, 3), num_cache_frames=6)
+    pipe.inference(torch.randn(1, 6, 16, 4, 6), torch.randn(1, 5, 32))
+    kinds = [c[0] for c in ops.calls if c[0] in ("monarch",) or (c[0] == "dense" and c[1] != 8)]
+    assert kinds == ["dense"] * 10 + ["monarch"] * 10          # first chunk (3 cached frames) runs dense
+    assert [c[3] for c in ops.calls if c[0] == "prologue"][:10] == [(1, 1, 1)] * 10
+    ops2 = OracleOps()
+    pipe2 = pl.CausalInferencePipeline(_tiny(ops2, disable_monarch=True), frame_hw=(2, 3), num_cache_frames=6)
+    pipe2.inference(torch.randn(1, 3, 16, 4, 6), torch.randn(1, 5, 32))
+    assert not any(c[0] == "monarch" for c in ops2.calls)
+
+
+def test_env_flags_are_read_like_the_reference(monkeypatch):
+    monkeypatch.setenv("MONARCH_ATTN_FRAMEWISE", "1")
+    monkeypatch.setenv("MONARCH_ATTN_H_REDUCE", "2")
+    monkeypatch.setenv("MONARCH_ATTN_DISABLE_LAYERS", "0,3")
+    f0, f1 = cm.AttentionFlags(0), cm.AttentionFlags(1)
+    assert f0.use_framewise and f0.h_reduce == 2 and f0.disable_monarch and not f1.disable_monarch
+    monkeypatch.setenv("MONARCH_ATTN_NUM_ITERS", "8")
+    with pytest.raises(NotImplementedError):
+        cm.AttentionFlags(1)
+
+
+def test_patchify_equals_conv3d_and_unpatchify_inverts():
+    m = _tiny(OracleOps()).model
+    x = torch.randn(2, 16, 3, 4, 6)
+    tok, grid = m._patchify(x)
+    ref = m.patch_embedding(x).flatten(2).transpose(1, 2)
+    assert grid == (3, 2, 3) and torch.allclose(tok, ref, atol=1e-5)
+    y = torch.randn(2, 18, 64)
+    u = m.unpatchify(y, grid)
+    assert u.shape == (2, 16, 3, 4, 6)
+    # token (f,h,w), patch offset (q,r), channel c lands at [c, f, 2h+q, 2w+r]
+    assert u[1, 5, 2, 3, 4] == y[1, (2 * 2 + 1) * 3 + 2].view(1, 2, 2, 16)[0, 1, 0, 5]
