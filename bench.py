@@ -1,9 +1,11 @@
 #!/usr/bin/env python3
-"""Benchmark of the attention hot path on one MI355X.
+"""Benchmark of the causal Wan-1.3B generator and its attention hot path on one MI355X.
 
-One step = one call of monarch_attn_with_kv_cache (cache write of the new 3-frame chunk + two-step
-Monarch attention) at the Wan-1.3B 480x832 chunk shape: B=1, H=12, D=128, 4680 queries against a
-21-frame (32760-token) KV cache, bf16, inputs resident in HBM.  Prints ONE JSON line.
+Headline (one step = one 21-latent-frame video): latent frames/s of the random-init causal Wan-1.3B DiT at
+480x832 (latents 21x16x60x104), 7 chunks of 3 frames x (4 denoising passes + 1 cache-refresh pass), Monarch
+framewise attention with per-layer KV cache, bf16, synthetic text context — BASELINE.json configs[2].
+Alongside, the attention op alone at the chunk shape (configs[1]): ms/call, per-kernel HIP-event durations,
+roofline of the dominant hot-path kernel, dense fallback, and a CPU baseline.  Prints ONE JSON line.
 """
 import argparse
 import ctypes as C
@@ -28,53 +30,51 @@ ROWS = B * H * A * B2 * F * B1                        # rows of Kbar / Y
 STEP1_BYTES = (2 * SKV + SQ) * H * D * 2 + 2 * ROWS * D * 2 + ROWS * 4      # read K,V,Q; write Kbar,Y,cl
 STEP2_BYTES = 2 * ROWS * D * 2 + ROWS * 4 + 2 * SQ * H * D * 2              # read Kbar,Y,cl,Q; write O
 
-
 # HBM bytes per launch measured with rocprofv3 (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 1 GiB
 # device copy in the same run); the runs and raw counters are in profiles/monarch_step{1,2}_c2.md.
 MEASURED_TRAFFIC = {"monarch_step1_kernel": 868.7e6, "monarch_step2_kernel": 647.2e6}
 
+LAYERS, CHUNKS, PASSES = 30, 7, 5
+
 
 def cpu_baseline(torch):
-    """The reference's CPU torch formulation restated by the oracle, fp32, on ONE of the 12 heads of the
-    same workload; scaled by 12 to a per-call figure."""
-    from oracle import monarch
-    torch.set_num_threads(os.cpu_count())
-    g = torch.Generator().manual_seed(0)
-    q = torch.randn(1, A, B1, B2, 1, D, generator=g)
-    k = torch.randn(1, F, B1, B2, 1, D, generator=g)
-    v = torch.randn(1, F, B1, B2, 1, D, generator=g)
-    monarch.monarch_1iter(q[:, :, :, :, :, :], k[:, :3], v[:, :3], D ** -0.5, dtype=torch.float32)   # warm-up
-    times = []
-    for _ in range(3):
-        t0 = time.perf_counter()
-        monarch.monarch_1iter(q, k, v, D ** -0.5, dtype=torch.float32)
-        times.append(time.perf_counter() - t0)
-    ms_call = sorted(times)[1] * 1e3 * H
-    return {"value": ms_call, "unit": "ms/call", "cores": os.cpu_count(), "kind": "port",
-            "sample": "1 of 12 heads of the same call (fp32 torch einsum oracle), median of 3, scaled x12"}
-
-
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--heads-per-pass", type=int, default=0)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--copy-probe", action="store_true",
-                    help="also run a plain 1 GiB device copy (known HBM traffic, for scaling rocprof counters)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU only: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
-        sys.exit(2)
-
-    import torch
+    """The same module code with the oracle's attention operators on the host cores, bf16 weights: ONE
+    transformer block, one pass over one 3-frame chunk against a 12-frame cache (the mean cache length of a
+    video), scaled by the 30 x 7 x 5 block passes of a video."""
     import self_forcing_amd as sfa
+    from oracle.ops import OracleOps
+    cm = sfa.causal_model
+    torch.set_num_threads(os.cpu_count())
+    torch.manual_seed(0)
+    blk = cm.CausalWanAttentionBlock(1536, 8960, 12, block_num=0, flags=cm.AttentionFlags(0, use_framewise=True),
+                                     ops=OracleOps()).to(torch.bfloat16).eval()
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, SQ, 1536, generator=g).to(torch.bfloat16)
+    e = torch.randn(1, 3, 6, 1536, generator=g).to(torch.bfloat16) * 0.1
+    ctx = torch.randn(1, 512, 1536, generator=g).to(torch.bfloat16)
+    kv = {"k": torch.randn(1, SKV, 12, 128, generator=g).to(torch.bfloat16),
+          "v": torch.randn(1, SKV, 12, 128, generator=g).to(torch.bfloat16),
+          "global_end_index": torch.tensor([9 * 1560]), "local_end_index": torch.tensor([9 * 1560])}
+    ca = {"k": None, "v": None, "is_init": False}
+    times = []
+    with torch.no_grad():
+        for _ in range(3):
+            kv["_global_end"] = kv["_local_end"] = 9 * 1560
+            t0 = time.perf_counter()
+            blk(x, e, (3, 30, 52), ctx, kv, ca, 9 * 1560)
+            times.append(time.perf_counter() - t0)
+    per_block = sorted(times)[0]
+    return {"value": 21.0 / (per_block * LAYERS * CHUNKS * PASSES), "unit": "latent frames/s", "cores": os.cpu_count(),
+            "kind": "port",
+            "sample": "1 of 1050 block passes of a video (bf16 torch-CPU block with oracle Monarch attention, "
+                      f"4680 tokens vs 12-frame cache), best of 3 = {per_block:.2f} s, scaled x1050"}
+
+
+def op_level(torch, sfa, args):
+    """Attention op alone at the chunk shape (BASELINE.json configs[1])."""
     from self_forcing_amd import lib as L
     from self_forcing_amd.monarch_attn import _desc
-
     dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
     g = torch.Generator().manual_seed(0)
     bf = torch.bfloat16
     q = torch.randn(B, SQ, H, D, generator=g).to(bf).to(dev)
@@ -88,14 +88,15 @@ def main():
         return sfa.monarch_attn.monarch_attn_with_kv_cache(q, kc, vc, nk, nv, start, end, 1, 1, 1, B1, B2,
                                                            heads_per_pass=args.heads_per_pass)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(10):
         out = step()
     torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    n = 50
+    t0 = time.perf_counter()
+    for _ in range(n):
+        out = step()
+    torch.cuda.synchronize()
+    ms_call = (time.perf_counter() - t0) * 1e3 / n
 
     # per-kernel durations, HIP events on the launch stream (inside the library)
     lib = L.load()
@@ -104,7 +105,7 @@ def main():
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     t1s, t2s = [], []
-    for _ in range(max(5, min(args.steps, 20))):
+    for _ in range(20):
         a1, a2 = C.c_float(0), C.c_float(0)
         L.check(lib.sfm_monarch_fwd_timed(C.byref(d), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), out.data_ptr(),
                                           ws.data_ptr(), nbytes, stream, C.byref(a1), C.byref(a2)))
@@ -112,7 +113,6 @@ def main():
         t2s.append(a2.value)
     s1_ms, s2_ms = sum(t1s) / len(t1s), sum(t2s) / len(t2s)
 
-    # dense fallback on the same tensors (for the record)
     for _ in range(2):
         sfa.attention.attention(q, kc, vc)
     torch.cuda.synchronize()
@@ -131,25 +131,75 @@ def main():
 
     s1_gbs = STEP1_BYTES / (s1_ms * 1e-3) / 1e9
     s2_gbs = STEP2_BYTES / (s2_ms * 1e-3) / 1e9
-    rec = {
-        "metric": "Monarch attn ms/call, causal Wan-1.3B 480x832 chunk shape (4680 q x 32760 kv, H12 D128), bf16",
-        "value": ms_per_step, "unit": "ms/call", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "configs[1]: monarch_attn_with_kv_cache, B1 H12 D128, a=3 f=21 b1=30 b2=52, "
-                               "new chunk written at tokens 28080..32760", "heads_per_pass": args.heads_per_pass},
-        "monarch_tflops": MONARCH_FLOPS / (ms_per_step * 1e-3) / 1e12,
-        "monarch_mfma_frac": MONARCH_FLOPS / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-        "kernel_ms": {"monarch_step1": s1_ms, "monarch_step2": s2_ms},
+    tfl = MONARCH_FLOPS / (ms_call * 1e-3) / 1e12
+    return {
+        "monarch_attn": {"workload": "configs[1]: monarch_attn_with_kv_cache, B1 H12 D128, a=3 f=21 b1=30 b2=52 "
+                                     "(4680 q x 32760 kv), new chunk written at tokens 28080..32760",
+                         "ms_per_call": ms_call, "tflops": tfl, "mfma_frac": tfl / MFMA_BF16_PEAK_TFLOPS,
+                         "kernel_ms": {"monarch_step1": s1_ms, "monarch_step2": s2_ms}},
         "dense_fallback": {"ms_per_call": dense_ms, "tflops": DENSE_FLOPS / (dense_ms * 1e-3) / 1e12,
                            "mfma_frac": DENSE_FLOPS / (dense_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS},
-        "roofline": {"kernel": "monarch_step1_kernel", "bound": "hbm", "achieved": s1_gbs, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": s1_gbs / HBM_PEAK_GBS, "algorithmic_bytes": STEP1_BYTES,
-                     "traffic": MEASURED_TRAFFIC["monarch_step1_kernel"]},
-        "roofline_step2": {"kernel": "monarch_step2_kernel", "bound": "hbm", "achieved": s2_gbs,
+        "roofline": {"kernel": "monarch_step1_kernel (configs[1] shape)", "bound": "hbm", "achieved": s1_gbs,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s1_gbs / HBM_PEAK_GBS,
+                     "algorithmic_bytes": STEP1_BYTES, "traffic": MEASURED_TRAFFIC["monarch_step1_kernel"]},
+        "roofline_step2": {"kernel": "monarch_step2_kernel (configs[1] shape)", "bound": "hbm", "achieved": s2_gbs,
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s2_gbs / HBM_PEAK_GBS,
                            "algorithmic_bytes": STEP2_BYTES, "traffic": MEASURED_TRAFFIC["monarch_step2_kernel"]},
     }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3, help="timed videos (21 latent frames each)")
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--heads-per-pass", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--op-only", action="store_true", help="skip the model; time the attention op only")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 1 GiB device copy (known HBM traffic, for scaling rocprof counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import self_forcing_amd as sfa
+
+    torch.cuda.set_device(0)
+    rec = {"metric": "latent frames/s, causal Wan-1.3B 480x832 bf16 (+ Monarch attn ms/call, MFMA %)",
+           "unit": "latent frames/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "configs[2]: random-init causal Wan-1.3B (30 layers, dim 1536, 12x128 heads, FFN 8960), "
+                                  "latents 21x16x60x104 in 7 chunks of 3 frames, 4 denoising steps + 1 cache-refresh "
+                                  "pass per chunk, Monarch framewise attention, per-layer KV cache, text context "
+                                  "[1,512,4096] ~ N(0,1); VAE and text encoder excluded",
+                      "heads_per_pass": args.heads_per_pass}}
+    if not args.op_only:
+        pl = sfa.pipeline
+        gen = pl.build_generator("1.3B", attention_flags=dict(use_framewise=True))
+        pipe = pl.CausalInferencePipeline(gen)
+        g = torch.Generator().manual_seed(0)
+        noise = torch.randn(1, 21, 16, 60, 104, generator=g).to(torch.bfloat16).cuda()
+        ctx = torch.randn(1, 512, 4096, generator=g).to(torch.bfloat16).cuda()
+        for _ in range(args.warmup):
+            pipe.inference(noise, ctx)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out = pipe.inference(noise, ctx)
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - t0) / args.steps
+        assert torch.isfinite(out).all()
+        rec["value"] = 21.0 / sec
+        rec["ms_per_step"] = sec * 1e3
+        del pipe, gen
+        torch.cuda.empty_cache()
+    rec.update(op_level(torch, sfa, args))
+    if args.op_only:
+        rec["metric"] = "Monarch attn ms/call, causal Wan-1.3B 480x832 chunk shape, bf16"
+        rec["unit"], rec["higher_is_better"] = "ms/call", False
+        rec["value"] = rec["ms_per_step"] = rec["monarch_attn"]["ms_per_call"]
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(rec))
