@@ -27,7 +27,7 @@ struct DnLds {
 };
 
 template <class E, int D>
-__global__ __launch_bounds__(256) void dense_fwd_kernel(sfm_dense_desc p, const uint16_t* __restrict__ q,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void dense_fwd_kernel(sfm_dense_desc p, const uint16_t* __restrict__ q,
                                                         const uint16_t* __restrict__ kp,
                                                         const uint16_t* __restrict__ vp, uint16_t* __restrict__ out,
                                                         float* __restrict__ lse) {
@@ -102,7 +102,7 @@ __global__ __launch_bounds__(256) void dense_fwd_kernel(sfm_dense_desc p, const 
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) oacc[dt][v] = 0.f;
-    float mrun = -INFINITY, lrun = 0.f;
+    float mrun = -INFINITY, lrun = 0.f;            // running max (scaled, base-2 units) and sum
     const float sc2 = p.sm_scale * kLog2e;
     const int ntile = (nk + 63) / 64;
 
@@ -125,31 +125,33 @@ __global__ __launch_bounds__(256) void dense_fwd_kernel(sfm_dense_desc p, const 
                 s[t] = E::mfma32(a, qb[ds], s[t]);
             }
         }
+        // online softmax in base 2; the scale is folded into the exponent argument (one fma per logit)
         const int lrem = nk - 64 * tile;           // valid keys in this tile (>= 1)
-        float mx = -INFINITY;
+        if (lrem < 64) {                           // ragged last tile only (wave-uniform)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int l = 32 * t + 8 * (v >> 2) + 4 * hf + (v & 3);
+                    s[t][v] = l < lrem ? s[t][v] : kMaskLogit;
+                }
+        }
+        float mx = s[0][0];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                int l = 32 * t + 8 * (v >> 2) + 4 * hf + (v & 3);
-                float z = l < lrem ? s[t][v] * sc2 : -INFINITY;
-                s[t][v] = z;
-                mx = fmaxf(mx, z);
-            }
-        mx = xhalf_max(mx);
+            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[t][v]);
+        mx = xhalf_max(mx) * sc2;
         const float mnew = fmaxf(mrun, mx);
-        const float alpha = exp2f(mrun - mnew);
         float psum = 0.f;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                float e = exp2f(s[t][v] - mnew);
+                float e = fast_exp2(fmaf(s[t][v], sc2, -mnew));
                 psum += e;
                 s[t][v] = e;
             }
-        lrun = lrun * alpha + psum;
-        mrun = mnew;
         u32x4 pb[4];
 #pragma unroll
         for (int st = 0; st < 4; ++st) {
@@ -159,10 +161,19 @@ __global__ __launch_bounds__(256) void dense_fwd_kernel(sfm_dense_desc p, const 
             pb[st].z = pack2<E>(s[t][v0 + 4], s[t][v0 + 5]);
             pb[st].w = pack2<E>(s[t][v0 + 6], s[t][v0 + 7]);
         }
+        // rescale the running output only when some query of the wave raised its maximum
+        if (__builtin_amdgcn_ballot_w64(mnew > mrun) != 0) {
+            const float alpha = fast_exp2(mrun - mnew);
+            lrun *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
+            mrun = mnew;
+        }
+        lrun += psum;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
             const uint16_t* arow = lds + L::kVT + (32 * dt + m) * L::kTPitch + 8 * hf;
 #pragma unroll
             for (int st = 0; st < 4; ++st) {

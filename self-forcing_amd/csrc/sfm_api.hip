@@ -137,7 +137,7 @@ static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
         set_error("k and v must share strides");
         return SFM_ERR_STRIDE;
     }
-    pl->r_pad = (pl->nf * pl->b1 + 31) / 32 * 32;
+    pl->r_pad = (pl->nf * pl->b1 + 31) / 32 * 32;   // whole 32-row chunks per (a, j) block
     pl->units = d->B * d->H;
     pl->mfma = monarch_mfma_supported(d->dtype, d->D, pl->b2);
     const size_t rows = (size_t)pl->na * pl->b2 * pl->r_pad;
