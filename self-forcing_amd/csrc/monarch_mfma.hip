@@ -33,14 +33,8 @@ template <int D>
 struct S1Lds {
     static constexpr int kRowPitch = D + 8;    // u16 per row of row-major K   [64][D+8]
     static constexpr int kTPitch = 72;         // u16 per row of K^T / V^T     [D][64+8]
-    static constexpr int kStagePitch = 40;     // u16 per row of a wave's output stage [32][32+8]
-    static constexpr int kStagePerWave = 32 * kStagePitch;
-    // The stages share their LDS with the row-major K tile: that tile is dead once every wave has its
-    // logits, and the stages are dead before the next tile is committed.
-    static __host__ __device__ constexpr int union_elems(int nwaves) {
-        return 64 * kRowPitch > nwaves * kStagePerWave ? 64 * kRowPitch : nwaves * kStagePerWave;
-    }
-    static __host__ __device__ constexpr size_t bytes(int nwaves) { return 2 * (size_t)(union_elems(nwaves) + 2 * D * kTPitch); }
+    static constexpr int kElems = 64 * kRowPitch + 2 * D * kTPitch;
+    static __host__ __device__ constexpr size_t bytes() { return 2 * (size_t)kElems; }
 };
 
 template <class E, int D>
@@ -62,11 +56,10 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int m = lane & 31;
     const int hf = lane >> 5;
 
-    uint16_t* const lds = lds_all + grp * (L::bytes(nwaves) / 2);
-    uint16_t* const lds_krow = lds;                                  // [64][D+8], aliased by the stages
-    uint16_t* const lds_kt = lds + L::union_elems(nwaves);           // [D][72]
+    uint16_t* const lds = lds_all + grp * L::kElems;
+    uint16_t* const lds_krow = lds;                                  // [64][D+8]
+    uint16_t* const lds_kt = lds + 64 * L::kRowPitch;                // [D][72]
     uint16_t* const lds_vt = lds_kt + D * L::kTPitch;                // [D][72]
-    uint16_t* const stage = lds + wave * L::kStagePerWave;           // [32][40], private to the wave
 
     // Workgroup = (unit, a-chunk, key block row k, range of kv block-frames f).  The query rows
     // Q[a, k, :, :] of the chunk depend on k only, so they are loaded once and stay in registers for
@@ -116,18 +109,10 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
     }
 
-    // rows this lane stores in the epilogue: 2 rows, c = 16*it + lane/4 of the wave's 32 columns,
-    // 16 bytes (lane%4) of each 64-byte piece.  BYTE offsets from the (uniform) scratch row of (f, k).
-    uint32_t orow[2];                                     // ~0u = no row
-#pragma unroll
-    for (int it = 0; it < 2; ++it) {
-        int c = wave * 32 + it * 16 + (lane >> 2);
-        bool ok = c < ncols;
-        int aa = a0 + (ok ? c / b2 : 0);
-        int jj = ok ? c % b2 : 0;
-        uint32_t o = ((uint32_t)(aa * b2 + jj) * p.ws_aj * D + (lane & 3) * 8) * 2;
-        orow[it] = ok ? o : ~0u;
-    }
+    // Output rows are stored straight from the accumulators: after one cross-half swap lane (c, hf) holds
+    // 8 consecutive head-dim elements of row c.  BYTE offset of this lane's row from the (uniform)
+    // scratch row of (f, k), ~0u = no row.
+    const uint32_t crow = col_ok ? ((uint32_t)(ca * b2 + cj) * p.ws_aj * D + 8 * hf) * 2 : ~0u;
     const uint32_t cloff = (uint32_t)(ca * b2 + cj) * p.ws_aj * 4;     // byte offset into cl, same convention
     const uint32_t ubase = (uint32_t)ul * p.ws_unit + (uint32_t)k * p.ws_row;   // scratch row of (unit, k), f = 0
     const uint32_t fstep = (uint32_t)p.b1 * p.ws_row;     // scratch rows between consecutive f
@@ -203,7 +188,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     for (int fb = f0; fb < f1; fb += G) {
         const int f = fb + grp;
         const bool has_f = f < f1;       // a group may run out of block-frames one round early; it still joins the barriers
-        lds_barrier();                   // previous iteration finished reading the tiles and the stages
+        lds_barrier();                   // previous iteration finished reading the tiles
         if (has_f) commit();
         if (f + G < f1) prefetch(f + G);
         lds_barrier();                   // K/V tiles visible
@@ -266,10 +251,10 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             if (col_ok && hf == 0)                 // sum_l R log2 R
                 *(float*)((char*)p.cl + (size_t)(ubase + (uint32_t)f * fstep) * 4 + cloff) = ent * inv_l - (mx + log2f(sum));
         }
-        lds_barrier();                   // every wave has its logits: the row-major K tile may be overwritten
-
-        // contractions with K^T then V^T, 32 head-dim columns at a time; each 32 x 32 piece goes out
-        // through the wave's LDS stage so that a row's 64 bytes are stored by 4 adjacent lanes
+        // contractions with K^T then V^T, 32 head-dim columns at a time.  A 32 x 32 accumulator tile holds,
+        // per lane (column c, half hf), head-dim 8g + 4hf + 0..3 for g = 0..3; swapping the g-odd dwords of the
+        // lower half with the g-even dwords of the upper half (v_permlane32_swap) leaves 8 consecutive
+        // elements per lane, i.e. 16-byte stores with the two halves of a row side by side.
 #pragma unroll
         for (int which = 0; which < 2; ++which) {
             const uint16_t* tbase = which == 0 ? lds_kt : lds_vt;
@@ -289,22 +274,16 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                         }
                     }
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        u32x2 w;
-                        w.x = pack2<E>(acc[4 * g + 0], acc[4 * g + 1]);
-                        w.y = pack2<E>(acc[4 * g + 2], acc[4 * g + 3]);
-                        *(u32x2*)(stage + m * L::kStagePitch + 8 * g + 4 * hf) = w;
+                    for (int gp = 0; gp < 2; ++gp) {
+                        const int g0 = 2 * gp, g1 = 2 * gp + 1;
+                        auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 0], acc[4 * g0 + 1]),
+                                                                   pack2<E>(acc[4 * g1 + 0], acc[4 * g1 + 1]), false, false);
+                        auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 2], acc[4 * g0 + 3]),
+                                                                   pack2<E>(acc[4 * g1 + 2], acc[4 * g1 + 3]), false, false);
+                        u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+                        if (crow != ~0u) *(u32x4*)(og + crow + (32 * dt + 16 * gp) * 2) = w;
                     }
                 }
-                lds_wave_sync();             // the stage is private to the wave
-                if (tile_active) {
-#pragma unroll
-                    for (int it = 0; it < 2; ++it) {
-                        u32x4 w = *(const u32x4*)(stage + (it * 16 + (lane >> 2)) * L::kStagePitch + (lane & 3) * 8);
-                        if (orow[it] != ~0u) *(u32x4*)(og + orow[it] + 64 * dt) = w;
-                    }
-                }
-                lds_wave_sync();
             }
         }
     }
@@ -525,7 +504,7 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const 
         return SFM_ERR_UNSUPPORTED;
     }
     const int groups = nwaves <= 5 ? 2 : 1;             // wave groups per workgroup (<= 10 waves in all)
-    const size_t lds1 = S1Lds<D>::bytes(nwaves) * groups;
+    const size_t lds1 = S1Lds<D>::bytes() * groups;
     if (lds1 > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)monarch_step1_kernel<E, D>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1);
