@@ -139,6 +139,22 @@ int sfm_qk_prologue(const sfm_prologue_desc* desc, const void* xq, const void* x
                     const void* wq, const void* wk, const double* rope_cos_sin, int32_t rope_max_pos,
                     void* q_out, void* k_cache, void* v_cache, void* stream);
 
+/* Block-level element-wise fusions around the attention op (rows = B*L token rows of C channels, C <= 8192,
+ * row strides in elements).  They keep the rounding points of the reference's eager ops.
+ *
+ * sfm_ln_modulate: y = LayerNorm(x) * (1 + scale[f]) + shift[f] with per-frame modulation rows
+ *   scale/shift + (row / rows_per_frame) * mod_stride (wan/modules/causal_model.py:1179-1183, 1198-1201), or,
+ *   when weight/bias are given (scale = shift = NULL), the affine LayerNorm of norm3 (causal_model.py:1194).
+ * sfm_gate_residual: x += y * gate[f] in place (causal_model.py:1189, 1203-1204); gate = NULL gives x += y.
+ * sfm_rms_norm: WanRMSNorm (wan/modules/model.py:462-478). */
+int sfm_ln_modulate(int32_t dtype, int64_t rows, int32_t C, float eps, const void* x, int64_t x_stride, void* y,
+                    int64_t y_stride, const void* scale, const void* shift, int64_t mod_stride, int32_t rows_per_frame,
+                    const void* weight, const void* bias, void* stream);
+int sfm_gate_residual(int32_t dtype, int64_t rows, int32_t C, void* x, int64_t x_stride, const void* y, int64_t y_stride,
+                      const void* gate, int64_t mod_stride, int32_t rows_per_frame, void* stream);
+int sfm_rms_norm(int32_t dtype, int64_t rows, int32_t C, float eps, const void* x, int64_t x_stride, void* y,
+                 int64_t y_stride, const void* weight, void* stream);
+
 /* Thread-local description of the last error returned on this thread ("" if none). */
 const char* sfm_last_error(void);
 

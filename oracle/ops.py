@@ -35,3 +35,22 @@ class OracleOps:
     def dense(self, q, k, v):
         self.calls.append(("dense", k.shape[1]))
         return dense.attention(q, k, v, dtype=self.compute_dtype).to(q.dtype)
+
+    # element-wise operators of the block: the reference's eager chains (causal_model.py:1176-1205, model.py:462-478)
+    def ln_modulate(self, x, scale, shift, eps):
+        nf = scale.shape[1]
+        n = torch.nn.functional.layer_norm(x, (x.shape[-1],), None, None, eps).type_as(x)
+        return (n.unflatten(1, (nf, x.shape[1] // nf)) * (1 + scale) + shift).flatten(1, 2)
+
+    def ln_affine(self, x, weight, bias, eps):
+        return torch.nn.functional.layer_norm(x, (x.shape[-1],), weight, bias, eps).type_as(x)
+
+    def gate_residual(self, x, y, gate=None):
+        if gate is None:
+            return x + y
+        nf = gate.shape[1]
+        return x + (y.unflatten(1, (nf, x.shape[1] // nf)) * gate).flatten(1, 2)
+
+    def rms_norm(self, x, weight, eps):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)).type_as(x) * weight

@@ -1,0 +1,68 @@
+"""Fused element-wise operators of the causal Wan block (LayerNorm + adaLN modulation, gated residual,
+RMSNorm); counterparts of the eager chains in wan/modules/causal_model.py:1176-1205 and
+wan/modules/model.py:462-478.  [B, L, C] tensors, modulation rows [B, F, 1, C] (one per latent frame)."""
+import torch
+
+from . import lib as _l
+from .monarch_attn import _DT, _stream
+
+
+def _rows(x):
+    if x.dim() != 3 or x.stride(2) != 1 or x.stride(0) != x.shape[1] * x.stride(1):
+        raise ValueError("expected a [B, L, C] tensor with contiguous channels and evenly strided rows")
+    return x.shape[0] * x.shape[1], x.shape[2], x.stride(1)
+
+
+def _mod(e, x):
+    """[B, F, 1, C] (or [B, F, C]) modulation tensor -> (tensor, frame stride, rows per frame)."""
+    B, L, C = x.shape
+    e = e.reshape(B, -1, C)
+    if e.stride(2) != 1 or (B > 1 and e.stride(0) != e.shape[1] * e.stride(1)):
+        e = e.contiguous()
+    if L % e.shape[1]:
+        raise ValueError("token count is not a multiple of the number of modulation frames")
+    return e, e.stride(1), L // e.shape[1]
+
+
+def ln_modulate(x, scale, shift, eps=1e-6):
+    """LayerNorm(x) (no affine) * (1 + scale) + shift with per-frame scale/shift."""
+    rows, C, xs = _rows(x)
+    sc, ms, rpf = _mod(scale, x)
+    sh, ms2, _ = _mod(shift, x)
+    if ms2 != ms:
+        sc, sh = sc.contiguous(), sh.contiguous()
+        ms = sc.stride(1)
+    y = torch.empty_like(x, memory_format=torch.contiguous_format)
+    with torch.cuda.device(x.device):
+        _l.check(_l.load().sfm_ln_modulate(_DT[x.dtype], rows, C, eps, x.data_ptr(), xs, y.data_ptr(), C, sc.data_ptr(),
+                                           sh.data_ptr(), ms, rpf, None, None, _stream(x)))
+    return y
+
+
+def ln_affine(x, weight, bias, eps=1e-6):
+    rows, C, xs = _rows(x)
+    y = torch.empty_like(x, memory_format=torch.contiguous_format)
+    with torch.cuda.device(x.device):
+        _l.check(_l.load().sfm_ln_modulate(_DT[x.dtype], rows, C, eps, x.data_ptr(), xs, y.data_ptr(), C, None, None, 0, 1,
+                                           weight.data_ptr(), bias.data_ptr(), _stream(x)))
+    return y
+
+
+def gate_residual_(x, y, gate=None):
+    """x += y * gate (per-frame gate) in place; gate=None: x += y."""
+    rows, C, xs = _rows(x)
+    _, _, ys = _rows(y)
+    g, ms, rpf = (None, 0, 1) if gate is None else _mod(gate, x)
+    with torch.cuda.device(x.device):
+        _l.check(_l.load().sfm_gate_residual(_DT[x.dtype], rows, C, x.data_ptr(), xs, y.data_ptr(), ys,
+                                             None if g is None else g.data_ptr(), ms, rpf, _stream(x)))
+    return x
+
+
+def rms_norm(x, weight, eps=1e-6):
+    rows, C, xs = _rows(x)
+    y = torch.empty_like(x, memory_format=torch.contiguous_format)
+    with torch.cuda.device(x.device):
+        _l.check(_l.load().sfm_rms_norm(_DT[x.dtype], rows, C, eps, x.data_ptr(), xs, y.data_ptr(), C, weight.data_ptr(),
+                                        _stream(x)))
+    return y

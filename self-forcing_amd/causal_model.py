@@ -24,6 +24,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import attention as _attn
+from . import block_ops as _blk
 from . import monarch_attn as _mon
 from . import prologue as _pro
 
@@ -33,8 +34,9 @@ TOTAL_SEQ_LEN = 21 * 30 * 52
 
 
 class HipAttentionOps:
-    """The attention operators the model calls.  Tests may pass another object with the same four
-    methods (e.g. one built on the CPU oracle) to obtain a reference run of the same module code."""
+    """The HIP operators the model calls (attention, fused prologue, fused block element-wise ops).  Tests
+    may pass another object with the same methods (e.g. one built on the CPU oracle and eager torch ops) to
+    obtain a reference run of the same module code."""
 
     def rope_table(self, head_dim, device):
         return _pro.rope_table(head_dim, device=device)
@@ -47,6 +49,19 @@ class HipAttentionOps:
 
     def dense(self, q, k, v):
         return _attn.attention(q, k, v, dtype=q.dtype)
+
+    # fused element-wise operators of the block (block_ops.py)
+    def ln_modulate(self, x, scale, shift, eps):
+        return _blk.ln_modulate(x, scale, shift, eps)
+
+    def ln_affine(self, x, weight, bias, eps):
+        return _blk.ln_affine(x, weight, bias, eps)
+
+    def gate_residual(self, x, y, gate=None):
+        return _blk.gate_residual_(x, y if y.stride(2) == 1 else y.contiguous(), gate)
+
+    def rms_norm(self, x, weight, eps):
+        return _blk.rms_norm(x, weight, eps)
 
 
 def _env_int(name, default):
@@ -215,7 +230,7 @@ class WanT2VCrossAttention(nn.Module):
 
     def forward(self, x, context, crossattn_cache=None):
         b, n, d = x.size(0), self.num_heads, self.head_dim
-        q = self.norm_q(self.q(x)).view(b, -1, n, d)
+        q = self.ops.rms_norm(self.q(x), self.norm_q.weight, self.norm_q.eps).view(b, -1, n, d)
         if crossattn_cache is not None and crossattn_cache["is_init"]:
             k, v = crossattn_cache["k"], crossattn_cache["v"]
         else:
@@ -233,6 +248,8 @@ class CausalWanAttentionBlock(nn.Module):
                  eps=1e-6, block_num=None, frame_hw=(FRAME_HEIGHT, FRAME_WIDTH), total_seq_len=None, flags=None,
                  ops=None):
         super().__init__()
+        self.eps = eps
+        self.ops = ops if ops is not None else HipAttentionOps()
         self.norm1 = WanLayerNorm(dim, eps)
         self.self_attn = CausalWanSelfAttention(dim, num_heads, local_attn_size, sink_size, qk_norm, eps, block_num,
                                                 frame_hw, total_seq_len, flags, ops)
@@ -244,14 +261,17 @@ class CausalWanAttentionBlock(nn.Module):
 
     def forward(self, x, e, grid, context, kv_cache, crossattn_cache, current_start):
         """x [B, L, C]; e [B, F, 6, C] per-frame modulation."""
-        nf, fs = e.shape[1], x.shape[1] // e.shape[1]
+        ops = self.ops
         e = (self.modulation.unsqueeze(1) + e).chunk(6, dim=2)
-        y = self.self_attn((self.norm1(x).unflatten(1, (nf, fs)) * (1 + e[1]) + e[0]).flatten(1, 2), grid, kv_cache,
-                           current_start)
-        x = x + (y.unflatten(1, (nf, fs)) * e[2]).flatten(1, 2)
-        x = x + self.cross_attn(self.norm3(x), context, crossattn_cache)
-        y = self.ffn((self.norm2(x).unflatten(1, (nf, fs)) * (1 + e[4]) + e[3]).flatten(1, 2))
-        return x + (y.unflatten(1, (nf, fs)) * e[5]).flatten(1, 2)
+        y = self.self_attn(ops.ln_modulate(x, e[1], e[0], self.eps), grid, kv_cache, current_start)
+        x = ops.gate_residual(x, y, e[2])
+        if isinstance(self.norm3, nn.Identity):
+            xn = x
+        else:
+            xn = ops.ln_affine(x, self.norm3.weight, self.norm3.bias, self.eps)
+        x = ops.gate_residual(x, self.cross_attn(xn, context, crossattn_cache))
+        y = self.ffn(ops.ln_modulate(x, e[4], e[3], self.eps))
+        return ops.gate_residual(x, y, e[5])
 
 
 class CausalHead(nn.Module):

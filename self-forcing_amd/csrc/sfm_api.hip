@@ -26,6 +26,30 @@ int launch_prologue(const sfm_prologue_desc& d, const TokMap& map, const void* x
                     const void* wq, const void* wk, const double* rope, void* q_out, void* kc, void* vc,
                     hipStream_t stream);
 bool monarch_generic_supported(const MonarchArgs& a);
+int launch_ln_modulate(int dtype, int64_t rows, int C, float eps, const void* x, int64_t xs, void* y, int64_t ys,
+                       const void* scale, const void* shift, int64_t ms, int rows_per_frame, const void* weight,
+                       const void* bias, hipStream_t stream);
+int launch_gate_residual(int dtype, int64_t rows, int C, void* x, int64_t xs, const void* y, int64_t ys,
+                         const void* gate, int64_t ms, int rows_per_frame, hipStream_t stream);
+int launch_rms_norm(int dtype, int64_t rows, int C, float eps, const void* x, int64_t xs, void* y, int64_t ys,
+                    const void* weight, hipStream_t stream);
+
+static int check_rows(int dtype, int64_t rows, int C, int64_t xs, int64_t ys) {
+    if (dtype != SFM_BF16 && dtype != SFM_F16 && dtype != SFM_F32) {
+        set_error("unsupported dtype %d", dtype);
+        return SFM_ERR_DTYPE;
+    }
+    if (rows < 1 || rows > 0x7fffffff || C < 8 || C % 8 || C > 8192) {
+        set_error("rows=%lld, C=%d: need rows >= 1 and C a multiple of 8 up to 8192", (long long)rows, C);
+        return SFM_ERR_SHAPE;
+    }
+    const int esz = dtype == SFM_F32 ? 4 : 2;
+    if (xs < C || ys < C || (xs * esz) % 16 || (ys * esz) % 16) {
+        set_error("row strides must be >= C and multiples of 16 bytes");
+        return SFM_ERR_STRIDE;
+    }
+    return SFM_OK;
+}
 
 static int elem_size(int dtype) { return dtype == SFM_F32 ? 4 : 2; }
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15) == 0; }
@@ -507,6 +531,63 @@ int sfm_qk_prologue(const sfm_prologue_desc* d, const void* xq, const void* xk, 
     }
     TokMap map = make_map(d->tiling, 1);
     return launch_prologue(*d, map, xq, xk, xv, wq, wk, rope_cos_sin, q_out, k_cache, v_cache, (hipStream_t)stream);
+}
+
+int sfm_ln_modulate(int32_t dtype, int64_t rows, int32_t C, float eps, const void* x, int64_t x_stride, void* y,
+                    int64_t y_stride, const void* scale, const void* shift, int64_t mod_stride, int32_t rows_per_frame,
+                    const void* weight, const void* bias, void* stream) {
+    int rc = check_rows(dtype, rows, C, x_stride, y_stride);
+    if (rc) return rc;
+    const bool affine = weight != nullptr || bias != nullptr;
+    if (!x || !y || (affine && (!weight || !bias)) || (!affine && (!scale || !shift))) {
+        set_error("x, y and either (scale, shift) or (weight, bias) must be non-NULL");
+        return SFM_ERR_NULL;
+    }
+    if (!affine && (rows_per_frame < 1 || mod_stride < 0 || (mod_stride * (dtype == SFM_F32 ? 4 : 2)) % 16)) {
+        set_error("rows_per_frame must be >= 1 and mod_stride a multiple of 16 bytes");
+        return SFM_ERR_STRIDE;
+    }
+    if (!aligned16(x) || !aligned16(y) || !aligned16(scale) || !aligned16(shift) || !aligned16(weight) || !aligned16(bias)) {
+        set_error("tensors must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    return launch_ln_modulate(dtype, rows, C, eps, x, x_stride, y, y_stride, scale, shift, mod_stride,
+                              affine ? 1 : rows_per_frame, weight, bias, (hipStream_t)stream);
+}
+
+int sfm_gate_residual(int32_t dtype, int64_t rows, int32_t C, void* x, int64_t x_stride, const void* y, int64_t y_stride,
+                      const void* gate, int64_t mod_stride, int32_t rows_per_frame, void* stream) {
+    int rc = check_rows(dtype, rows, C, x_stride, y_stride);
+    if (rc) return rc;
+    if (!x || !y) {
+        set_error("x and y must be non-NULL");
+        return SFM_ERR_NULL;
+    }
+    if (gate && (rows_per_frame < 1 || mod_stride < 0 || (mod_stride * (dtype == SFM_F32 ? 4 : 2)) % 16)) {
+        set_error("rows_per_frame must be >= 1 and mod_stride a multiple of 16 bytes");
+        return SFM_ERR_STRIDE;
+    }
+    if (!aligned16(x) || !aligned16(y) || !aligned16(gate)) {
+        set_error("tensors must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    return launch_gate_residual(dtype, rows, C, x, x_stride, y, y_stride, gate, mod_stride, gate ? rows_per_frame : 1,
+                                (hipStream_t)stream);
+}
+
+int sfm_rms_norm(int32_t dtype, int64_t rows, int32_t C, float eps, const void* x, int64_t x_stride, void* y,
+                 int64_t y_stride, const void* weight, void* stream) {
+    int rc = check_rows(dtype, rows, C, x_stride, y_stride);
+    if (rc) return rc;
+    if (!x || !y || !weight) {
+        set_error("x, y and weight must be non-NULL");
+        return SFM_ERR_NULL;
+    }
+    if (!aligned16(x) || !aligned16(y) || !aligned16(weight)) {
+        set_error("tensors must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    return launch_rms_norm(dtype, rows, C, eps, x, x_stride, y, y_stride, weight, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -19,7 +19,8 @@ ERR_NAMES = {
 # every symbol include/sfm_attn.h declares
 SYMBOLS = [
     "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
-    "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_last_error", "sfm_version",
+    "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
+    "sfm_rms_norm", "sfm_last_error", "sfm_version",
 ]
 
 
@@ -81,6 +82,9 @@ def load():
     lib.sfm_dense_fwd.argtypes = [C.POINTER(DenseDesc), P, P, P, P, P, P]
     lib.sfm_full_attention_with_kv_cache.argtypes = [C.POINTER(DenseDesc), P, P, P, P, P, S3, I64, I64, P, P, P]
     lib.sfm_qk_prologue.argtypes = [C.POINTER(PrologueDesc), P, P, P, P, P, P, C.c_int32, P, P, P, P]
+    lib.sfm_ln_modulate.argtypes = [C.c_int32, I64, C.c_int32, C.c_float, P, I64, P, I64, P, P, I64, C.c_int32, P, P, P]
+    lib.sfm_gate_residual.argtypes = [C.c_int32, I64, C.c_int32, P, I64, P, I64, P, I64, C.c_int32, P]
+    lib.sfm_rms_norm.argtypes = [C.c_int32, I64, C.c_int32, C.c_float, P, I64, P, I64, P, P]
     for name in SYMBOLS:
         if name not in ("sfm_version", "sfm_last_error"):
             getattr(lib, name).restype = C.c_int
