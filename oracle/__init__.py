@@ -14,17 +14,20 @@ in ``tests/test_oracle_*.py``.
 ====================  ========================================================
 function              pinned by
 ====================  ========================================================
-blocks.to_blocks /    explicit index formula checked token by token, round
-blocks.from_blocks    trip, identity-in-memory special case (f_tied=1,
+blocks.to_blocks /    golden permutations of the reference's _get_rearrange_fns;
+blocks.from_blocks    explicit index formula checked token by token, round
+                      trip, identity-in-memory special case (f_tied=1,
                       w_reduce=1)
-monarch.monarch_1iter b2=1 => dense softmax attention; b1=1,f=1 => dense;
+monarch.monarch_1iter golden vectors of the reference's monarch_attn_ref_op
+                      (tests/golden/); b2=1 => dense softmax attention; b1=1,f=1 => dense;
                       implied N x N matrix L*R built with scalar loops has
                       unit row sums and reproduces the output; constant V;
                       permutation of KV block-frames; LSE merge of KV chunks;
                       Gibbs equality of the step-2 logit on the i==k diagonal
-monarch.monarch_iter  num_iters=1 equals monarch_1iter up to the 1/(1+1e-6)
-                      factor; b2=1 => dense for any num_iters.  Intermediate
-                      iterates for num_iters>1: PARITY UNPINNED
+monarch.monarch_iter  golden vectors of the reference's own monarch_attn_slow for
+                      num_iters in {1,2,3,8} (tests/golden/, <= 2e-6: the reference
+                      runs its softmaxes in float32); num_iters=1 equals
+                      monarch_1iter up to the 1/(1+1e-6) factor; b2=1 => dense
 monarch.*_kv_cache,   compositions of the above with a cache write; pinned by
 monarch.causal        slicing identities (causal == chunk by chunk)
 dense.attention       torch.nn.functional.scaled_dot_product_attention (library

@@ -115,8 +115,8 @@ def monarch_iter(Q, K, V, sm_scale, num_iters=1, dtype=torch.float64):
     Each pass recomputes the right factor from per-block query representatives
         rep[a,f,k,j] = sum_i L[a,i,j,(f,k)] Q[a,i,j]  with weight  w = sum_i L
     (first pass: rep = Q[a,k,j], w = 1) using logits <rep, K> * min(1/(w+1e-6), 1e4),
-    then the left factor as in `monarch_1iter`.  PARITY UNPINNED for the
-    intermediate iterates when num_iters > 1 (no independent closed form)."""
+    then the left factor as in `monarch_1iter`.  Pinned by golden vectors of the
+    reference function for num_iters in {1, 2, 3, 8} (tests/test_oracle_golden.py)."""
     B, na, b1, b2, H, D = Q.shape
     nf = K.shape[1]
     out = torch.empty((B, na, b1, b2, H, D), dtype=dtype)
