@@ -53,6 +53,9 @@ typedef struct sfm_monarch_desc {
     int32_t causal_block_frames; /* 0 = every query sees every key; else block-causal in units of
                                  block-frames (monarch_attn.py:139-141, 804-807), requires Sq == Skv */
     float   sm_scale;         /* logit scale; the reference default is D^-0.5 (monarch_attn.py:1780-1781) */
+    int32_t num_iters;        /* 1: the two-kernel fast path; > 1: alternating refinement of the two factors
+                                 (monarch_attn_slow, monarch_attn.py:1705-1751), fp32 kernels, no causal mask */
+    int32_t reserved;         /* 0 */
     int64_t q_stride[3];      /* batch, token, head */
     int64_t k_stride[3];
     int64_t v_stride[3];      /* must equal k_stride (monarch_attn.py:1261) */

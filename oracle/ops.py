@@ -23,12 +23,15 @@ class OracleOps:
         self.calls.append(("prologue", start_frame, start_idx, (f_tied, h_reduce, w_reduce)))
         return q
 
-    def monarch_cached(self, q, k_view, v_view, f_tied, h_reduce, w_reduce, h, w):
+    def monarch_cached(self, q, k_view, v_view, f_tied, h_reduce, w_reduce, h, w, num_iters=1):
         B, _, H, D = q.shape
         qb = blocks.to_blocks(q, f_tied, h_reduce, w_reduce, h, w)
         b1, b2 = qb.shape[2], qb.shape[3]
-        out = monarch.monarch_1iter(qb, k_view.reshape(B, -1, b1, b2, H, D), v_view.reshape(B, -1, b1, b2, H, D),
-                                    D ** -0.5, dtype=self.compute_dtype)
+        kb, vb = k_view.reshape(B, -1, b1, b2, H, D), v_view.reshape(B, -1, b1, b2, H, D)
+        if num_iters == 1:
+            out = monarch.monarch_1iter(qb, kb, vb, D ** -0.5, dtype=self.compute_dtype)
+        else:
+            out = monarch.monarch_iter(qb, kb, vb, D ** -0.5, num_iters, dtype=self.compute_dtype)
         self.calls.append(("monarch", k_view.shape[1]))
         return blocks.from_blocks(out, f_tied, h_reduce, w_reduce, h, w).to(q.dtype)
 

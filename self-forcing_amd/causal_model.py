@@ -44,8 +44,9 @@ class HipAttentionOps:
     def qk_prologue(self, *args, **kwargs):
         return _pro.qk_prologue(*args, **kwargs)
 
-    def monarch_cached(self, q, k_view, v_view, f_tied, h_reduce, w_reduce, h, w):
-        return _mon.monarch_attn(q, k_view, v_view, f_tied, h_reduce, w_reduce, h, w, kv_block_order=True)
+    def monarch_cached(self, q, k_view, v_view, f_tied, h_reduce, w_reduce, h, w, num_iters=1):
+        return _mon.monarch_attn(q, k_view, v_view, f_tied, h_reduce, w_reduce, h, w, kv_block_order=True,
+                                 num_iters=num_iters)
 
     def dense(self, q, k, v):
         return _attn.attention(q, k, v, dtype=q.dtype)
@@ -87,8 +88,6 @@ class AttentionFlags:
             if not hasattr(self, k):
                 raise TypeError(f"unknown attention flag {k}")
             setattr(self, k, v)
-        if self.num_iters != 1 and not self.disable_monarch:
-            raise NotImplementedError("MONARCH_ATTN_NUM_ITERS > 1 is not built")
 
 
 class WanRMSNorm(nn.Module):
@@ -209,7 +208,7 @@ class CausalWanSelfAttention(nn.Module):
         if dense:
             y = self.ops.dense(q, k_view, v_view)
         else:
-            y = self.ops.monarch_cached(q, k_view, v_view, f_tied, fl.h_reduce, fl.w_reduce, h, w)
+            y = self.ops.monarch_cached(q, k_view, v_view, f_tied, fl.h_reduce, fl.w_reduce, h, w, fl.num_iters)
         cache_commit(kv_cache, current_end, local_end)
         return self.o(y.flatten(2))
 

@@ -154,16 +154,244 @@ __global__ __launch_bounds__(256) void monarch_generic_step2(MonarchArgs p) {
     }
 }
 
-static size_t generic_lds1(const MonarchArgs& a) { return sizeof(float) * ((size_t)2 * a.b2 * (a.D + 1) + a.D + a.b2); }
+static size_t generic_lds1_bytes(const MonarchArgs& a) { return sizeof(float) * ((size_t)2 * a.b2 * (a.D + 1) + a.D + a.b2); }
+
+// ------------------------------------------------------------------------------------------------
+// Iterated refinement (num_iters > 1): wan/modules/monarch_attn.py:1705-1751 (monarch_attn_slow), which the
+// reference runs as pure-torch einsums.  Each pass recomputes the right factor from per-block query
+// representatives rep[a,f,k,j,:] = sum_i L[a,i,j,(f,k)] Q s^1/2 with weight w = sum_i L (first pass:
+// rep = Q[a,k,j] s^1/2, w = 1) using logits <rep, K s^1/2> * min(1/(w + 1e-6), 1e4), then the left factor.
+// fp32 throughout; Kbar here is R (K s^1/2), cl = sum_l R ln R (natural log), rep / w live in the scratch.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void monarch_iter_step1(MonarchArgs p, int first, int last) {
+    extern __shared__ float sm[];
+    const int D = p.D, b2 = p.b2, DP = D + 1;
+    float* Ks = sm;                    // [b2][D+1]  K * sqrt(s)
+    float* Vs = Ks + b2 * DP;          // [b2][D+1]
+    float* qs = Vs + b2 * DP;          // [D]        representative
+    float* zs = qs + D;                // [b2]
+    const int k = blockIdx.x, f = blockIdx.y;
+    const int ul = blockIdx.z / p.na, a = blockIdx.z % p.na;
+    const int unit = p.unit0 + ul;
+    const int b = unit / p.H, h = unit % p.H;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const float rs = sqrtf(p.scale);
+
+    const int64_t krow0 = p.kmap.row(f, k);
+    for (int e = tid; e < b2 * D; e += nt) {
+        int l = e / D, d = e % D;
+        Ks[l * DP + d] = rs * Ld<T>::get(p.k, (int64_t)b * p.ks[0] + (krow0 + l) * p.ks[1] + (int64_t)h * p.ks[2] + d);
+        Vs[l * DP + d] = last ? Ld<T>::get(p.v, (int64_t)b * p.vs[0] + (krow0 + l) * p.vs[1] + (int64_t)h * p.vs[2] + d) : 0.f;
+    }
+    const int64_t qrow0 = p.qmap.row(a, k);
+    float* kbar = (float*)p.kbar;
+    float* yw = (float*)p.y;
+    const float* rep = (const float*)p.rep;
+
+    for (int j = 0; j < b2; ++j) {
+        const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj + (int64_t)(f * p.b1 + k) * p.ws_row;
+        __syncthreads();
+        for (int d = tid; d < D; d += nt)
+            qs[d] = first ? rs * Ld<T>::get(p.q, (int64_t)b * p.qs[0] + (qrow0 + j) * p.qs[1] + (int64_t)h * p.qs[2] + d)
+                          : rep[blk * D + d];
+        const float wsc = first ? 1.0f / (1.0f + 1e-6f) : fminf(1.0f / (p.wgt[blk] + 1e-6f), 1e4f);
+        __syncthreads();
+        for (int l = tid; l < b2; l += nt) {
+            float acc = 0.f;
+            for (int d = 0; d < D; ++d) acc += qs[d] * Ks[l * DP + d];
+            zs[l] = acc * wsc;
+        }
+        __syncthreads();
+        float mx = -INFINITY;
+        for (int l = 0; l < b2; ++l) mx = fmaxf(mx, zs[l]);
+        float sum = 0.f, ent = 0.f;
+        for (int l = 0; l < b2; ++l) {
+            float e = expf(zs[l] - mx);
+            sum += e;
+            ent += e * zs[l];
+        }
+        const float inv = 1.f / sum;
+        if (tid == 0) p.cl[blk] = ent * inv - (mx + logf(sum));
+        for (int d = tid; d < D; d += nt) {
+            float ak = 0.f, av = 0.f;
+            for (int l = 0; l < b2; ++l) {
+                float r = expf(zs[l] - mx) * inv;
+                ak += r * Ks[l * DP + d];
+                av += r * Vs[l * DP + d];
+            }
+            kbar[blk * D + d] = ak;
+            if (last) yw[blk * D + d] = av;
+        }
+    }
+}
+
+constexpr int kIterRows = 32;   // query rows of one (a, j) column held in registers / LDS at a time
+
+// workgroup = (unit, a, j): left factor L[i, r] over all rows r = (f, k); then either the new representatives
+// (rep[r,:] = sum_i L[i,r] q_i, w[r] = sum_i L[i,r]) or, in the last pass, the output rows sum_r L[i,r] Y[r,:].
+// Query rows are taken `ic` at a time (rows of L are independent; rep and w accumulate over the chunks).
+template <typename T>
+__global__ __launch_bounds__(256) void monarch_iter_step2(MonarchArgs p, int last, int ic) {
+    extern __shared__ float sm[];
+    const int D = p.D, b2 = p.b2, b1 = p.b1, DP = D + 1;
+    const int a = blockIdx.x / b2, j = blockIdx.x % b2;
+    const int ul = blockIdx.y;
+    const int unit = p.unit0 + ul;
+    const int b = unit / p.H, h = unit % p.H;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const int R = p.nf * b1;
+    const float rs = sqrtf(p.scale);
+    float* qs = sm;                    // [ic][D+1]   Q[a, i, j, :] * sqrt(s)
+    float* S = qs + ic * DP;           // [ic][R]     logits, then L
+    float* red = S + (size_t)ic * R;   // [2 * ic]    row max, 1 / row sum
+
+    const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj;
+    const int64_t rsd = p.ws_row;
+    const float* kbar = (const float*)p.kbar + blk * D;
+    const float* yw = (const float*)p.y + blk * D;
+    const float* cl = p.cl + blk;
+    float* rep = (float*)p.rep + blk * D;
+    float* wgt = p.wgt + blk;
+
+    for (int i0 = 0; i0 < b1; i0 += ic) {
+        const int ni = b1 - i0 < ic ? b1 - i0 : ic;
+        __syncthreads();
+        for (int e = tid; e < ni * D; e += nt) {
+            int i = e / D, d = e % D;
+            qs[i * DP + d] =
+                rs * Ld<T>::get(p.q, (int64_t)b * p.qs[0] + (p.qmap.row(a, i0 + i) + j) * p.qs[1] + (int64_t)h * p.qs[2] + d);
+        }
+        __syncthreads();
+        for (int r = tid; r < R; r += nt) {            // logits of row r against the chunk's query rows
+            float acc[kIterRows];
+#pragma unroll
+            for (int i = 0; i < kIterRows; ++i) acc[i] = 0.f;
+            const float* row = kbar + (int64_t)r * rsd * D;
+            for (int d = 0; d < D; ++d) {
+                const float kv = row[d];
+#pragma unroll
+                for (int i = 0; i < kIterRows; ++i)
+                    if (i < ni) acc[i] += qs[i * DP + d] * kv;
+            }
+            const float c = cl[r * rsd];
+#pragma unroll
+            for (int i = 0; i < kIterRows; ++i)
+                if (i < ni) S[(size_t)i * R + r] = acc[i] - c;
+        }
+        __syncthreads();
+        for (int i = tid >> 6; i < ni; i += nt >> 6) {  // one wave per query row: max and sum over r
+            float mx = -INFINITY;
+            for (int r = tid & 63; r < R; r += 64) mx = fmaxf(mx, S[(size_t)i * R + r]);
+            for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            float sum = 0.f;
+            for (int r = tid & 63; r < R; r += 64) sum += expf(S[(size_t)i * R + r] - mx);
+            for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+            if ((tid & 63) == 0) {
+                red[2 * i] = mx;
+                red[2 * i + 1] = 1.f / sum;
+            }
+        }
+        __syncthreads();
+        for (int e = tid; e < ni * R; e += nt) {
+            int i = e / R;
+            S[e] = expf(S[e] - red[2 * i]) * red[2 * i + 1];
+        }
+        __syncthreads();
+        if (!last) {
+            for (int r = tid; r < R; r += nt) {
+                float w = i0 ? wgt[r * rsd] : 0.f;
+                for (int i = 0; i < ni; ++i) w += S[(size_t)i * R + r];
+                wgt[r * rsd] = w;
+                float* dst = rep + (int64_t)r * rsd * D;
+                for (int d = 0; d < D; ++d) {
+                    float acc = i0 ? dst[d] : 0.f;
+                    for (int i = 0; i < ni; ++i) acc += S[(size_t)i * R + r] * qs[i * DP + d];
+                    dst[d] = acc;
+                }
+            }
+        } else {
+            for (int d = tid; d < D; d += nt) {
+                float acc[kIterRows];
+#pragma unroll
+                for (int i = 0; i < kIterRows; ++i) acc[i] = 0.f;
+                for (int r = 0; r < R; ++r) {
+                    const float yv = yw[(int64_t)r * rsd * D + d];
+#pragma unroll
+                    for (int i = 0; i < kIterRows; ++i)
+                        if (i < ni) acc[i] += S[(size_t)i * R + r] * yv;
+                }
+#pragma unroll
+                for (int i = 0; i < kIterRows; ++i)
+                    if (i < ni)
+                        Ld<T>::put(p.out,
+                                   (int64_t)b * p.os[0] + (p.qmap.row(a, i0 + i) + j) * p.os[1] + (int64_t)h * p.os[2] + d,
+                                   acc[i]);
+            }
+        }
+    }
+}
+
+// query rows per chunk: as many as fit 128 KB of LDS next to the chunk's logits, at most kIterRows
+static int iter_rows(const MonarchArgs& a) {
+    const size_t per_row = sizeof(float) * ((size_t)(a.D + 1) + (size_t)a.nf * a.b1 + 2);
+    size_t ic = (128 * 1024) / per_row;
+    if (ic > (size_t)kIterRows) ic = kIterRows;
+    if (ic > (size_t)a.b1) ic = a.b1;
+    return (int)ic;
+}
+
+static size_t iter_lds2(const MonarchArgs& a) {
+    return sizeof(float) * (size_t)iter_rows(a) * ((size_t)(a.D + 1) + (size_t)a.nf * a.b1 + 2);
+}
+
+bool monarch_iter_supported(const MonarchArgs& a) { return iter_rows(a) >= 1 && generic_lds1_bytes(a) <= 160 * 1024; }
+
+template <typename T>
+static int launch_iter_t(const MonarchArgs& a, int nunits, int num_iters, hipStream_t stream) {
+    const size_t l1 = generic_lds1_bytes(a), l2 = iter_lds2(a);
+    hipError_t err = hipSuccess;
+    if (l1 > 64 * 1024)
+        err = hipFuncSetAttribute((const void*)monarch_iter_step1<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)l1);
+    if (err == hipSuccess && l2 > 64 * 1024)
+        err = hipFuncSetAttribute((const void*)monarch_iter_step2<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)l2);
+    if (err != hipSuccess) {
+        set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(err));
+        return SFM_ERR_HIP;
+    }
+    for (int it = 0; it < num_iters; ++it) {
+        const int last = it + 1 == num_iters;
+        hipLaunchKernelGGL((monarch_iter_step1<T>), dim3(a.b1, a.nf, nunits * a.na), dim3(256), l1, stream, a, it == 0, last);
+        hipLaunchKernelGGL((monarch_iter_step2<T>), dim3(a.na * a.b2, nunits), dim3(256), l2, stream, a, last, iter_rows(a));
+    }
+    err = hipGetLastError();
+    if (err != hipSuccess) {
+        set_error("hip launch failed: %s", hipGetErrorString(err));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream) {
+    if (!monarch_iter_supported(a)) {
+        set_error("iterated Monarch: block shape b1=%d, b2=%d, rows=%d, D=%d exceeds the limits of this path", a.b1, a.b2,
+                  a.nf * a.b1, a.D);
+        return SFM_ERR_UNSUPPORTED;
+    }
+    if (dtype == SFM_F32) return launch_iter_t<float>(a, nunits, num_iters, stream);
+    if (dtype == SFM_BF16) return launch_iter_t<BF16>(a, nunits, num_iters, stream);
+    return launch_iter_t<F16>(a, nunits, num_iters, stream);
+}
+
 static size_t generic_lds2(const MonarchArgs& a) { return sizeof(float) * ((size_t)a.D + (size_t)a.nf * a.b1 + 256); }
 
 bool monarch_generic_supported(const MonarchArgs& a) {
-    return generic_lds1(a) <= 160 * 1024 && generic_lds2(a) <= 160 * 1024;
+    return generic_lds1_bytes(a) <= 160 * 1024 && generic_lds2(a) <= 160 * 1024;
 }
 
 template <typename T>
 static int launch_generic_t(const MonarchArgs& a, int nunits, hipStream_t stream, const StepEvents* ev) {
-    const size_t l1 = generic_lds1(a), l2 = generic_lds2(a);
+    const size_t l1 = generic_lds1_bytes(a), l2 = generic_lds2(a);
     hipError_t err = hipSuccess;
     if (l1 > 64 * 1024)
         err = hipFuncSetAttribute((const void*)monarch_generic_step1<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)l1);

@@ -103,7 +103,7 @@ static int check_strides(const char* name, const int64_t s[3], int64_t tokens, i
 
 struct MonarchPlan {
     int na, nf, b1, b2, r_pad, units;
-    bool mfma;
+    bool mfma, iter;
     size_t per_unit;   // workspace bytes per (batch x head) unit
 };
 
@@ -163,9 +163,18 @@ static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
     }
     pl->r_pad = (pl->nf * pl->b1 + 31) / 32 * 32;   // whole 32-row chunks per (a, j) block
     pl->units = d->B * d->H;
-    pl->mfma = monarch_mfma_supported(d->dtype, d->D, pl->b2);
+    if (d->num_iters < 1) {
+        set_error("num_iters must be >= 1");
+        return SFM_ERR_SHAPE;
+    }
+    if (d->num_iters > 1 && d->causal_block_frames) {
+        set_error("block-causal masking is defined for num_iters == 1 only");
+        return SFM_ERR_UNSUPPORTED;
+    }
+    pl->iter = d->num_iters > 1;
+    pl->mfma = !pl->iter && monarch_mfma_supported(d->dtype, d->D, pl->b2);
     const size_t rows = (size_t)pl->na * pl->b2 * pl->r_pad;
-    pl->per_unit = rows * d->D * (pl->mfma ? 2 : 4) * 2 + rows * sizeof(float);
+    pl->per_unit = rows * d->D * (pl->mfma ? 2 : 4) * (pl->iter ? 3 : 2) + rows * sizeof(float) * (pl->iter ? 2 : 1);
     pl->per_unit = (pl->per_unit + 255) / 256 * 256;
     return SFM_OK;
 }
@@ -186,7 +195,7 @@ using namespace sfm;
 
 extern "C" {
 
-int sfm_version(void) { return 1; }
+int sfm_version(void) { return 2; }
 
 const char* sfm_last_error(void) { return g_err; }
 
@@ -270,6 +279,17 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
         a.kbar = workspace;
         a.y = (char*)workspace + mat_bytes * upp;
         a.cl = (float*)((char*)workspace + 2 * mat_bytes * upp);
+        if (pl.iter) {
+            a.rep = (char*)a.cl + rows * sizeof(float) * upp;
+            a.wgt = (float*)((char*)a.rep + mat_bytes * upp);
+            if (step_ms) {
+                set_error("the timed variant covers num_iters == 1 only");
+                return SFM_ERR_UNSUPPORTED;
+            }
+            rc = launch_monarch_iter(a, desc->dtype, n, desc->num_iters, (hipStream_t)stream);
+            if (rc) return rc;
+            continue;
+        }
         StepEvents se;
         if (step_ms) {
             for (int i = 0; i < 3; ++i)

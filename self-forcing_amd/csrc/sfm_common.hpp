@@ -130,6 +130,8 @@ struct MonarchArgs {
     void* kbar;      // [units_per_pass][na][b2][r_pad][D]   16-bit (MFMA path) or float (generic path)
     void* y;         // same shape
     float* cl;       // [units_per_pass][na][b2][r_pad]      sum_l R log2 R  (log2 units)
+    void* rep;       // iterated refinement only: query representatives, float, same shape as kbar
+    float* wgt;      // iterated refinement only: their weights, same shape as cl
     int B, H, D, na, nf, b1, b2;
     int r_pad;       // rows per (a, j) block of the workspace: round_up(nf*b1, 32)
     // scratch row index of (unit ul, a, j, r) = ul*ws_unit + (a*b2 + j)*ws_aj + r*ws_row
@@ -154,6 +156,7 @@ struct StepEvents {
 int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev);
 int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev);
 bool monarch_mfma_supported(int dtype, int D, int b2);
+int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
 
 void set_error(const char* fmt, ...);
 

@@ -33,6 +33,7 @@ class MonarchDesc(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
                 ("q_tokens", C.c_int32), ("kv_tokens", C.c_int32), ("tiling", Tiling),
                 ("kv_block_order", C.c_int32), ("causal_block_frames", C.c_int32), ("sm_scale", C.c_float),
+                ("num_iters", C.c_int32), ("reserved", C.c_int32),
                 ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
                 ("o_stride", C.c_int64 * 3)]
 

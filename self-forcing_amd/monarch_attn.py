@@ -5,6 +5,8 @@
 
 Inputs are [B, S, H, D] CUDA tensors (bf16 / fp16 / fp32, head_dim contiguous) in token order;
 the KV cache holds rows in Monarch block order and is updated in place.  Forward only.
+num_iters > 1 runs the alternating refinement the reference implements in pure torch
+(monarch_attn_slow, wan/modules/monarch_attn.py:1705-1751) as fp32 HIP kernels.
 """
 import ctypes as C
 
@@ -28,7 +30,7 @@ def _check4(name, t, dtype=None, device=None):
         raise ValueError(f"{name}: device {t.device} differs from q's {device}")
 
 
-def _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, kv_block_order, causal_block_frames):
+def _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, kv_block_order, causal_block_frames, num_iters=1):
     if q.dtype not in _DT:
         raise ValueError(f"unsupported dtype {q.dtype}")
     d = _l.MonarchDesc()
@@ -39,6 +41,7 @@ def _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, kv_block_ord
     d.kv_block_order = kv_block_order
     d.causal_block_frames = causal_block_frames
     d.sm_scale = float(sm_scale)
+    d.num_iters = int(num_iters)
     d.q_stride = _l.strides3(q)
     d.k_stride = _l.strides3(k)
     d.v_stride = _l.strides3(v)
@@ -60,8 +63,6 @@ def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end
                                sm_scale=None, num_iters=1, grad_only_new_kv=False, heads_per_pass=0):
     """Writes new_k/new_v into k_cache/v_cache[:, start_idx:end_idx] (block order, in place) and
     returns one-iteration Monarch attention of q against the whole cache view."""
-    if num_iters != 1:
-        raise NotImplementedError("num_iters > 1 (the reference's pure-torch refinement) is not built")
     if torch.is_grad_enabled() and (q.requires_grad or new_k.requires_grad or new_v.requires_grad):
         raise NotImplementedError("forward only: call under torch.no_grad()")
     _check4("q", q)
@@ -77,7 +78,7 @@ def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end
     if sm_scale is None:
         sm_scale = q.shape[-1] ** -0.5
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    d = _desc(q, k_cache, v_cache, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1, 0)
+    d = _desc(q, k_cache, v_cache, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1, 0, num_iters)
     nbytes = monarch_workspace_bytes(d, heads_per_pass)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):
@@ -93,8 +94,6 @@ def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block
     block-frames of later causal blocks.  `kv_block_order=True` (no counterpart in the reference) says
     that k, v are a KV-cache view whose rows are already in Monarch block order, e.g. after
     prologue.qk_prologue wrote them."""
-    if num_iters != 1:
-        raise NotImplementedError("num_iters > 1 (the reference's pure-torch refinement) is not built")
     if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
         raise NotImplementedError("forward only: call under torch.no_grad()")
     _check4("q", q)
@@ -114,8 +113,10 @@ def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block
         if block_causal_size % per_block:
             raise ValueError("block_causal_size must align with Monarch block sizes")
         cbf = block_causal_size // per_block
+        if num_iters != 1:
+            raise ValueError("causal currently only supported for num_iters=1")
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    d = _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1 if kv_block_order else 0, cbf)
+    d = _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1 if kv_block_order else 0, cbf, num_iters)
     nbytes = monarch_workspace_bytes(d, heads_per_pass)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):

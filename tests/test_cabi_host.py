@@ -23,13 +23,13 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 9 and set(names) == set(L.SYMBOLS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sfm_version() == 1
+    assert lib.sfm_version() == 2
 
 
 def test_struct_sizes_match_header_layout():
     # int32 x 6, tiling (5 x int32), 2 x int32, float, pad to 8, 12 x int64
     assert C.sizeof(L.Tiling) == 20
-    assert C.sizeof(L.MonarchDesc) == 56 + 12 * 8
+    assert C.sizeof(L.MonarchDesc) == 64 + 12 * 8
     assert C.sizeof(L.DenseDesc) == 32 + 12 * 8
     assert C.sizeof(L.PrologueDesc) == 64 + 8 * 8 + 16
 
@@ -39,7 +39,7 @@ def _desc(**kw):
     d.dtype, d.B, d.H, d.D = L.SFM_BF16, 1, 2, 128
     d.q_tokens, d.kv_tokens = 3 * 30 * 52, 21 * 30 * 52
     d.tiling = L.Tiling(1, 1, 1, 30, 52)
-    d.kv_block_order, d.causal_block_frames, d.sm_scale = 1, 0, 128 ** -0.5
+    d.kv_block_order, d.causal_block_frames, d.sm_scale, d.num_iters = 1, 0, 128 ** -0.5, 1
     for name in ("q_stride", "k_stride", "v_stride", "o_stride"):
         toks = d.kv_tokens if name[0] in "kv" else d.q_tokens
         setattr(d, name, (C.c_int64 * 3)(toks * 256, 256, 128))
@@ -67,10 +67,15 @@ def test_workspace_bytes_accounting():
     # fp32 tensors take the generic path, which keeps its scratch rows in float
     rc, nf32 = _ws(_desc(dtype=L.SFM_F32), 1)
     assert rc == 0 and nf32 == rows * 128 * 4 * 2 + rows * 4
+    # iterated refinement: fp32 Kbar, Y and representatives plus two fp32 scalars per row
+    rc, nit = _ws(_desc(num_iters=3), 1)
+    assert rc == 0 and nit == rows * 128 * 4 * 3 + rows * 4 * 2
 
 
 @pytest.mark.parametrize("kw,code", [
     (dict(dtype=7), -2),
+    (dict(num_iters=0), -3),
+    (dict(num_iters=2, causal_block_frames=1, kv_block_order=0, q_tokens=21 * 30 * 52), -9),
     (dict(D=100), -3),
     (dict(q_tokens=1000), -3),
     (dict(kv_tokens=30 * 52 + 1), -3),

@@ -185,5 +185,3 @@ def test_host_argument_errors():
         mattn.monarch_attn(q.cpu(), kc, kc, 1, 1, 1, 3, 20)
     with pytest.raises(ValueError):
         mattn.monarch_attn(q, kc, kc, 1, 1, 1, 3, 20, block_causal_size=60)                  # needs Skv == Sq
-    with pytest.raises(NotImplementedError):
-        mattn.monarch_attn(q, kc, kc, 1, 1, 1, 3, 20, num_iters=4)

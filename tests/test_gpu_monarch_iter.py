@@ -1,0 +1,94 @@
+"""GPU parity of the iterated-refinement Monarch path (num_iters > 1) through the C ABI, against the
+reference's own golden vectors (monarch_attn_slow, tests/golden/) and the CPU oracle.
+
+Tolerances: fp32 tensors <= 2e-5 max-abs (fp32 kernels against a float64 oracle, several chained
+softmaxes); 16-bit tensors the reference's atol = rtol = 1e-2 (bf16) / 1e-3 (fp16)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import self_forcing_amd as sfa
+from gpu_util import assert_close_16bit, max_abs, randn
+from oracle import monarch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+mattn = sfa.monarch_attn
+GOLD = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "monarch_reference_vectors.npz"))
+
+
+def _golden_inputs(ci):
+    seed, B, a, f, b1, b2, H, D = (int(x) for x in GOLD[f"case{ci}_meta"])
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, a, b1, b2, H, D, generator=g, dtype=torch.float64)
+    k = torch.randn(B, f, b1, b2, H, D, generator=g, dtype=torch.float64)
+    v = torch.randn(B, f, b1, b2, H, D, generator=g, dtype=torch.float64)
+    return q, k, v, float(GOLD[f"case{ci}_scale"]), (B, a, f, b1, b2, H, D)
+
+
+@pytest.mark.parametrize("ci", [0, 1, 2])
+@pytest.mark.parametrize("n", [2, 3, 8])
+def test_golden_vectors_of_the_reference_refinement(ci, n):
+    """With f_tied = h_reduce = w_reduce = 1 and h = b1, w = b2 token order is block order, so the stored
+    blocked tensors are the token-order inputs reshaped."""
+    q, k, v, s, (B, a, f, b1, b2, H, D) = _golden_inputs(ci)
+    tok = lambda t: t.reshape(B, -1, H, D).float().to(DEV)
+    out = mattn.monarch_attn(tok(q), tok(k), tok(v), 1, 1, 1, b1, b2, sm_scale=s, num_iters=n)
+    gold = torch.from_numpy(GOLD[f"case{ci}_slow{n}"]).reshape(B, -1, H, D)
+    assert max_abs(out, gold) < 2e-5
+
+
+@pytest.mark.parametrize("tiling,h,w", [((1, 1, 1), 6, 20), ((1, 2, 1), 6, 20), ((3, 1, 1), 4, 12), ((1, 1, 2), 5, 8)])
+@pytest.mark.parametrize("n", [2, 4])
+def test_fp32_tilings_against_oracle(tiling, h, w, n):
+    F = 3
+    q = randn((2, F * h * w, 2, 64), 70, torch.float32)
+    k, v = (randn((2, 2 * F * h * w, 2, 64), 71 + i, torch.float32) for i in range(2))
+    ref = monarch.monarch_attn(q, k, v, *tiling, h, w, num_iters=n)
+    out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), *tiling, h, w, num_iters=n)
+    assert max_abs(out, ref) < 2e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_16bit_inputs_and_cache_entry_point(dtype):
+    """Cache holds 2 of 3 frames, the third arrives with the call; rows are in block order (h_reduce = 2)."""
+    h, w, H, D = 6, 20, 3, 128
+    q = randn((1, h * w, H, D), 80, dtype)
+    k, v = (randn((1, 3 * h * w, H, D), 81 + i, dtype) for i in range(2))
+    ref = monarch.monarch_attn(q, k, v, 1, 2, 1, h, w, num_iters=3, dtype=torch.float32)
+    kc, vc = torch.zeros(1, 3 * h * w, H, D, dtype=dtype, device=DEV), torch.zeros(1, 3 * h * w, H, D, dtype=dtype, device=DEV)
+    mattn.monarch_attn_with_kv_cache(q.to(DEV), kc, vc, k[:, :2 * h * w].to(DEV), v[:, :2 * h * w].to(DEV), 0, 2 * h * w,
+                                     1, 2, 1, h, w)
+    out = mattn.monarch_attn_with_kv_cache(q.to(DEV), kc, vc, k[:, 2 * h * w:].to(DEV), v[:, 2 * h * w:].to(DEV),
+                                           2 * h * w, 3 * h * w, 1, 2, 1, h, w, num_iters=3)
+    assert_close_16bit(out, ref, dtype)
+
+
+def test_one_and_many_iterations_share_limits():
+    """num_iters == 1 stays on the fast path (no 1/(1 + 1e-6) factor); the first refinement pass of the iterated
+    path carries it, as the reference's pure-torch function does."""
+    q, k, v = (randn((1, n * 4 * 16, 2, 64), 90 + i, torch.float32) for i, n in enumerate((2, 3, 3)))
+    one = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, 4, 16, num_iters=1)
+    ref1 = monarch.monarch_attn(q, k, v, 1, 1, 1, 4, 16)
+    assert max_abs(one, ref1) < 1e-5
+    with pytest.raises(ValueError):
+        mattn.monarch_attn(q.to(DEV), q.to(DEV), q.to(DEV), 1, 1, 1, 4, 16, block_causal_size=64, num_iters=2)
+
+
+@pytest.mark.parametrize("f_tied", [1, 3])
+def test_c2_shape_two_iterations_bf16(f_tied):
+    """Full 480p sizes (3 query frames, 21 cached frames of 30 x 52 tokens), 2 heads, frame-wise blocks
+    (b1 = 30) and three frames tied per block (b1 = 90, query rows taken in chunks): against the oracle on
+    head 0 and through the size-independent property that constant V gives constant output."""
+    a, f, b1, b2, H, D = 3, 21, 30, 52, 2, 128
+    q = randn((1, a * b1 * b2, H, D), 95, torch.bfloat16)
+    k = randn((1, f * b1 * b2, H, D), 96, torch.bfloat16)
+    v = randn((1, f * b1 * b2, H, D), 97, torch.bfloat16)
+    out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), f_tied, 1, 1, b1, b2, num_iters=2)
+    ref = monarch.monarch_attn(q[:, :, :1], k[:, :, :1], v[:, :, :1], f_tied, 1, 1, b1, b2, num_iters=2, dtype=torch.float32)
+    assert_close_16bit(out[:, :, :1], ref, torch.bfloat16)
+    vc = torch.full_like(v, 0.75)
+    outc = mattn.monarch_attn(q.to(DEV), k.to(DEV), vc.to(DEV), f_tied, 1, 1, b1, b2, num_iters=2)
+    assert max_abs(outc, torch.full_like(q, 0.75)) < 4e-3

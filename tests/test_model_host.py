@@ -98,8 +98,7 @@ def test_env_flags_are_read_like_the_reference(monkeypatch):
     f0, f1 = cm.AttentionFlags(0), cm.AttentionFlags(1)
     assert f0.use_framewise and f0.h_reduce == 2 and f0.disable_monarch and not f1.disable_monarch
     monkeypatch.setenv("MONARCH_ATTN_NUM_ITERS", "8")
-    with pytest.raises(NotImplementedError):
-        cm.AttentionFlags(1)
+    assert cm.AttentionFlags(1).num_iters == 8
 
 
 def test_patchify_equals_conv3d_and_unpatchify_inverts():
