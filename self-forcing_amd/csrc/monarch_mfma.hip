@@ -44,14 +44,14 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     constexpr int DP = D / 2;    // dword columns of a K/V row
     extern __shared__ __attribute__((aligned(16))) uint16_t lds_all[];
 
-    // A workgroup is `p.s1_groups` independent wave groups that share nothing but the barriers: group g
-    // works on kv block-frame f0 + g, f0 + g + groups, ... with its own LDS tiles.  Two groups of 5 waves
-    // put 3,3,2,2 waves on the four SIMDs, which one group of 5 cannot (waves go to SIMDs round-robin).
-    const int nthreads = blockDim.x / p.s1_groups;        // threads of one group
-    const int grp = threadIdx.x / nthreads;
+    // A workgroup is `p.s1_groups` independent wave groups that share nothing but the barriers, each with
+    // its own LDS tiles.  Two groups of 5 waves put 3,3,2,2 waves on the four SIMDs, which one group of 5
+    // cannot (waves go to SIMDs round-robin).
+    const int G = p.s1_groups;
+    const int nthreads = blockDim.x / G;                  // threads of one group
+    const int grp = __builtin_amdgcn_readfirstlane(threadIdx.x / nthreads);
     const int tid = threadIdx.x - grp * nthreads;
-    const int nwaves = nthreads >> 6;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int m = lane & 31;
     const int hf = lane >> 5;
@@ -61,103 +61,88 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     uint16_t* const lds_kt = lds + 64 * L::kRowPitch;                // [D][72]
     uint16_t* const lds_vt = lds_kt + D * L::kTPitch;                // [D][72]
 
-    // Workgroup = (unit, a-chunk, key block row k, range of kv block-frames f).  The query rows
-    // Q[a, k, :, :] of the chunk depend on k only, so they are loaded once and stay in registers for
-    // every f of the range.  Workgroups are handed to the 8 XCDs round-robin (id % 8); give each XCD a
-    // contiguous range of the logical order.
-    const int per_xcd = gridDim.x >> 3;
-    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= p.s1_total) return;
-    const int nfs = (p.nf + p.f_per_wg - 1) / p.f_per_wg;
-    const int fs = logical % nfs;
-    const int kz = logical / nfs;
-    const int k = kz % p.b1;
-    const int z = kz / p.b1;
-    const int ul = z / p.n_achunks;                       // unit within this pass
-    const int a0 = (z % p.n_achunks) * p.a_chunk;
-    const int a_cnt = min(p.a_chunk, p.na - a0);
-    const int unit = p.unit0 + ul;
-    const int b = unit / p.H, h = unit % p.H;
-    const int f0 = fs * p.f_per_wg;
-    int f1 = min(f0 + p.f_per_wg, p.nf);
-    if (p.causal) f1 = min(f1, ((a0 + a_cnt - 1) / p.causal + 1) * p.causal);   // later block-frames are masked for every a
-    if (f0 >= f1) return;
-
-    const int b2 = p.b2;
-    const int ncols = a_cnt * b2;
-    const int NT = b2 > 32 ? 2 : 1;                       // 32-row tiles of the key axis l
-    const bool tile_ok = wave * 32 < ncols;
-
-    // Uniform 64-bit bases; everything that varies per lane is a 32-bit element offset from them
-    // (the host checks that each tensor and the scratch of one pass stay below 2^31 elements).
-    const uint16_t* qg = (const uint16_t*)p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[2];
-    const uint16_t* kg = (const uint16_t*)p.k + (int64_t)b * p.ks[0] + (int64_t)h * p.ks[2];
-    const uint16_t* vg = (const uint16_t*)p.v + (int64_t)b * p.vs[0] + (int64_t)h * p.vs[2];
-    const uint32_t qs1 = (uint32_t)p.qs[1], ks1 = (uint32_t)p.ks[1];
-
-    // column owned by this lane in the logits/contraction phase
-    const int cg = wave * 32 + m;
-    const bool col_ok = cg < ncols;
-    const int ca = a0 + (col_ok ? cg / b2 : 0);
-    const int cj = col_ok ? cg % b2 : 0;
-
-    // logits operand (B): this lane's query row Q[ca, k, cj, 16 ds + 8 hf + 0..7]
-    u32x4 qb[DS];
-    {
-        const uint16_t* qrow = qg + ((uint32_t)(p.qmap.row(ca, k) + cj) * qs1 + 8 * hf);
-#pragma unroll
-        for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
+    // Work items are K/V tiles t = ((ul * b1 + k) * n_achunks + ac) * nf + f, i.e. one kv block row (f, k) of
+    // one unit against the query rows Q[a, k, :, :] of one chunk of query block-frames.  The launch has one
+    // workgroup per CU and every workgroup takes an equal contiguous share of the tile list (its groups
+    // alternate within the share), so no round of workgroups is left partly filled.  The query operands
+    // stay in registers while consecutive tiles differ in f only.
+    const int T = p.s1_total;
+    const int t0 = (int)((int64_t)blockIdx.x * T / gridDim.x);
+    const int t1 = (int)((int64_t)(blockIdx.x + 1) * T / gridDim.x);
+    const int rounds = (t1 - t0 + G - 1) / G;
+    const int mine = (t1 - t0 - grp + G - 1) / G;         // tiles of this group: t0 + grp, t0 + grp + G, ...
+    if (mine <= 0) {                                      // still joins the barriers of the other group
+        for (int r = 0; r < rounds; ++r) {
+            lds_barrier();
+            lds_barrier();
+        }
+        return;
     }
 
-    // Output rows are stored straight from the accumulators: after one cross-half swap lane (c, hf) holds
-    // 8 consecutive head-dim elements of row c.  BYTE offset of this lane's row from the (uniform)
-    // scratch row of (f, k), ~0u = no row.
-    const uint32_t crow = col_ok ? ((uint32_t)(ca * b2 + cj) * p.ws_aj * D + 8 * hf) * 2 : ~0u;
-    const uint32_t cloff = (uint32_t)(ca * b2 + cj) * p.ws_aj * 4;     // byte offset into cl, same convention
-    const uint32_t ubase = (uint32_t)ul * p.ws_unit + (uint32_t)k * p.ws_row;   // scratch row of (unit, k), f = 0
+    const int b2 = p.b2;
+    const int NT = b2 > 32 ? 2 : 1;                       // 32-row tiles of the key axis l
+    const uint32_t qs1 = (uint32_t)p.qs[1], ks1 = (uint32_t)p.ks[1];
     const uint32_t fstep = (uint32_t)p.b1 * p.ws_row;     // scratch rows between consecutive f
 
+    struct Tile {
+        int f, k, ul, a0, ncols;
+    };
+    auto decode = [&](int t) {
+        Tile x;
+        x.f = t % p.nf;
+        int r = t / p.nf;
+        const int ac = r % p.n_achunks;
+        r /= p.n_achunks;
+        x.k = r % p.b1;
+        x.ul = r / p.b1;
+        x.a0 = ac * p.a_chunk;
+        x.ncols = min(p.a_chunk, p.na - x.a0) * b2;
+        return x;
+    };
+
     // staging tasks: (sh = 2*s + hf', dword column pc); 8 rows perm_row(s, hf', 0..7) each.  With
-    // D = 128 the 64 lanes of a wave share sh, which makes the row-validity tests scalar branches.
+    // D = 128 the 64 lanes of a wave share sh.  A thread without a second task of its own repeats
+    // another thread's (same data to the same LDS words), so that every thread issues the same loads.
     constexpr int kTasks = 8 * DP;
     constexpr int kMaxTask = 2;                             // host launches >= kTasks/2 threads
     const int ntask = (kTasks + nthreads - 1) / nthreads;
     if (ntask > kMaxTask) return;                           // (checked on the host as well)
     uint32_t pk[kMaxTask][8], pv[kMaxTask][8];
-    int tsh[kMaxTask];                                      // sh of the task, 8 = none
+    int tsh[kMaxTask];
     uint32_t tcol[kMaxTask];                                // byte offset of dword column pc
 #pragma unroll
     for (int t = 0; t < kMaxTask; ++t) {
-        int task = tid + t * nthreads;
-        bool ok = t < ntask && task < kTasks;
-        int sh = ok ? task / DP : 8;
+        int task = (tid + t * nthreads) % kTasks;
+        int sh = task / DP;
         if (DP == 64) sh = __builtin_amdgcn_readfirstlane(sh);
         tsh[t] = sh;
         tcol[t] = (uint32_t)(task % DP) * 4;
     }
 
-    auto prefetch = [&](int f) {
-        const uint32_t krow0 = (uint32_t)p.kmap.row(f, k);            // uniform
+    // Rows past the end of a short tile (l >= b2) load row b2 - 1 again; their logits are masked below.
+    auto prefetch = [&](const Tile& x) {
+        const int unit = p.unit0 + x.ul;
+        const int b = unit / p.H, h = unit % p.H;
+        const char* kg = (const char*)p.k + ((int64_t)b * p.ks[0] + (int64_t)h * p.ks[2]) * 2;
+        const char* vg = (const char*)p.v + ((int64_t)b * p.vs[0] + (int64_t)h * p.vs[2]) * 2;
+        const uint32_t krow0 = (uint32_t)p.kmap.row(x.f, x.k);        // uniform
 #pragma unroll
         for (int t = 0; t < kMaxTask; ++t) {
+            if (t < ntask) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int l = perm_row(tsh[t] >> 1, tsh[t] & 1, e);
-                uint32_t kk = 0, vv = 0;
-                if (tsh[t] < 8 && l < b2) {
+                for (int e = 0; e < 8; ++e) {
+                    const int l = min(perm_row(tsh[t] >> 1, tsh[t] & 1, e), b2 - 1);
                     const size_t rowb = (size_t)((krow0 + (uint32_t)l) * ks1) * 2;
-                    kk = *(const uint32_t*)((const char*)kg + rowb + tcol[t]);
-                    vv = *(const uint32_t*)((const char*)vg + rowb + tcol[t]);
+                    pk[t][e] = *(const uint32_t*)(kg + rowb + tcol[t]);
+                    pv[t][e] = *(const uint32_t*)(vg + rowb + tcol[t]);
                 }
-                pk[t][e] = kk;
-                pv[t][e] = vv;
             }
         }
     };
     auto commit = [&]() {
 #pragma unroll
         for (int t = 0; t < kMaxTask; ++t) {
-            if (tsh[t] < 8) {
+            if (t < ntask) {
                 const int pc = tcol[t] >> 2, sh = tsh[t];
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -183,20 +168,66 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 
     const float sc2 = p.scale * kLog2e;
 
-    const int G = p.s1_groups;
-    if (f0 + grp < f1) prefetch(f0 + grp);
-    for (int fb = f0; fb < f1; fb += G) {
-        const int f = fb + grp;
-        const bool has_f = f < f1;       // a group may run out of block-frames one round early; it still joins the barriers
+    // Everything from the logits to the output stores runs without a branch, and a lane whose column
+    // index is past the chunk's last column works on that last column again (same values to the same
+    // addresses).  The number of stores between a prefetch and the wait for it is then the same on
+    // every path, so that wait leaves the stores in flight instead of draining them.
+    u32x4 qb[DS];                                          // logits operand (B): this lane's query row
+    uint32_t crow = 0;                                     // byte offset of this lane's scratch row in its (f, k) slab
+    uint32_t cloff = 0;                                    // same for cl
+    int qkey = -1;
+
+    // Makes the compiler wait here for loads into the given registers.  The waits it places are the most
+    // cautious over all paths that reach a use; closing a load's wait on the rarely taken path (kernel
+    // entry, change of query rows) keeps the wait in the steady-state loop as loose as that path allows.
+    auto settle4 = [](uint32_t& a, uint32_t& b, uint32_t& c, uint32_t& d) { asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d)); };
+
+    Tile cur = decode(t0 + grp), nxt = cur;
+    prefetch(cur);
+#pragma unroll
+    for (int t = 0; t < kMaxTask; ++t) {
+        settle4(pk[t][0], pk[t][1], pk[t][2], pk[t][3]);
+        settle4(pk[t][4], pk[t][5], pk[t][6], pk[t][7]);
+        settle4(pv[t][0], pv[t][1], pv[t][2], pv[t][3]);
+        settle4(pv[t][4], pv[t][5], pv[t][6], pv[t][7]);
+    }
+    for (int r = 0; r < rounds; ++r) {
+        const bool fresh = r < mine;     // in its last round a group may have no tile left: it repeats its previous one
         lds_barrier();                   // previous iteration finished reading the tiles
-        if (has_f) commit();
-        if (f + G < f1) prefetch(f + G);
+        if (fresh) {
+            cur = nxt;
+            commit();
+        }
+        const int key = (cur.ul * p.b1 + cur.k) * p.n_achunks + cur.a0;
+        if (key != qkey) {
+            qkey = key;
+            const int unit = p.unit0 + cur.ul;
+            const int b = unit / p.H, h = unit % p.H;
+            const uint16_t* qg = (const uint16_t*)p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[2];
+            const int cg = min(wave * 32 + m, cur.ncols - 1);
+            const int cl_a = cg / b2;
+            const int cj = cg - cl_a * b2;
+            const int ca = cur.a0 + cl_a;
+            const uint16_t* qrow = qg + ((uint32_t)(p.qmap.row(ca, cur.k) + cj) * qs1 + 8 * hf);
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds) asm volatile("" : "+v"(qb[ds]));
+            crow = ((uint32_t)(ca * b2 + cj) * p.ws_aj * D + 8 * hf) * 2;
+            cloff = (uint32_t)(ca * b2 + cj) * p.ws_aj * 4;
+        }
+        {
+            // the tile after this one; past the end of the share the current tile is loaded again and dropped
+            const int tn = t0 + grp + (r + 1) * G;
+            nxt = decode(tn < t1 ? tn : t0 + grp + (mine - 1) * G);
+            prefetch(nxt);
+        }
         lds_barrier();                   // K/V tiles visible
 
+        const uint32_t srow = (uint32_t)cur.ul * p.ws_unit + (uint32_t)cur.k * p.ws_row + (uint32_t)cur.f * fstep;
+
         u32x4 pb[4];                     // R^T as B operands, 16 contraction rows per step
-        float inv_l = 0.f;
-        const bool tile_active = has_f && tile_ok;
-        if (tile_active) {
+        {
             f32x16 s[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
@@ -238,7 +269,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 }
             sum = xhalf_sum(sum);
             ent = xhalf_sum(ent);
-            inv_l = 1.f / sum;
+            const float inv_l = 1.f / sum;
             // R = e / sum is rounded to 16 bit once, as the reference's right factor is
 #pragma unroll
             for (int st = 0; st < 4; ++st) {
@@ -248,8 +279,8 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 pb[st].z = pack2<E>(s[t][v0 + 4] * inv_l, s[t][v0 + 5] * inv_l);
                 pb[st].w = pack2<E>(s[t][v0 + 6] * inv_l, s[t][v0 + 7] * inv_l);
             }
-            if (col_ok && hf == 0)                 // sum_l R log2 R
-                *(float*)((char*)p.cl + (size_t)(ubase + (uint32_t)f * fstep) * 4 + cloff) = ent * inv_l - (mx + log2f(sum));
+            // sum_l R log2 R (both halves of a column hold, and store, the same value)
+            *(float*)((char*)p.cl + (size_t)srow * 4 + cloff) = ent * inv_l - (mx + log2f(sum));
         }
         // contractions with K^T then V^T, 32 head-dim columns at a time.  A 32 x 32 accumulator tile holds,
         // per lane (column c, half hf), head-dim 8g + 4hf + 0..3 for g = 0..3; swapping the g-odd dwords of the
@@ -258,31 +289,29 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #pragma unroll
         for (int which = 0; which < 2; ++which) {
             const uint16_t* tbase = which == 0 ? lds_kt : lds_vt;
-            char* og = (char*)(which == 0 ? p.kbar : p.y) + (size_t)(ubase + (uint32_t)f * fstep) * (D * 2);
+            char* og = (char*)(which == 0 ? p.kbar : p.y) + (size_t)srow * (D * 2);
 #pragma unroll
             for (int dt = 0; dt < D / 32; ++dt) {
-                if (tile_active) {
-                    f32x16 acc;
+                f32x16 acc;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-                    const uint16_t* arow = tbase + (32 * dt + m) * L::kTPitch + 8 * hf;
+                for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+                const uint16_t* arow = tbase + (32 * dt + m) * L::kTPitch + 8 * hf;
 #pragma unroll
-                    for (int st = 0; st < 4; ++st) {
-                        if (st < 2 * NT) {
-                            u32x4 a = *(const u32x4*)(arow + 16 * st);
-                            acc = E::mfma32(a, pb[st], acc);
-                        }
+                for (int st = 0; st < 4; ++st) {
+                    if (st < 2 * NT) {
+                        u32x4 a = *(const u32x4*)(arow + 16 * st);
+                        acc = E::mfma32(a, pb[st], acc);
                     }
+                }
 #pragma unroll
-                    for (int gp = 0; gp < 2; ++gp) {
-                        const int g0 = 2 * gp, g1 = 2 * gp + 1;
-                        auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 0], acc[4 * g0 + 1]),
-                                                                   pack2<E>(acc[4 * g1 + 0], acc[4 * g1 + 1]), false, false);
-                        auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 2], acc[4 * g0 + 3]),
-                                                                   pack2<E>(acc[4 * g1 + 2], acc[4 * g1 + 3]), false, false);
-                        u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
-                        if (crow != ~0u) *(u32x4*)(og + crow + (32 * dt + 16 * gp) * 2) = w;
-                    }
+                for (int gp = 0; gp < 2; ++gp) {
+                    const int g0 = 2 * gp, g1 = 2 * gp + 1;
+                    auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 0], acc[4 * g0 + 1]),
+                                                               pack2<E>(acc[4 * g1 + 0], acc[4 * g1 + 1]), false, false);
+                    auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 2], acc[4 * g0 + 3]),
+                                                               pack2<E>(acc[4 * g1 + 2], acc[4 * g1 + 3]), false, false);
+                    u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+                    *(u32x4*)(og + crow + (32 * dt + 16 * gp) * 2) = w;
                 }
             }
         }
@@ -493,12 +522,24 @@ bool monarch_mfma_supported(int dtype, int D, int b2) {
     return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 >= 1 && b2 <= 64;
 }
 
+static int cu_count() {
+    static thread_local int cached_dev = -1, cached = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (dev != cached_dev) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached = n;
+        cached_dev = dev;
+    }
+    return cached;
+}
+
 template <class E, int D>
 static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const StepEvents* ev) {
     const int ncols = a.a_chunk * a.b2;
     const int ntiles = (ncols + 31) / 32;
     const int nwaves = ntiles < 4 ? 4 : ntiles;   // at least 4 waves so that K/V staging is <= 2 tasks per thread
-    const int nfs = (a.nf + a.f_per_wg - 1) / a.f_per_wg;
     if (ntiles < 1 || nwaves > 8 || (8 * (D / 2) + nwaves * 64 - 1) / (nwaves * 64) > 2) {
         set_error("internal: step-1 launch shape (a_chunk=%d, b2=%d)", a.a_chunk, a.b2);
         return SFM_ERR_UNSUPPORTED;
@@ -514,9 +555,12 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const 
         }
     }
     MonarchArgs a1 = a;
-    a1.s1_total = nfs * a.b1 * nunits * a.n_achunks;
+    a1.s1_total = a.nf * a.b1 * nunits * a.n_achunks;
     a1.s1_groups = groups;
-    dim3 g1((a1.s1_total + 7) / 8 * 8);
+    // one workgroup per CU (a CU holds one: 3 waves per SIMD), fewer when there are not two tiles for each
+    int wgs = a.s1_wgs > 0 ? a.s1_wgs : cu_count();
+    if (wgs > (a1.s1_total + groups - 1) / groups) wgs = (a1.s1_total + groups - 1) / groups;
+    dim3 g1(wgs);
     if (ev) (void)hipEventRecord(ev->ev[0], stream);
     hipLaunchKernelGGL((monarch_step1_kernel<E, D>), g1, dim3(nwaves * 64 * groups), lds1, stream, a1);
     if (ev) (void)hipEventRecord(ev->ev[1], stream);

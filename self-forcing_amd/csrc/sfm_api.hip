@@ -267,10 +267,10 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
     a.n_achunks = (pl.na + a_max - 1) / a_max;
     a.a_chunk = (pl.na + a.n_achunks - 1) / a.n_achunks;
     a.n_achunks = (pl.na + a.a_chunk - 1) / a.a_chunk;
-    a.f_per_wg = pl.nf < 7 ? pl.nf : 7;
-    if (const char* e = getenv("SFM_F_PER_WG")) {          // tuning override: kv block-frames per step-1 workgroup
+    a.s1_wgs = 0;
+    if (const char* e = getenv("SFM_S1_WGS")) {            // tuning override: step-1 workgroups (default one per CU)
         int v = atoi(e);
-        if (v >= 1) a.f_per_wg = v < pl.nf ? v : pl.nf;
+        if (v >= 1 && v <= 65535) a.s1_wgs = v;
     }
     for (int u0 = 0; u0 < pl.units; u0 += upp) {
         const int n = pl.units - u0 < upp ? pl.units - u0 : upp;

@@ -143,9 +143,9 @@ struct MonarchArgs {
     int64_t qs[3], ks[3], vs[3], os[3];
     int a_chunk;     // query block-frames per step-1 workgroup
     int n_achunks;
-    int f_per_wg;    // kv block-frames per step-1 workgroup
+    int s1_wgs;      // step-1 workgroups, 0 = one per CU (tuning override)
     int s1_groups;   // wave groups per step-1 workgroup
-    int s1_total;    // step-1 workgroups that have work (the grid is padded to a multiple of 8)
+    int s1_total;    // step-1 work items: (unit, k, a-chunk, f) tiles
 };
 
 // Optional timing hooks: ev[0] is recorded before step 1, ev[1] between the steps, ev[2] after step 2.
