@@ -54,6 +54,9 @@ class OracleOps:
         nf = gate.shape[1]
         return x + (y.unflatten(1, (nf, x.shape[1] // nf)) * gate).flatten(1, 2)
 
+    def linear_gelu(self, x, linear):
+        return torch.nn.functional.gelu(linear(x), approximate='tanh')
+
     def rms_norm(self, x, weight, eps):
         xf = x.float()
         return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)).type_as(x) * weight

@@ -64,6 +64,13 @@ class HipAttentionOps:
     def rms_norm(self, x, weight, eps):
         return _blk.rms_norm(x, weight, eps)
 
+    def linear_gelu(self, x, linear):
+        """GELU(tanh)(x W^T + b) with the activation applied in the GEMM's epilogue (hipBLASLt through
+        torch's addmm-with-activation); the reference runs Linear and nn.GELU(approximate='tanh') apart
+        (model.py:648-650)."""
+        out = torch._addmm_activation(linear.bias, x.reshape(-1, x.shape[-1]), linear.weight.t(), use_gelu=True)
+        return out.view(*x.shape[:-1], out.shape[-1])
+
 
 def _env_int(name, default):
     return int(os.getenv(name, str(default)))
@@ -146,8 +153,10 @@ def cache_step(kv_cache, current_start, num_new, frame_seqlen, local_attn_size, 
 def cache_commit(kv_cache, current_end, local_end):
     """causal_model.py:1102-1103 (the reference stores the view-relative local end)."""
     kv_cache["_global_end"], kv_cache["_local_end"] = current_end, local_end
-    kv_cache["global_end_index"].fill_(current_end)
-    kv_cache["local_end_index"].fill_(local_end)
+    if kv_cache.get("_written") != (current_end, local_end):     # unchanged when a chunk is re-run at another timestep
+        kv_cache["global_end_index"].fill_(current_end)
+        kv_cache["local_end_index"].fill_(local_end)
+        kv_cache["_written"] = (current_end, local_end)
 
 
 class CausalWanSelfAttention(nn.Module):
@@ -269,7 +278,7 @@ class CausalWanAttentionBlock(nn.Module):
         else:
             xn = ops.ln_affine(x, self.norm3.weight, self.norm3.bias, self.eps)
         x = ops.gate_residual(x, self.cross_attn(xn, context, crossattn_cache))
-        y = self.ffn(ops.ln_modulate(x, e[4], e[3], self.eps))
+        y = self.ffn[2](ops.linear_gelu(ops.ln_modulate(x, e[4], e[3], self.eps), self.ffn[0]))
         return ops.gate_residual(x, y, e[5])
 
 

@@ -125,6 +125,7 @@ class CausalInferencePipeline(nn.Module):
             c["global_end_index"] = torch.tensor([0], dtype=torch.long, device=device)
             c["local_end_index"] = torch.tensor([0], dtype=torch.long, device=device)
             c["_global_end"] = c["_local_end"] = 0
+            c.pop("_written", None)
 
     def _next_seed(self):
         if self.seeds is None:
