@@ -80,6 +80,28 @@ int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, 
 int sfm_monarch_fwd_timed(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
                           void* workspace, size_t workspace_bytes, void* stream, float* step1_ms, float* step2_ms);
 
+/* Backward of sfm_monarch_fwd (num_iters == 1).  Replaces the Triton kernels _z_bwd_preprocess, _z_bwd,
+ * _al_cl_y_bwd and their orchestration in _attention_with_cache.backward / _attention_no_cache.backward
+ * (monarch_attn.py:852-886, 1034-1222, 403-596, 1326-1470, 1566-1693).
+ *   fwd                 the forward descriptor; o_stride describes `dout`
+ *   dq                  float32 [B, q_tokens, H, D] (the reference returns grad_q in float32, :1470)
+ *   dk, dv              tensor dtype, [B, (kv_grad_frame_end - kv_grad_frame_start) * b1 * b2, H, D], rows in the
+ *                       order of k: token order, or block order when fwd.kv_block_order = 1
+ *   kv_grad_frame_*     kv block-frames whose gradients are produced; a proper sub-range is the reference's
+ *                       grad_only_new_kv (:1364-1374) and needs block order
+ * Everything is recomputed from q, k, v (the forward saves nothing but its inputs). */
+typedef struct sfm_monarch_bwd_desc {
+    sfm_monarch_desc fwd;
+    int64_t dq_stride[3];
+    int64_t dkv_stride[3];
+    int32_t kv_grad_frame_start;
+    int32_t kv_grad_frame_end;
+} sfm_monarch_bwd_desc;
+
+int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t heads_per_pass, size_t* bytes);
+int sfm_monarch_bwd(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* dout,
+                    float* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Writes new_k/new_v [B, n_new, H, D] (token order) into k_cache/v_cache[:, start_idx:end_idx]
  * in Monarch block order.  Replaces monarch_attn.py:1784-1785 + 1230-1231.
  * strides: new_stride for new_k and new_v, cache_stride for both caches. */

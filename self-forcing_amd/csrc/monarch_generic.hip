@@ -383,6 +383,281 @@ int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_ite
     return launch_iter_t<F16>(a, nunits, num_iters, stream);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Backward of the one-iteration forward (replaces _z_bwd_preprocess, _z_bwd, _al_cl_y_bwd,
+// wan/modules/monarch_attn.py:852-886, 1034-1222, 403-596, and the orchestration :1326-1470, 1566-1693), fp32.
+// With S1 = s q.k, R = softmax_l S1, Kbar = R K, Y = R V, c = sum_l R ln R, S2 = s q.Kbar - c, L = softmax_(f,k) S2,
+// O = L Y and a given dO:
+//   dLm[i,r] = dO_i . Y_r            dS2 = L (dLm - sum_r L dLm)
+//   dY_r = sum_i L[i,r] dO_i         dKbar_r = s sum_i dS2[i,r] q_i       dc_r = - sum_i dS2[i,r]
+//   dQ(a,i,j) = s sum_r dS2[i,r] Kbar_r                                              (left factor)
+//   dR_l = dKbar . K_l + dY . V_l + dc (ln R_l + 1)        dS1 = R (dR - sum_l R dR)
+//   dQ(a,k,j) += s sum_f sum_l dS1_l K_l     dK_l += R_l dKbar + s dS1_l q     dV_l += R_l dY   (right factor)
+// Three launches per pass: the forward's step 1 (Kbar, Y, c into the scratch), the left-factor kernel
+// (workgroup = (unit, a, j); writes dKbar, dY, dc to the scratch and its part of dQ), the right-factor
+// kernel (workgroup = (unit, k), which owns the rows dQ[a, k, :] and the tiles dK/dV[f, k, :], so that
+// nothing needs an atomic).  The "+ 1" drops out of the softmax backward.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void monarch_bwd_left(MonarchBwdArgs g, int ic) {
+    extern __shared__ float sm[];
+    const MonarchArgs& p = g.p;
+    const int D = p.D, b2 = p.b2, b1 = p.b1, DP = D + 1;
+    const int a = blockIdx.x / b2, j = blockIdx.x % b2;
+    const int ul = blockIdx.y;
+    const int unit = p.unit0 + ul;
+    const int b = unit / p.H, h = unit % p.H;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const int f_lim = p.causal ? min(p.nf, (a / p.causal + 1) * p.causal) : p.nf;
+    const int R = f_lim * b1;
+    const int RP = p.nf * b1;          // row pitch of the LDS arrays
+    const float sc2 = p.scale * kLog2e;
+    float* qs = sm;                    // [ic][D+1]   q_i
+    float* dos = qs + ic * DP;         // [ic][D+1]   dO_i
+    float* S = dos + ic * DP;          // [ic][RP]    logits (log2 units), then L
+    float* G = S + (size_t)ic * RP;    // [ic][RP]    dLm, then dS2
+
+    const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj;
+    const int64_t rsd = p.ws_row;
+    const float* kbar = (const float*)p.kbar + blk * D;
+    const float* yw = (const float*)p.y + blk * D;
+    const float* cl = p.cl + blk;
+    float* dkbar = g.dkbar + blk * D;
+    float* dy = g.dy + blk * D;
+    float* dcl = g.dcl + blk;
+
+    for (int i0 = 0; i0 < b1; i0 += ic) {
+        const int ni = b1 - i0 < ic ? b1 - i0 : ic;
+        __syncthreads();
+        for (int e = tid; e < ni * D; e += nt) {
+            const int i = e / D, d = e % D;
+            const int64_t tok = p.qmap.row(a, i0 + i) + j;
+            qs[i * DP + d] = Ld<T>::get(p.q, (int64_t)b * p.qs[0] + tok * p.qs[1] + (int64_t)h * p.qs[2] + d);
+            dos[i * DP + d] = Ld<T>::get(g.dout, (int64_t)b * g.dos[0] + tok * g.dos[1] + (int64_t)h * g.dos[2] + d);
+        }
+        __syncthreads();
+        for (int r = tid; r < R; r += nt) {
+            float as[kIterRows], al[kIterRows];
+#pragma unroll
+            for (int i = 0; i < kIterRows; ++i) as[i] = al[i] = 0.f;
+            const float* krow = kbar + (int64_t)r * rsd * D;
+            const float* yrow = yw + (int64_t)r * rsd * D;
+            for (int d = 0; d < D; ++d) {
+                const float kv = krow[d], yv = yrow[d];
+#pragma unroll
+                for (int i = 0; i < kIterRows; ++i)
+                    if (i < ni) {
+                        as[i] += qs[i * DP + d] * kv;
+                        al[i] += dos[i * DP + d] * yv;
+                    }
+            }
+            const float c = cl[r * rsd];
+#pragma unroll
+            for (int i = 0; i < kIterRows; ++i)
+                if (i < ni) {
+                    S[(size_t)i * RP + r] = as[i] * sc2 - c;
+                    G[(size_t)i * RP + r] = al[i];
+                }
+        }
+        __syncthreads();
+        for (int i = tid >> 6; i < ni; i += nt >> 6) {      // one wave per query row
+            float* Si = S + (size_t)i * RP;
+            float* Gi = G + (size_t)i * RP;
+            float mx = -INFINITY;
+            for (int r = tid & 63; r < R; r += 64) mx = fmaxf(mx, Si[r]);
+            for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+            float sum = 0.f;
+            for (int r = tid & 63; r < R; r += 64) sum += exp2f(Si[r] - mx);
+            for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+            const float inv = 1.f / sum;
+            float dot = 0.f;
+            for (int r = tid & 63; r < R; r += 64) {
+                const float l = exp2f(Si[r] - mx) * inv;
+                Si[r] = l;
+                dot += l * Gi[r];
+            }
+            for (int o = 32; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
+            for (int r = tid & 63; r < R; r += 64) Gi[r] = Si[r] * (Gi[r] - dot);
+        }
+        __syncthreads();
+        for (int e = tid; e < R * D; e += nt) {
+            const int r = e / D, d = e % D;
+            float ay = 0.f, ak = 0.f;
+            for (int i = 0; i < ni; ++i) {
+                ay += S[(size_t)i * RP + r] * dos[i * DP + d];
+                ak += G[(size_t)i * RP + r] * qs[i * DP + d];
+            }
+            const int64_t o = (int64_t)r * rsd * D + d;
+            if (i0 == 0) {
+                dy[o] = ay;
+                dkbar[o] = ak * p.scale;
+            } else {
+                dy[o] += ay;
+                dkbar[o] += ak * p.scale;
+            }
+        }
+        for (int r = tid; r < R; r += nt) {
+            float sds = 0.f;
+            for (int i = 0; i < ni; ++i) sds += G[(size_t)i * RP + r];
+            if (i0 == 0) dcl[r * rsd] = -sds;
+            else dcl[r * rsd] -= sds;
+        }
+        for (int e = tid; e < ni * D; e += nt) {
+            const int i = e / D, d = e % D;
+            float acc = 0.f;
+            for (int r = 0; r < R; ++r) acc += G[(size_t)i * RP + r] * kbar[(int64_t)r * rsd * D + d];
+            const int64_t tok = p.qmap.row(a, i0 + i) + j;
+            g.dq[(int64_t)b * g.dqs[0] + tok * g.dqs[1] + (int64_t)h * g.dqs[2] + d] = acc * p.scale;
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void monarch_bwd_right(MonarchBwdArgs g) {
+    extern __shared__ float sm[];
+    const MonarchArgs& p = g.p;
+    const int D = p.D, b2 = p.b2, DP = D + 1;
+    float* Ks = sm;                    // [b2][D+1]
+    float* Vs = Ks + b2 * DP;          // [b2][D+1]
+    float* dKs = Vs + b2 * DP;         // [b2][D+1]
+    float* dVs = dKs + b2 * DP;        // [b2][D+1]
+    float* qs = dVs + b2 * DP;         // [D]
+    float* dkb = qs + D;               // [D]
+    float* dyv = dkb + D;              // [D]
+    float* zs = dyv + D;               // [b2]
+    float* Rr = zs + b2;               // [b2]
+    float* dR = Rr + b2;               // [b2]
+
+    const int k = blockIdx.x, ul = blockIdx.y;
+    const int unit = p.unit0 + ul;
+    const int b = unit / p.H, h = unit % p.H;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const float sc2 = p.scale * kLog2e;
+    constexpr float kLn2 = 0.6931471805599453f;
+
+    for (int f = 0; f < p.nf; ++f) {
+        const int64_t krow0 = p.kmap.row(f, k);
+        __syncthreads();
+        for (int e = tid; e < b2 * D; e += nt) {
+            const int l = e / D, d = e % D;
+            Ks[l * DP + d] = Ld<T>::get(p.k, (int64_t)b * p.ks[0] + (krow0 + l) * p.ks[1] + (int64_t)h * p.ks[2] + d);
+            Vs[l * DP + d] = Ld<T>::get(p.v, (int64_t)b * p.vs[0] + (krow0 + l) * p.vs[1] + (int64_t)h * p.vs[2] + d);
+            dKs[l * DP + d] = 0.f;
+            dVs[l * DP + d] = 0.f;
+        }
+        for (int a = 0; a < p.na; ++a) {
+            if (p.causal && (a / p.causal) < (f / p.causal)) continue;
+            const int64_t qrow0 = p.qmap.row(a, k);
+            for (int j = 0; j < b2; ++j) {
+                const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj + (int64_t)(f * p.b1 + k) * p.ws_row;
+                __syncthreads();
+                for (int d = tid; d < D; d += nt) {
+                    qs[d] = Ld<T>::get(p.q, (int64_t)b * p.qs[0] + (qrow0 + j) * p.qs[1] + (int64_t)h * p.qs[2] + d);
+                    dkb[d] = g.dkbar[blk * D + d];
+                    dyv[d] = g.dy[blk * D + d];
+                }
+                __syncthreads();
+                for (int l = tid; l < b2; l += nt) {
+                    float acc = 0.f;
+                    for (int d = 0; d < D; ++d) acc += qs[d] * Ks[l * DP + d];
+                    zs[l] = acc * sc2;
+                }
+                __syncthreads();
+                float mx = -INFINITY;
+                for (int l = 0; l < b2; ++l) mx = fmaxf(mx, zs[l]);
+                float sum = 0.f;
+                for (int l = 0; l < b2; ++l) sum += exp2f(zs[l] - mx);
+                const float lse2 = mx + log2f(sum);
+                const float dc = g.dcl[blk];
+                for (int l = tid; l < b2; l += nt) {
+                    const float lr2 = zs[l] - lse2;              // log2 R_l
+                    float acc = 0.f;
+                    for (int d = 0; d < D; ++d) acc += dkb[d] * Ks[l * DP + d] + dyv[d] * Vs[l * DP + d];
+                    Rr[l] = exp2f(lr2);
+                    dR[l] = acc + dc * (lr2 * kLn2);
+                }
+                __syncthreads();
+                float dot = 0.f;
+                for (int l = 0; l < b2; ++l) dot += Rr[l] * dR[l];
+                __syncthreads();
+                for (int l = tid; l < b2; l += nt) dR[l] = Rr[l] * (dR[l] - dot);      // dS1
+                __syncthreads();
+                for (int e = tid; e < b2 * D; e += nt) {
+                    const int l = e / D, d = e % D;
+                    dKs[l * DP + d] += Rr[l] * dkb[d] + p.scale * dR[l] * qs[d];
+                    dVs[l * DP + d] += Rr[l] * dyv[d];
+                }
+                for (int d = tid; d < D; d += nt) {
+                    float acc = 0.f;
+                    for (int l = 0; l < b2; ++l) acc += dR[l] * Ks[l * DP + d];
+                    g.dq[(int64_t)b * g.dqs[0] + (qrow0 + j) * g.dqs[1] + (int64_t)h * g.dqs[2] + d] += acc * p.scale;
+                }
+            }
+        }
+        __syncthreads();
+        if (f >= g.kv_f0 && f < g.kv_f1) {
+            for (int e = tid; e < b2 * D; e += nt) {
+                const int l = e / D, d = e % D;
+                const int64_t o = (int64_t)b * g.dks[0] + (krow0 + l - g.dk_row0) * g.dks[1] + (int64_t)h * g.dks[2] + d;
+                Ld<T>::put(g.dk, o, dKs[l * DP + d]);
+                Ld<T>::put(g.dv, o, dVs[l * DP + d]);
+            }
+        }
+    }
+}
+
+static int bwd_rows(const MonarchArgs& a) {
+    const size_t per_row = sizeof(float) * (2 * (size_t)(a.D + 1) + 2 * (size_t)a.nf * a.b1);
+    size_t ic = (128 * 1024) / per_row;
+    if (ic > (size_t)kIterRows) ic = kIterRows;
+    if (ic > (size_t)a.b1) ic = a.b1;
+    return (int)ic;
+}
+static size_t bwd_lds_left(const MonarchArgs& a) {
+    return sizeof(float) * (size_t)bwd_rows(a) * (2 * (size_t)(a.D + 1) + 2 * (size_t)a.nf * a.b1);
+}
+static size_t bwd_lds_right(const MonarchArgs& a) {
+    return sizeof(float) * (4 * (size_t)a.b2 * (a.D + 1) + 3 * (size_t)a.D + 3 * (size_t)a.b2);
+}
+
+template <typename T>
+static int launch_bwd_t(const MonarchBwdArgs& g, int nunits, hipStream_t stream) {
+    const MonarchArgs& a = g.p;
+    const size_t l1 = generic_lds1_bytes(a), ll = bwd_lds_left(a), lr = bwd_lds_right(a);
+    hipError_t err = hipSuccess;
+    if (l1 > 64 * 1024)
+        err = hipFuncSetAttribute((const void*)monarch_generic_step1<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)l1);
+    if (err == hipSuccess && ll > 64 * 1024)
+        err = hipFuncSetAttribute((const void*)monarch_bwd_left<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ll);
+    if (err == hipSuccess && lr > 64 * 1024)
+        err = hipFuncSetAttribute((const void*)monarch_bwd_right<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lr);
+    if (err != hipSuccess) {
+        set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(err));
+        return SFM_ERR_HIP;
+    }
+    hipLaunchKernelGGL((monarch_generic_step1<T>), dim3(a.b1, a.nf, nunits * a.na), dim3(256), l1, stream, a);
+    hipLaunchKernelGGL((monarch_bwd_left<T>), dim3(a.na * a.b2, nunits), dim3(256), ll, stream, g, bwd_rows(a));
+    hipLaunchKernelGGL((monarch_bwd_right<T>), dim3(a.b1, nunits), dim3(256), lr, stream, g);
+    err = hipGetLastError();
+    if (err != hipSuccess) {
+        set_error("hip launch failed: %s", hipGetErrorString(err));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+int launch_monarch_bwd(const MonarchBwdArgs& g, int dtype, int nunits, hipStream_t stream) {
+    const MonarchArgs& a = g.p;
+    if (bwd_rows(a) < 1 || generic_lds1_bytes(a) > 160 * 1024 || bwd_lds_right(a) > 160 * 1024) {
+        set_error("Monarch backward: block shape b1=%d, b2=%d, rows=%d, D=%d exceeds the LDS budget of this path", a.b1, a.b2,
+                  a.nf * a.b1, a.D);
+        return SFM_ERR_UNSUPPORTED;
+    }
+    if (dtype == SFM_F32) return launch_bwd_t<float>(g, nunits, stream);
+    if (dtype == SFM_BF16) return launch_bwd_t<BF16>(g, nunits, stream);
+    return launch_bwd_t<F16>(g, nunits, stream);
+}
+
 static size_t generic_lds2(const MonarchArgs& a) { return sizeof(float) * ((size_t)a.D + (size_t)a.nf * a.b1 + 256); }
 
 bool monarch_generic_supported(const MonarchArgs& a) {

@@ -195,7 +195,7 @@ using namespace sfm;
 
 extern "C" {
 
-int sfm_version(void) { return 2; }
+int sfm_version(void) { return 3; }
 
 const char* sfm_last_error(void) { return g_err; }
 
@@ -214,6 +214,40 @@ int sfm_monarch_workspace_bytes(const sfm_monarch_desc* desc, int32_t heads_per_
     int upp = heads_per_pass == 0 ? default_units_per_pass(pl) : (heads_per_pass > pl.units ? pl.units : heads_per_pass);
     *bytes = pl.per_unit * (size_t)upp;
     return SFM_OK;
+}
+
+// Everything of the kernel arguments that does not depend on the pass: shapes, index maps, strides, scratch
+// geometry.
+static void init_args(const sfm_monarch_desc* desc, const MonarchPlan& pl, MonarchArgs* pa) {
+    MonarchArgs& a = *pa;
+    memset(&a, 0, sizeof(a));
+    a.B = desc->B; a.H = desc->H; a.D = desc->D;
+    a.na = pl.na; a.nf = pl.nf; a.b1 = pl.b1; a.b2 = pl.b2; a.r_pad = pl.r_pad;
+    a.causal = desc->causal_block_frames;
+    a.scale = desc->sm_scale;
+    a.qmap = make_map(desc->tiling, 1);
+    a.kmap = make_map(desc->tiling, desc->kv_block_order ? 0 : 1);
+    for (int i = 0; i < 3; ++i) {
+        a.qs[i] = desc->q_stride[i]; a.ks[i] = desc->k_stride[i];
+        a.vs[i] = desc->v_stride[i]; a.os[i] = desc->o_stride[i];
+    }
+    const size_t rows = (size_t)pl.na * pl.b2 * pl.r_pad;
+    a.ws_unit = (uint32_t)rows;
+    // (a, j)-major scratch: the rows one step-2 wave streams are consecutive.  (An r-major layout, in
+    // which the rows a step-1 workgroup writes are consecutive instead, measured the same for step 1.)
+    a.ws_aj = (uint32_t)pl.r_pad;
+    a.ws_row = 1;
+    // step 1 takes as many query block-frames per workgroup as fit 256 (a, j) columns
+    int a_max = 256 / pl.b2;
+    if (a_max < 1) a_max = 1;
+    a.n_achunks = (pl.na + a_max - 1) / a_max;
+    a.a_chunk = (pl.na + a.n_achunks - 1) / a.n_achunks;
+    a.n_achunks = (pl.na + a.a_chunk - 1) / a.a_chunk;
+    a.s1_wgs = 0;
+    if (const char* e = getenv("SFM_S1_WGS")) {            // tuning override: step-1 workgroups (default one per CU)
+        int v = atoi(e);
+        if (v >= 1 && v <= 65535) a.s1_wgs = v;
+    }
 }
 
 static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
@@ -242,36 +276,10 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
     const int upp = upp_sz > (size_t)pl.units ? pl.units : (int)upp_sz;
 
     MonarchArgs a;
-    memset(&a, 0, sizeof(a));
+    init_args(desc, pl, &a);
     a.q = q; a.k = k; a.v = v; a.out = out;
-    a.B = desc->B; a.H = desc->H; a.D = desc->D;
-    a.na = pl.na; a.nf = pl.nf; a.b1 = pl.b1; a.b2 = pl.b2; a.r_pad = pl.r_pad;
-    a.causal = desc->causal_block_frames;
-    a.scale = desc->sm_scale;
-    a.qmap = make_map(desc->tiling, 1);
-    a.kmap = make_map(desc->tiling, desc->kv_block_order ? 0 : 1);
-    for (int i = 0; i < 3; ++i) {
-        a.qs[i] = desc->q_stride[i]; a.ks[i] = desc->k_stride[i];
-        a.vs[i] = desc->v_stride[i]; a.os[i] = desc->o_stride[i];
-    }
     const size_t rows = (size_t)pl.na * pl.b2 * pl.r_pad;
     const size_t mat_bytes = rows * desc->D * (pl.mfma ? 2 : 4);
-    a.ws_unit = (uint32_t)rows;
-    // (a, j)-major scratch: the rows one step-2 wave streams are consecutive.  (An r-major layout, in
-    // which the rows a step-1 workgroup writes are consecutive instead, measured the same for step 1.)
-    a.ws_aj = (uint32_t)pl.r_pad;
-    a.ws_row = 1;
-    // step 1 takes as many query block-frames per workgroup as fit 256 (a, j) columns
-    int a_max = 256 / pl.b2;
-    if (a_max < 1) a_max = 1;
-    a.n_achunks = (pl.na + a_max - 1) / a_max;
-    a.a_chunk = (pl.na + a.n_achunks - 1) / a.n_achunks;
-    a.n_achunks = (pl.na + a.a_chunk - 1) / a.a_chunk;
-    a.s1_wgs = 0;
-    if (const char* e = getenv("SFM_S1_WGS")) {            // tuning override: step-1 workgroups (default one per CU)
-        int v = atoi(e);
-        if (v >= 1 && v <= 65535) a.s1_wgs = v;
-    }
     for (int u0 = 0; u0 < pl.units; u0 += upp) {
         const int n = pl.units - u0 < upp ? pl.units - u0 : upp;
         a.unit0 = u0;
@@ -334,6 +342,113 @@ int sfm_monarch_fwd_timed(const sfm_monarch_desc* desc, const void* q, const voi
     *step1_ms = ms[0];
     *step2_ms = ms[1];
     return rc;
+}
+
+static int plan_bwd(const sfm_monarch_bwd_desc* bd, MonarchPlan* pl, size_t* per_unit) {
+    if (!bd) {
+        set_error("desc is NULL");
+        return SFM_ERR_NULL;
+    }
+    int rc = plan_monarch(&bd->fwd, pl);
+    if (rc) return rc;
+    if (bd->fwd.num_iters != 1) {
+        set_error("the backward covers num_iters == 1 (the reference's refinement path has no custom backward either)");
+        return SFM_ERR_UNSUPPORTED;
+    }
+    if (bd->kv_grad_frame_start < 0 || bd->kv_grad_frame_end > pl->nf || bd->kv_grad_frame_start >= bd->kv_grad_frame_end) {
+        set_error("kv gradient block-frames [%d, %d) outside [0, %d)", bd->kv_grad_frame_start, bd->kv_grad_frame_end, pl->nf);
+        return SFM_ERR_RANGE;
+    }
+    if (!bd->fwd.kv_block_order && (bd->kv_grad_frame_start != 0 || bd->kv_grad_frame_end != pl->nf)) {
+        set_error("a partial kv gradient needs k, v in block order (the KV-cache entry point)");
+        return SFM_ERR_UNSUPPORTED;
+    }
+    const int esz = bd->fwd.dtype == SFM_F32 ? 4 : 2;
+    const int64_t dkv_tokens = (int64_t)(bd->kv_grad_frame_end - bd->kv_grad_frame_start) * pl->b1 * pl->b2;
+    if ((rc = check_strides("dq", bd->dq_stride, bd->fwd.q_tokens, bd->fwd.H, bd->fwd.D, bd->fwd.B, 4))) return rc;
+    if ((rc = check_strides("dk/dv", bd->dkv_stride, dkv_tokens, bd->fwd.H, bd->fwd.D, bd->fwd.B, esz))) return rc;
+    const size_t rows = (size_t)pl->na * pl->b2 * pl->r_pad;
+    *per_unit = rows * bd->fwd.D * sizeof(float) * 4 + rows * sizeof(float) * 2;    // Kbar, Y, dKbar, dY; c, dc
+    return SFM_OK;
+}
+
+int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t heads_per_pass, size_t* bytes) {
+    if (!bytes) {
+        set_error("bytes is NULL");
+        return SFM_ERR_NULL;
+    }
+    MonarchPlan pl;
+    size_t per_unit = 0;
+    int rc = plan_bwd(desc, &pl, &per_unit);
+    if (rc) return rc;
+    if (heads_per_pass < 0) {
+        set_error("heads_per_pass must be >= 0");
+        return SFM_ERR_SHAPE;
+    }
+    size_t n = heads_per_pass > 0 ? (size_t)heads_per_pass : ((size_t)3 << 30) / per_unit;
+    if (n < 1) n = 1;
+    if (n > (size_t)pl.units) n = pl.units;
+    *bytes = per_unit * n;
+    return SFM_OK;
+}
+
+int sfm_monarch_bwd(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* dout,
+                    float* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream) {
+    MonarchPlan pl;
+    size_t per_unit = 0;
+    int rc = plan_bwd(desc, &pl, &per_unit);
+    if (rc) return rc;
+    if (!q || !k || !v || !dout || !dq || !dk || !dv) {
+        set_error("q, k, v, dout, dq, dk and dv must be non-NULL");
+        return SFM_ERR_NULL;
+    }
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv)) {
+        set_error("tensors must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    if (!workspace || (((uintptr_t)workspace) & 255) || workspace_bytes < per_unit) {
+        set_error("workspace must be non-NULL, 256-byte aligned and hold at least %zu bytes (one unit)", per_unit);
+        return SFM_ERR_WORKSPACE;
+    }
+    const size_t rows = (size_t)pl.na * pl.b2 * pl.r_pad;
+    // 32-bit element offsets into each scratch matrix (float)
+    size_t upp_sz = workspace_bytes / per_unit;
+    const size_t cap = (((size_t)1 << 31) - 1) / (rows * desc->fwd.D);
+    if (upp_sz > cap) upp_sz = cap;
+    if (upp_sz < 1) {
+        set_error("one (batch, head) unit needs %zu bytes of scratch, more than a pass can address", per_unit);
+        return SFM_ERR_UNSUPPORTED;
+    }
+    const int upp = upp_sz > (size_t)pl.units ? pl.units : (int)upp_sz;
+
+    MonarchBwdArgs g;
+    memset(&g, 0, sizeof(g));
+    init_args(&desc->fwd, pl, &g.p);
+    g.p.q = q; g.p.k = k; g.p.v = v; g.p.out = nullptr;
+    g.dout = dout; g.dq = dq; g.dk = dk; g.dv = dv;
+    for (int i = 0; i < 3; ++i) {
+        g.dos[i] = desc->fwd.o_stride[i];
+        g.dqs[i] = desc->dq_stride[i];
+        g.dks[i] = desc->dkv_stride[i];
+    }
+    g.kv_f0 = desc->kv_grad_frame_start;
+    g.kv_f1 = desc->kv_grad_frame_end;
+    g.dk_row0 = (int64_t)g.kv_f0 * pl.b1 * pl.b2;       // non-zero only in block order
+    const size_t mat = rows * desc->fwd.D * sizeof(float);
+    for (int u0 = 0; u0 < pl.units; u0 += upp) {
+        const int n = pl.units - u0 < upp ? pl.units - u0 : upp;
+        g.p.unit0 = u0;
+        char* w = (char*)workspace;
+        g.p.kbar = w;
+        g.p.y = w + mat * upp;
+        g.dkbar = (float*)(w + 2 * mat * upp);
+        g.dy = (float*)(w + 3 * mat * upp);
+        g.p.cl = (float*)(w + 4 * mat * upp);
+        g.dcl = g.p.cl + rows * upp;
+        rc = launch_monarch_bwd(g, desc->fwd.dtype, n, (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    return SFM_OK;
 }
 
 int sfm_kv_cache_write(int32_t dtype, int32_t B, int32_t H, int32_t D, const sfm_tiling* tiling, const void* new_k,

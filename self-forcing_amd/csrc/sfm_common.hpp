@@ -148,6 +148,23 @@ struct MonarchArgs {
     int s1_total;    // step-1 work items: (unit, k, a-chunk, f) tiles
 };
 
+// Backward: the forward arguments (scratch matrices in float) plus the gradient tensors.
+struct MonarchBwdArgs {
+    MonarchArgs p;
+    const void* dout;        // [B, Sq, H, D] tensor dtype, strides dos
+    int64_t dos[3];
+    float* dq;               // [B, Sq, H, D] float, strides dqs
+    int64_t dqs[3];
+    void* dk;                // tensor dtype, rows kmap.row(f, k) + l - dk_row0, strides dks
+    void* dv;
+    int64_t dks[3];
+    int64_t dk_row0;
+    float* dkbar;            // same layout as p.kbar
+    float* dy;               // same layout as p.y
+    float* dcl;              // same layout as p.cl: gradient of sum_l R ln R
+    int kv_f0, kv_f1;        // kv block-frames whose dK / dV are wanted
+};
+
 // Optional timing hooks: ev[0] is recorded before step 1, ev[1] between the steps, ev[2] after step 2.
 struct StepEvents {
     hipEvent_t ev[3];
@@ -157,6 +174,7 @@ int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t
 int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev);
 bool monarch_mfma_supported(int dtype, int D, int b2);
 int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
+int launch_monarch_bwd(const MonarchBwdArgs& g, int dtype, int nunits, hipStream_t stream);
 
 void set_error(const char* fmt, ...);
 

@@ -20,7 +20,7 @@ ERR_NAMES = {
 SYMBOLS = [
     "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
-    "sfm_rms_norm", "sfm_last_error", "sfm_version",
+    "sfm_rms_norm", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_last_error", "sfm_version",
 ]
 
 
@@ -36,6 +36,11 @@ class MonarchDesc(C.Structure):
                 ("num_iters", C.c_int32), ("reserved", C.c_int32),
                 ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
                 ("o_stride", C.c_int64 * 3)]
+
+
+class MonarchBwdDesc(C.Structure):
+    _fields_ = [("fwd", MonarchDesc), ("dq_stride", C.c_int64 * 3), ("dkv_stride", C.c_int64 * 3),
+                ("kv_grad_frame_start", C.c_int32), ("kv_grad_frame_end", C.c_int32)]
 
 
 class DenseDesc(C.Structure):
@@ -76,6 +81,8 @@ def load():
     lib.sfm_monarch_fwd.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, C.c_size_t, P]
     lib.sfm_monarch_fwd_timed.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, C.c_size_t, P,
                                           C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    lib.sfm_monarch_bwd_workspace_bytes.argtypes = [C.POINTER(MonarchBwdDesc), C.c_int32, C.POINTER(C.c_size_t)]
+    lib.sfm_monarch_bwd.argtypes = [C.POINTER(MonarchBwdDesc), P, P, P, P, P, P, P, P, C.c_size_t, P]
     lib.sfm_kv_cache_write.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(Tiling), P, P, S3, P, P,
                                        S3, I64, I64, I64, P]
     lib.sfm_monarch_attn_with_kv_cache.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, S3, I64, I64, P, P,

@@ -4,7 +4,8 @@
     monarch_attn                <->  wan/modules/monarch_attn.py:1753-1776
 
 Inputs are [B, S, H, D] CUDA tensors (bf16 / fp16 / fp32, head_dim contiguous) in token order;
-the KV cache holds rows in Monarch block order and is updated in place.  Forward only.
+the KV cache holds rows in Monarch block order and is updated in place.  Under autograd the operators
+are torch.autograd.Functions whose backward runs the library's fp32 backward kernels (num_iters == 1).
 num_iters > 1 runs the alternating refinement the reference implements in pure torch
 (monarch_attn_slow, wan/modules/monarch_attn.py:1705-1751) as fp32 HIP kernels.
 """
@@ -59,12 +60,113 @@ def _stream(t):
     return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
 
 
+def _from_block_order(x, f_tied, h_reduce, w_reduce, h, w):
+    """Inverse of the reference's rearrangement (monarch_attn.py:1696-1703) on a [B, n, H, D] tensor."""
+    if f_tied == 1 and h_reduce == 1 and w_reduce == 1:
+        return x
+    B, n, H, D = x.shape
+    x = x.reshape(B, -1, h_reduce, w_reduce, f_tied, h // h_reduce, w // w_reduce, H, D)
+    return x.permute(0, 1, 4, 2, 5, 3, 6, 7, 8).reshape(B, n, H, D)
+
+
+def _monarch_bwd(q, k, v, dout, tiling, sm_scale, kv_block_order, cbf, kv_f0=0, kv_f1=None, heads_per_pass=0):
+    """Raw call of sfm_monarch_bwd: returns (dq float32, dk, dv); dk, dv cover kv block-frames [kv_f0, kv_f1) in
+    the row order of k."""
+    f_tied, h_reduce, w_reduce, h, w = tiling
+    per_frame = f_tied * (h // h_reduce) * (w // w_reduce)
+    nf = k.shape[1] // per_frame
+    if kv_f1 is None:
+        kv_f1 = nf
+    if dout.stride(3) != 1:
+        dout = dout.contiguous()
+    dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    dk = torch.empty((k.shape[0], (kv_f1 - kv_f0) * per_frame, k.shape[2], k.shape[3]), dtype=k.dtype, device=k.device)
+    dv = torch.empty_like(dk)
+    bd = _l.MonarchBwdDesc()
+    bd.fwd = _desc(q, k, v, dout, f_tied, h_reduce, w_reduce, h, w, sm_scale, kv_block_order, cbf)
+    bd.dq_stride = _l.strides3(dq)
+    bd.dkv_stride = _l.strides3(dk)
+    bd.kv_grad_frame_start, bd.kv_grad_frame_end = kv_f0, kv_f1
+    n = C.c_size_t(0)
+    _l.check(_l.load().sfm_monarch_bwd_workspace_bytes(C.byref(bd), heads_per_pass, C.byref(n)))
+    ws = torch.empty(n.value, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        _l.check(_l.load().sfm_monarch_bwd(C.byref(bd), q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(),
+                                           dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), n.value,
+                                           _stream(q)))
+    return dq, dk, dv
+
+
+class _MonarchFn(torch.autograd.Function):
+    """monarch_attn under autograd (_attention_no_cache, monarch_attn.py:1472-1693)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, tiling, sm_scale, block_causal_size, heads_per_pass, kv_block_order):
+        out = monarch_attn(q, k, v, *tiling, sm_scale=sm_scale, block_causal_size=block_causal_size,
+                           heads_per_pass=heads_per_pass, kv_block_order=kv_block_order)
+        ctx.save_for_backward(q, k, v)
+        ctx.cfg = (tiling, sm_scale, block_causal_size, kv_block_order)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v = ctx.saved_tensors
+        tiling, sm_scale, block_causal_size, kv_block_order = ctx.cfg
+        cbf = 0
+        if block_causal_size is not None:
+            cbf = block_causal_size // (tiling[0] * (tiling[3] // tiling[1]) * (tiling[4] // tiling[2]))
+        dq, dk, dv = _monarch_bwd(q, k, v, dout, tiling, sm_scale, 1 if kv_block_order else 0, cbf)
+        return dq.to(q.dtype), dk, dv, None, None, None, None, None
+
+
+class _MonarchCacheFn(torch.autograd.Function):
+    """monarch_attn_with_kv_cache under autograd (_attention_with_cache, monarch_attn.py:1225-1470): the caches
+    are written in place in the forward and saved by reference, as the reference does; with grad_only_new_kv
+    only the block-frames written by this call get K/V gradients (:1364-1374)."""
+
+    @staticmethod
+    def forward(ctx, q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, tiling, sm_scale, grad_only_new_kv,
+                heads_per_pass):
+        out = monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, *tiling,
+                                         sm_scale=sm_scale, heads_per_pass=heads_per_pass)
+        ctx.save_for_backward(q, k_cache, v_cache)
+        ctx.cfg = (start_idx, end_idx, tiling, sm_scale, grad_only_new_kv)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k_cache, v_cache = ctx.saved_tensors
+        start_idx, end_idx, tiling, sm_scale, grad_only_new_kv = ctx.cfg
+        f_tied, h_reduce, w_reduce, h, w = tiling
+        per_frame = f_tied * (h // h_reduce) * (w // w_reduce)
+        if grad_only_new_kv:
+            dq, dk, dv = _monarch_bwd(q, k_cache, v_cache, dout, tiling, sm_scale, 1, 0, start_idx // per_frame,
+                                      end_idx // per_frame)
+            dk_cache = dv_cache = None
+            dk_new, dv_new = dk, dv
+        else:
+            dq, dk_cache, dv_cache = _monarch_bwd(q, k_cache, v_cache, dout, tiling, sm_scale, 1, 0)
+            dk_new, dv_new = dk_cache[:, start_idx:end_idx], dv_cache[:, start_idx:end_idx]
+        dk_new = _from_block_order(dk_new, *tiling)
+        dv_new = _from_block_order(dv_new, *tiling)
+        return dq.to(q.dtype), dk_cache, dv_cache, dk_new, dv_new, None, None, None, None, None, None
+
+
+def _needs_grad(*ts):
+    return torch.is_grad_enabled() and any(t.requires_grad for t in ts)
+
+
 def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, f_tied, h_reduce, w_reduce, h, w,
                                sm_scale=None, num_iters=1, grad_only_new_kv=False, heads_per_pass=0):
     """Writes new_k/new_v into k_cache/v_cache[:, start_idx:end_idx] (block order, in place) and
     returns one-iteration Monarch attention of q against the whole cache view."""
-    if torch.is_grad_enabled() and (q.requires_grad or new_k.requires_grad or new_v.requires_grad):
-        raise NotImplementedError("forward only: call under torch.no_grad()")
+    if _needs_grad(q, k_cache, v_cache, new_k, new_v):
+        if num_iters != 1:
+            raise NotImplementedError("num_iters > 1 has no backward")
+        if sm_scale is None:
+            sm_scale = q.shape[-1] ** -0.5
+        return _MonarchCacheFn.apply(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx,
+                                     (f_tied, h_reduce, w_reduce, h, w), sm_scale, grad_only_new_kv, heads_per_pass)
     _check4("q", q)
     for name, t in (("k_cache", k_cache), ("v_cache", v_cache), ("new_k", new_k), ("new_v", new_v)):
         _check4(name, t, q.dtype, q.device)
@@ -94,8 +196,13 @@ def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block
     block-frames of later causal blocks.  `kv_block_order=True` (no counterpart in the reference) says
     that k, v are a KV-cache view whose rows are already in Monarch block order, e.g. after
     prologue.qk_prologue wrote them."""
-    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
-        raise NotImplementedError("forward only: call under torch.no_grad()")
+    if _needs_grad(q, k, v):
+        if num_iters != 1:
+            raise NotImplementedError("num_iters > 1 has no backward")
+        if sm_scale is None:
+            sm_scale = q.shape[-1] ** -0.5
+        return _MonarchFn.apply(q, k, v, (f_tied, h_reduce, w_reduce, h, w), sm_scale, block_causal_size,
+                                heads_per_pass, kv_block_order)
     _check4("q", q)
     _check4("k", k, q.dtype, q.device)
     _check4("v", v, q.dtype, q.device)

@@ -1,0 +1,124 @@
+"""GPU parity of the Monarch backward (autograd Functions over sfm_monarch_bwd) against torch autograd through the
+float64 CPU oracle.  Shapes follow the reference's harness (run_kv_cache_test / run_causal_test,
+monarch_attn.py:1880-1957) at sizes the oracle finishes in seconds.
+
+Tolerances: fp32 tensors <= 2e-4 of the gradient's max-abs (fp32 kernels, sums of ~10^3 terms); 16-bit tensors the
+reference's rtol = 1e-2 (bf16) / 1e-3 (fp16) with atol = the same fraction of the gradient's max-abs (the reference
+compares raw values of O(1) gradients from randn inputs)."""
+import pytest
+import torch
+
+import self_forcing_amd as sfa
+from gpu_util import max_abs, randn
+from oracle import blocks, monarch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+mattn = sfa.monarch_attn
+
+
+def _leaf(t, dev=None):
+    t = t.clone().detach()
+    if dev:
+        t = t.to(dev)
+    return t.requires_grad_(True)
+
+
+def _close(got, ref, dtype):
+    got, ref = got.detach().float().cpu(), ref.detach().float()
+    if dtype == torch.float32:
+        assert (got - ref).abs().max() <= 2e-4 * max(1.0, ref.abs().max().item())
+    else:
+        tol = 1e-2 if dtype == torch.bfloat16 else 1e-3
+        # 16-bit gradients are rounded once at the end; accumulation is fp32
+        assert torch.allclose(got, ref, atol=tol * max(1.0, ref.abs().max().item()), rtol=tol)
+
+
+@pytest.mark.parametrize("tiling,h,w", [((1, 1, 1), 4, 8), ((1, 2, 1), 6, 8), ((3, 1, 1), 4, 6), ((1, 1, 2), 3, 8)])
+def test_no_cache_fp32_gradients(tiling, h, w):
+    F = 3
+    q0 = randn((2, F * h * w, 2, 32), 100, torch.float32)
+    k0, v0 = (randn((2, 2 * F * h * w, 2, 32), 101 + i, torch.float32) for i in range(2))
+    do = randn((2, F * h * w, 2, 32), 103, torch.float32)
+    qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
+    monarch.monarch_attn(qr, kr, vr, *tiling, h, w).backward(do.double())
+    qd, kd, vd = _leaf(q0, DEV), _leaf(k0, DEV), _leaf(v0, DEV)
+    out = mattn.monarch_attn(qd, kd, vd, *tiling, h, w)
+    out.backward(do.to(DEV))
+    _close(qd.grad, qr.grad, torch.float32)
+    _close(kd.grad, kr.grad, torch.float32)
+    _close(vd.grad, vr.grad, torch.float32)
+
+
+def test_block_causal_fp32_gradients():
+    h, w, F = 3, 8, 4
+    q0, k0, v0, do = (randn((1, F * h * w, 2, 64), 110 + i, torch.float32) for i in range(4))
+    qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
+    monarch.monarch_attn(qr, kr, vr, 1, 1, 1, h, w, block_causal_size=2 * h * w).backward(do.double())
+    qd, kd, vd = _leaf(q0, DEV), _leaf(k0, DEV), _leaf(v0, DEV)
+    mattn.monarch_attn(qd, kd, vd, 1, 1, 1, h, w, block_causal_size=2 * h * w).backward(do.to(DEV))
+    _close(qd.grad, qr.grad, torch.float32)
+    _close(kd.grad, kr.grad, torch.float32)
+    _close(vd.grad, vr.grad, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("partial", [False, True])
+def test_kv_cache_gradients_like_the_reference_harness(dtype, partial):
+    """q of 2 frames, cache of 5 frames of which the last 2 arrive with the call; h_reduce = 2 so that block
+    order differs from token order.  partial = grad_only_new_kv."""
+    h, w, H, D = 6, 20, 2, 64
+    tiling = (1, 2, 1)
+    n_old, n_new = 3 * h * w, 2 * h * w
+    q0 = randn((1, 2 * h * w, H, D), 120, dtype)
+    k_old, v_old = (randn((1, n_old, H, D), 121 + i, dtype) for i in range(2))       # cache rows (block order)
+    k_new, v_new = (randn((1, n_new, H, D), 123 + i, dtype) for i in range(2))       # token order
+    do = randn((1, 2 * h * w, H, D), 125, dtype)
+
+    # oracle: functional composition of the cache write, float64
+    qr, kor, vor, knr, vnr = (_leaf(t.double()) for t in (q0, k_old, v_old, k_new, v_new))
+    kfull = torch.cat([kor, blocks.to_blocks(knr, *tiling, h, w).reshape(1, n_new, H, D)], 1)
+    vfull = torch.cat([vor, blocks.to_blocks(vnr, *tiling, h, w).reshape(1, n_new, H, D)], 1)
+    qb = blocks.to_blocks(qr, *tiling, h, w)
+    b1, b2 = qb.shape[2], qb.shape[3]
+    ob = monarch.monarch_1iter(qb, kfull.reshape(1, -1, b1, b2, H, D), vfull.reshape(1, -1, b1, b2, H, D), D ** -0.5)
+    blocks.from_blocks(ob, *tiling, h, w).backward(do.double())
+
+    qd, knd, vnd = _leaf(q0, DEV), _leaf(k_new, DEV), _leaf(v_new, DEV)
+    kc = torch.zeros(1, n_old + n_new, H, D, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    kc[:, :n_old], vc[:, :n_old] = k_old.to(DEV), v_old.to(DEV)
+    kc.requires_grad_(not partial)
+    vc.requires_grad_(not partial)
+    out = mattn.monarch_attn_with_kv_cache(qd, kc, vc, knd, vnd, n_old, n_old + n_new, *tiling, h, w,
+                                           grad_only_new_kv=partial)
+    out.backward(do.to(DEV))
+    _close(qd.grad, qr.grad, dtype)
+    _close(knd.grad, knr.grad, dtype)
+    _close(vnd.grad, vnr.grad, dtype)
+    if not partial:
+        _close(kc.grad[:, :n_old], kor.grad, dtype)
+        _close(vc.grad[:, :n_old], vor.grad, dtype)
+    else:
+        assert kc.grad is None and vc.grad is None
+
+
+def test_480p_block_shape_bf16_one_head():
+    """b1 = 30, b2 = 52, D = 128 as in the 480p grid: 1 query frame against 3 cached frames, one head."""
+    h, w, D = 30, 52, 128
+    q0 = randn((1, h * w, 1, D), 130, torch.bfloat16)
+    k0, v0 = (randn((1, 3 * h * w, 1, D), 131 + i, torch.bfloat16) for i in range(2))
+    do = randn((1, h * w, 1, D), 133, torch.bfloat16)
+    qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
+    monarch.monarch_attn(qr, kr, vr, 1, 1, 1, h, w).backward(do.double())
+    qd, kd, vd = _leaf(q0, DEV), _leaf(k0, DEV), _leaf(v0, DEV)
+    mattn.monarch_attn(qd, kd, vd, 1, 1, 1, h, w).backward(do.to(DEV))
+    _close(qd.grad, qr.grad, torch.bfloat16)
+    _close(kd.grad, kr.grad, torch.bfloat16)
+    _close(vd.grad, vr.grad, torch.bfloat16)
+
+
+def test_descriptor_errors():
+    q = randn((1, 64, 1, 32), 140, torch.float32).to(DEV).requires_grad_(True)
+    with pytest.raises(NotImplementedError):
+        mattn.monarch_attn(q, q, q, 1, 1, 1, 4, 8, num_iters=2)
