@@ -122,6 +122,17 @@ def op_level(torch, sfa, args):
     torch.cuda.synchronize()
     dense_ms = (time.perf_counter() - t0) * 1e3 / 5
 
+    # backward of the same op (fp32 kernels), one timed call after one warm-up
+    from self_forcing_amd.monarch_attn import _monarch_bwd
+    do = torch.randn(B, SQ, H, D, generator=g).to(bf).to(dev)
+    bwd_ms = None
+    for it in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        _monarch_bwd(q, kc, vc, do, (1, 1, 1, B1, B2), D ** -0.5, 1, 0)
+        torch.cuda.synchronize()
+        bwd_ms = (time.perf_counter() - t0) * 1e3
+
     if args.copy_probe:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -137,6 +148,8 @@ def op_level(torch, sfa, args):
                                      "(4680 q x 32760 kv), new chunk written at tokens 28080..32760",
                          "ms_per_call": ms_call, "tflops": tfl, "mfma_frac": tfl / MFMA_BF16_PEAK_TFLOPS,
                          "kernel_ms": {"monarch_step1": s1_ms, "monarch_step2": s2_ms}},
+        "monarch_bwd": {"workload": "gradients of q and of all 21 cached K/V frames at the same shape (fp32 kernels)",
+                        "ms_per_call": bwd_ms},
         "dense_fallback": {"ms_per_call": dense_ms, "tflops": DENSE_FLOPS / (dense_ms * 1e-3) / 1e12,
                            "mfma_frac": DENSE_FLOPS / (dense_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS},
         "roofline": {"kernel": "monarch_step1_kernel (configs[1] shape)", "bound": "hbm", "achieved": s1_gbs,
@@ -177,6 +190,7 @@ def main():
                       "heads_per_pass": args.heads_per_pass}}
     if not args.op_only:
         pl = sfa.pipeline
+        pl.use_tuned_gemms()          # hipBLASLt solution per GEMM shape (shipped selections; unknown shapes tuned in warm-up)
         gen = pl.build_generator("1.3B", attention_flags=dict(use_framewise=True))
         pipe = pl.CausalInferencePipeline(gen)
         g = torch.Generator().manual_seed(0)

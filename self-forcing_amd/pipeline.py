@@ -179,6 +179,25 @@ class CausalInferencePipeline(nn.Module):
         return output
 
 
+def use_tuned_gemms(filename=None, tune=True):
+    """Lets PyTorch's TunableOp pick the hipBLASLt / rocBLAS solution of every GEMM shape around the attention
+    operators (projections, FFN, embeddings).  Selections for the 1.3B shapes measured on gfx950 ship next to
+    this file and are loaded first; with `tune` a shape that is not listed is timed once, on its first call.
+    New selections go to a file in the temporary directory, never back into the package."""
+    import os
+    import tempfile
+    import torch.cuda.tunable as tn
+    if filename is None:
+        filename = os.path.join(os.path.dirname(os.path.abspath(__file__)), "gemm_tuning_gfx950.csv")
+    tn.enable(True)
+    tn.tuning_enable(bool(tune))
+    tn.set_max_tuning_duration(50)
+    tn.set_max_tuning_iterations(30)
+    tn.set_filename(os.path.join(tempfile.gettempdir(), f"sfm_gemm_tuning_{os.getpid()}.csv"))
+    if os.path.exists(filename):
+        tn.read_file(filename)
+
+
 def build_generator(size="1.3B", dtype=torch.bfloat16, device="cuda:0", seed=0, zero_head=False, timestep_shift=5.0,
                     **model_overrides):
     """Random-init causal Wan generator of a named size (reference init, optionally with a non-zero head)."""
