@@ -89,7 +89,8 @@ int sfm_monarch_fwd_timed(const sfm_monarch_desc* desc, const void* q, const voi
  *                       order of k: token order, or block order when fwd.kv_block_order = 1
  *   kv_grad_frame_*     kv block-frames whose gradients are produced; a proper sub-range is the reference's
  *                       grad_only_new_kv (:1364-1374) and needs block order
- * Everything is recomputed from q, k, v (the forward saves nothing but its inputs). */
+ * Everything is recomputed from q, k, v (the forward saves nothing but its inputs).  The workspace size depends
+ * on the implementation in use (sfm_monarch_bwd_uses_gemm); query it in the same process state. */
 typedef struct sfm_monarch_bwd_desc {
     sfm_monarch_desc fwd;
     int64_t dq_stride[3];
@@ -99,6 +100,10 @@ typedef struct sfm_monarch_bwd_desc {
 } sfm_monarch_bwd_desc;
 
 int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t heads_per_pass, size_t* bytes);
+/* 1 when the backward runs as batched rocBLAS GEMMs + row kernels (rocBLAS found at run time and SFM_BWD_SIMT
+ * unset), 0 when it runs the fp32 SIMT kernels.  The first GEMM call on a device creates a rocBLAS handle,
+ * which allocates; every other entry point of this header allocates nothing.  No counterpart in the reference. */
+int sfm_monarch_bwd_uses_gemm(void);
 int sfm_monarch_bwd(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* dout,
                     float* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream);
 

@@ -372,6 +372,15 @@ static int plan_bwd(const sfm_monarch_bwd_desc* bd, MonarchPlan* pl, size_t* per
     return SFM_OK;
 }
 
+// The batched-GEMM backward is used whenever rocBLAS can be loaded; SFM_BWD_SIMT=1 selects the fp32 SIMT kernels.
+static bool bwd_uses_gemm() {
+    const char* e = getenv("SFM_BWD_SIMT");
+    if (e && atoi(e) != 0) return false;
+    return monarch_bwd_gemm_available();
+}
+
+int sfm_monarch_bwd_uses_gemm(void) { return bwd_uses_gemm() ? 1 : 0; }
+
 int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t heads_per_pass, size_t* bytes) {
     if (!bytes) {
         set_error("bytes is NULL");
@@ -384,6 +393,15 @@ int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t he
     if (heads_per_pass < 0) {
         set_error("heads_per_pass must be >= 0");
         return SFM_ERR_SHAPE;
+    }
+    if (bwd_uses_gemm()) {
+        MonarchArgs a;
+        init_args(&desc->fwd, pl, &a);
+        int n = heads_per_pass > 0 ? (heads_per_pass > pl.units ? pl.units : heads_per_pass) : pl.units;
+        if (heads_per_pass == 0)
+            while (n > 1 && monarch_bwd_gemm_bytes(a, desc->fwd.dtype, n) > ((size_t)7 << 29)) --n;     // 3.5 GiB
+        *bytes = monarch_bwd_gemm_bytes(a, desc->fwd.dtype, n);
+        return SFM_OK;
     }
     size_t n = heads_per_pass > 0 ? (size_t)heads_per_pass : ((size_t)3 << 30) / per_unit;
     if (n < 1) n = 1;
@@ -406,8 +424,40 @@ int sfm_monarch_bwd(const sfm_monarch_bwd_desc* desc, const void* q, const void*
         set_error("tensors must be 16-byte aligned");
         return SFM_ERR_ALIGN;
     }
-    if (!workspace || (((uintptr_t)workspace) & 255) || workspace_bytes < per_unit) {
-        set_error("workspace must be non-NULL, 256-byte aligned and hold at least %zu bytes (one unit)", per_unit);
+    if (!workspace || (((uintptr_t)workspace) & 255)) {
+        set_error("workspace must be non-NULL and 256-byte aligned");
+        return SFM_ERR_WORKSPACE;
+    }
+    if (bwd_uses_gemm()) {
+        MonarchBwdArgs g;
+        memset(&g, 0, sizeof(g));
+        init_args(&desc->fwd, pl, &g.p);
+        int n = pl.units;
+        while (n > 1 && monarch_bwd_gemm_bytes(g.p, desc->fwd.dtype, n) > workspace_bytes) --n;
+        if (monarch_bwd_gemm_bytes(g.p, desc->fwd.dtype, n) > workspace_bytes) {
+            set_error("workspace holds %zu bytes, one (batch, head) unit needs %zu", workspace_bytes,
+                      monarch_bwd_gemm_bytes(g.p, desc->fwd.dtype, 1));
+            return SFM_ERR_WORKSPACE;
+        }
+        g.p.q = q; g.p.k = k; g.p.v = v;
+        g.dout = dout; g.dq = dq; g.dk = dk; g.dv = dv;
+        for (int i = 0; i < 3; ++i) {
+            g.dos[i] = desc->fwd.o_stride[i];
+            g.dqs[i] = desc->dq_stride[i];
+            g.dks[i] = desc->dkv_stride[i];
+        }
+        g.kv_f0 = desc->kv_grad_frame_start;
+        g.kv_f1 = desc->kv_grad_frame_end;
+        g.dk_row0 = (int64_t)g.kv_f0 * pl.b1 * pl.b2;
+        for (int u0 = 0; u0 < pl.units; u0 += n) {
+            g.p.unit0 = u0;
+            rc = launch_monarch_bwd_gemm(g, desc->fwd.dtype, pl.units - u0 < n ? pl.units - u0 : n, workspace, (hipStream_t)stream);
+            if (rc) return rc;
+        }
+        return SFM_OK;
+    }
+    if (workspace_bytes < per_unit) {
+        set_error("workspace must hold at least %zu bytes (one unit)", per_unit);
         return SFM_ERR_WORKSPACE;
     }
     const size_t rows = (size_t)pl.na * pl.b2 * pl.r_pad;

@@ -175,6 +175,9 @@ int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStrea
 bool monarch_mfma_supported(int dtype, int D, int b2);
 int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
 int launch_monarch_bwd(const MonarchBwdArgs& g, int dtype, int nunits, hipStream_t stream);
+bool monarch_bwd_gemm_available();
+size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits);
+int launch_monarch_bwd_gemm(const MonarchBwdArgs& g, int dtype, int nunits, void* workspace, hipStream_t stream);
 
 void set_error(const char* fmt, ...);
 

@@ -20,7 +20,7 @@ ERR_NAMES = {
 SYMBOLS = [
     "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
-    "sfm_rms_norm", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_last_error", "sfm_version",
+    "sfm_rms_norm", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm", "sfm_last_error", "sfm_version",
 ]
 
 

@@ -34,8 +34,17 @@ def _close(got, ref, dtype):
         assert torch.allclose(got, ref, atol=tol * max(1.0, ref.abs().max().item()), rtol=tol)
 
 
+@pytest.fixture(params=["gemm", "simt"])
+def bwd_path(request, monkeypatch):
+    """Both backward implementations behind sfm_monarch_bwd: batched library GEMMs + row kernels (default) and the
+    fp32 SIMT kernels (SFM_BWD_SIMT=1, also what runs when rocBLAS cannot be loaded)."""
+    monkeypatch.setenv("SFM_BWD_SIMT", "1" if request.param == "simt" else "0")
+    assert sfa.lib.load().sfm_monarch_bwd_uses_gemm() == (1 if request.param == "gemm" else 0)
+    return request.param
+
+
 @pytest.mark.parametrize("tiling,h,w", [((1, 1, 1), 4, 8), ((1, 2, 1), 6, 8), ((3, 1, 1), 4, 6), ((1, 1, 2), 3, 8)])
-def test_no_cache_fp32_gradients(tiling, h, w):
+def test_no_cache_fp32_gradients(tiling, h, w, bwd_path):
     F = 3
     q0 = randn((2, F * h * w, 2, 32), 100, torch.float32)
     k0, v0 = (randn((2, 2 * F * h * w, 2, 32), 101 + i, torch.float32) for i in range(2))
@@ -50,7 +59,7 @@ def test_no_cache_fp32_gradients(tiling, h, w):
     _close(vd.grad, vr.grad, torch.float32)
 
 
-def test_block_causal_fp32_gradients():
+def test_block_causal_fp32_gradients(bwd_path):
     h, w, F = 3, 8, 4
     q0, k0, v0, do = (randn((1, F * h * w, 2, 64), 110 + i, torch.float32) for i in range(4))
     qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
@@ -64,7 +73,7 @@ def test_block_causal_fp32_gradients():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("partial", [False, True])
-def test_kv_cache_gradients_like_the_reference_harness(dtype, partial):
+def test_kv_cache_gradients_like_the_reference_harness(dtype, partial, bwd_path):
     """q of 2 frames, cache of 5 frames of which the last 2 arrive with the call; h_reduce = 2 so that block
     order differs from token order.  partial = grad_only_new_kv."""
     h, w, H, D = 6, 20, 2, 64
@@ -103,7 +112,7 @@ def test_kv_cache_gradients_like_the_reference_harness(dtype, partial):
         assert kc.grad is None and vc.grad is None
 
 
-def test_480p_block_shape_bf16_one_head():
+def test_480p_block_shape_bf16_one_head(bwd_path):
     """b1 = 30, b2 = 52, D = 128 as in the 480p grid: 1 query frame against 3 cached frames, one head."""
     h, w, D = 30, 52, 128
     q0 = randn((1, h * w, 1, D), 130, torch.bfloat16)
