@@ -127,10 +127,22 @@ __global__ __launch_bounds__(256) void gather_rows(typename El<E>::type* dst, co
     *(uint64_t*)(dst + (e / pieces) * D + pc * kPer) = *(const uint64_t*)sp;
 }
 
-// Right factor: one wave per segment (u, k, aj, f) of b2 logits S1[(u,k)][aj][f][:].
-// Rb[t][aj][:] = softmax(s * S1) rounded to the operand type; c[t][aj] = sum_l R ln R.
+// Right factor: one wave per segment (u, k, aj, f) of b2 logits S1[(u,k)][aj][f][:], lane l holding logits
+// l, l + 64, ... (one per lane when b2 <= 64).
+// Rb[t][aj][:] = softmax(s * S1) rounded to the operand type; c[(u, aj)][r] = sum_l R ln R.
+constexpr int kSegPerLane = 4;          // b2 <= 256
+
+__device__ __forceinline__ float wave_max(float v) {
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
 template <typename E>
-__global__ __launch_bounds__(256) void softmax_right(const float* S1, typename El<E>::type* Rb, float* c, int AJ, int nf, int b2,
+__global__ __launch_bounds__(256) void softmax_right(const float* S1, typename El<E>::type* Rb, float* c, int b1, int AJ, int nf, int b2,
                                                      float scale, int64_t nseg) {
     const int64_t seg = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (seg >= nseg) return;
@@ -139,28 +151,44 @@ __global__ __launch_bounds__(256) void softmax_right(const float* S1, typename E
     const int64_t row = seg / nf;                       // uk * AJ + aj
     const int aj = (int)(row % AJ);
     const int64_t uk = row / AJ;
+    const int k = (int)(uk % b1);
+    const int64_t u = uk / b1;
     const int64_t blk = (uk * nf + f) * AJ + aj;
     const float* z = S1 + seg * b2;
+    float v[kSegPerLane];
     float mx = -INFINITY;
-    for (int l = lane; l < b2; l += 64) mx = fmaxf(mx, z[l] * scale);
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+#pragma unroll
+    for (int q = 0; q < kSegPerLane; ++q) {
+        const int l = lane + 64 * q;
+        v[q] = l < b2 ? z[l] * scale : -INFINITY;
+        mx = fmaxf(mx, v[q]);
+    }
+    mx = wave_max(mx);
     float sum = 0.f;
-    for (int l = lane; l < b2; l += 64) sum += __expf(z[l] * scale - mx);
-    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+#pragma unroll
+    for (int q = 0; q < kSegPerLane; ++q) sum += __expf(v[q] - mx);
+    sum = wave_sum(sum);
     const float lse = mx + __logf(sum);
     float ent = 0.f;
-    for (int l = lane; l < b2; l += 64) {
-        const float lr = z[l] * scale - lse;
-        const float r = __expf(lr);
-        El<E>::put(Rb, blk * b2 + l, r);
-        ent += r * lr;
+#pragma unroll
+    for (int q = 0; q < kSegPerLane; ++q) {
+        const int l = lane + 64 * q;
+        if (l < b2) {
+            const float lr = v[q] - lse;
+            const float r = __expf(lr);
+            El<E>::put(Rb, blk * b2 + l, r);
+            ent += r * lr;
+        }
     }
-    for (int o = 32; o > 0; o >>= 1) ent += __shfl_xor(ent, o);
-    if (lane == 0) c[blk] = ent;
+    ent = wave_sum(ent);
+    if (lane == 0) c[(u * AJ + aj) * ((int64_t)nf * b1) + (int64_t)k * nf + f] = ent;
 }
 
-// Left factor: one workgroup per row (u, aj, i) of RR logits S2[(u,aj)][i][r].
+// Left factor: one workgroup per row (u, aj, i) of RR logits S2[(u,aj)][i][r], thread t holding logits
+// t, t + 256, ... (RR <= 256 * kLeftPerThread).
 // L = softmax(s * S2 - c) (masked block-frames give 0), dS2 = L (dLm - sum L dLm); both in the operand type.
+constexpr int kLeftPerThread = 8;
+
 template <typename E>
 __global__ __launch_bounds__(256) void softmax_left(const float* S2, const float* dLm, const float* c, typename El<E>::type* L,
                                                     typename El<E>::type* dS2, int b1, int b2, int AJ, int nf, int causal, float scale) {
@@ -169,66 +197,77 @@ __global__ __launch_bounds__(256) void softmax_left(const float* S2, const float
     const int64_t row = blockIdx.x;                     // (u * AJ + aj) * b1 + i
     const int64_t uaj = row / b1;
     const int aj = (int)(uaj % AJ);
-    const int64_t u = uaj / AJ;
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const float* z = S2 + row * RR;
     const float* g = dLm + row * RR;
-    const float* cc = c + u * RR * AJ + aj;              // c of row r at cc[r * AJ]
+    const float* cc = c + uaj * RR;
     const int flim = causal ? min(nf, ((aj / b2) / causal + 1) * causal) : nf;      // visible kv block-frames
     auto block_max = [&](float v) {
-        for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+        v = wave_max(v);
         __syncthreads();
         if (lane == 0) red[wv] = v;
         __syncthreads();
-        float r = red[0];
-        for (int w = 1; w < (int)(blockDim.x >> 6); ++w) r = fmaxf(r, red[w]);
-        return r;
+        return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
     };
     auto block_sum = [&](float v) {
-        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        v = wave_sum(v);
         __syncthreads();
         if (lane == 0) red[wv] = v;
         __syncthreads();
-        float r = 0.f;
-        for (int w = 0; w < (int)(blockDim.x >> 6); ++w) r += red[w];
-        return r;
+        return red[0] + red[1] + red[2] + red[3];
     };
-    auto logit = [&](int r) { return (r % nf) < flim ? z[r] * scale - cc[(int64_t)r * AJ] : -INFINITY; };
+    float v[kLeftPerThread], gv[kLeftPerThread];
     float mx = -INFINITY;
-    for (int r = tid; r < RR; r += blockDim.x) mx = fmaxf(mx, logit(r));
+#pragma unroll
+    for (int q = 0; q < kLeftPerThread; ++q) {
+        const int r = tid + 256 * q;
+        const bool ok = r < RR && (r % nf) < flim;
+        v[q] = ok ? z[r] * scale - cc[r] : -INFINITY;
+        gv[q] = r < RR ? g[r] : 0.f;
+        mx = fmaxf(mx, v[q]);
+    }
     mx = block_max(mx);
     float sum = 0.f;
-    for (int r = tid; r < RR; r += blockDim.x) sum += __expf(logit(r) - mx);
+#pragma unroll
+    for (int q = 0; q < kLeftPerThread; ++q) {
+        v[q] = __expf(v[q] - mx);
+        sum += v[q];
+    }
     sum = block_sum(sum);
     const float inv = 1.f / sum;
     float dot = 0.f;
-    for (int r = tid; r < RR; r += blockDim.x) dot += __expf(logit(r) - mx) * inv * g[r];
+#pragma unroll
+    for (int q = 0; q < kLeftPerThread; ++q) {
+        v[q] *= inv;
+        dot += v[q] * gv[q];
+    }
     dot = block_sum(dot);
-    for (int r = tid; r < RR; r += blockDim.x) {
-        const float l = __expf(logit(r) - mx) * inv;
-        El<E>::put(L, row * RR + r, l);
-        El<E>::put(dS2, row * RR + r, l * (g[r] - dot));
+#pragma unroll
+    for (int q = 0; q < kLeftPerThread; ++q) {
+        const int r = tid + 256 * q;
+        if (r < RR) {
+            El<E>::put(L, row * RR + r, v[q]);
+            El<E>::put(dS2, row * RR + r, v[q] * (gv[q] - dot));
+        }
     }
 }
 
-// dc[(u, r)][aj] = - sum_i dS2[(u, aj)][i][r]
+// dc[(u, aj)][r] = - sum_i dS2[(u, aj)][i][r]
 template <typename E>
 __global__ __launch_bounds__(256) void reduce_dc(const typename El<E>::type* dS2, float* dc, int b1, int AJ, int RR, int64_t total) {
     const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;      // (u * AJ + aj) * RR + r
     if (e >= total) return;
     const int64_t uaj = e / RR;
     const int r = (int)(e % RR);
-    const int aj = (int)(uaj % AJ);
-    const int64_t u = uaj / AJ;
     float s = 0.f;
     for (int i = 0; i < b1; ++i) s += El<E>::get(dS2, (uaj * b1 + i) * RR + r);
-    dc[(u * RR + r) * AJ + aj] = -s;
+    dc[e] = -s;
 }
 
 // dS1[(u,k)][aj][f][:] = R (dR + dc ln R - sum_l R (dR + dc ln R)), same segments as softmax_right; R recomputed in float.
 template <typename E>
 __global__ __launch_bounds__(256) void softmax_right_bwd(const float* S1, const float* dRb, const float* dc, typename El<E>::type* dS1,
-                                                         int AJ, int nf, int b2, float scale, int64_t nseg) {
+                                                         int b1, int AJ, int nf, int b2, float scale, int64_t nseg) {
     const int64_t seg = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (seg >= nseg) return;
     const int lane = threadIdx.x & 63;
@@ -236,26 +275,43 @@ __global__ __launch_bounds__(256) void softmax_right_bwd(const float* S1, const 
     const int64_t row = seg / nf;
     const int aj = (int)(row % AJ);
     const int64_t uk = row / AJ;
+    const int k = (int)(uk % b1);
+    const int64_t u = uk / b1;
     const int64_t blk = (uk * nf + f) * AJ + aj;
     const float* z = S1 + seg * b2;
     const float* g = dRb + blk * b2;
-    const float dcv = dc[blk];
+    const float dcv = dc[(u * AJ + aj) * ((int64_t)nf * b1) + (int64_t)k * nf + f];
+    float v[kSegPerLane], gv[kSegPerLane];
     float mx = -INFINITY;
-    for (int l = lane; l < b2; l += 64) mx = fmaxf(mx, z[l] * scale);
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+#pragma unroll
+    for (int q = 0; q < kSegPerLane; ++q) {
+        const int l = lane + 64 * q;
+        v[q] = l < b2 ? z[l] * scale : -INFINITY;
+        gv[q] = l < b2 ? g[l] : 0.f;
+        mx = fmaxf(mx, v[q]);
+    }
+    mx = wave_max(mx);
     float sum = 0.f;
-    for (int l = lane; l < b2; l += 64) sum += __expf(z[l] * scale - mx);
-    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+#pragma unroll
+    for (int q = 0; q < kSegPerLane; ++q) sum += __expf(v[q] - mx);
+    sum = wave_sum(sum);
     const float lse = mx + __logf(sum);
     float dot = 0.f;
-    for (int l = lane; l < b2; l += 64) {
-        const float lr = z[l] * scale - lse;
-        dot += __expf(lr) * (g[l] + dcv * lr);
+#pragma unroll
+    for (int q = 0; q < kSegPerLane; ++q) {
+        const int l = lane + 64 * q;
+        if (l < b2) {
+            const float lr = v[q] - lse;
+            v[q] = __expf(lr);              // R
+            gv[q] += dcv * lr;              // dR + dc ln R
+            dot += v[q] * gv[q];
+        }
     }
-    for (int o = 32; o > 0; o >>= 1) dot += __shfl_xor(dot, o);
-    for (int l = lane; l < b2; l += 64) {
-        const float lr = z[l] * scale - lse;
-        El<E>::put(dS1, seg * b2 + l, __expf(lr) * (g[l] + dcv * lr - dot));
+    dot = wave_sum(dot);
+#pragma unroll
+    for (int q = 0; q < kSegPerLane; ++q) {
+        const int l = lane + 64 * q;
+        if (l < b2) El<E>::put(dS1, seg * b2 + l, v[q] * (gv[q] - dot));
     }
 }
 
@@ -281,15 +337,16 @@ __global__ __launch_bounds__(256) void scatter_dq(const float* dQa, const float*
     *(float4*)(dq + b * s0 + tok * s1 + h * s2 + pc * 4) = float4{x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w};
 }
 
-// dk / dv rows of kv block-frames [f0, f1) from the float accumulators dKk / dVk [u][k][f][l][D]
+// dk / dv rows of kv block-frames [f0, f1) from the float accumulators dKk / dVk [u][k][f][l][D], 4 elements a thread
 template <typename E>
 __global__ __launch_bounds__(256) void scatter_dkv(const float* dKk, const float* dVk, typename El<E>::type* dk, typename El<E>::type* dv,
                                                    int64_t s0, int64_t s1, int64_t s2, TokMap map, int nf, int f0, int f1,
                                                    int64_t row0, int H, int D, int unit0, int64_t total) {
-    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;      // one element each
+    const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= total) return;
-    const int d = (int)(e % D);
-    int64_t row = e / D;
+    const int pieces = D / 4;
+    const int d = (int)(e % pieces) * 4;
+    int64_t row = e / pieces;
     const int l = (int)(row % map.b2);
     row /= map.b2;
     const int ff = (int)(row % (f1 - f0));
@@ -301,8 +358,9 @@ __global__ __launch_bounds__(256) void scatter_dkv(const float* dKk, const float
     const int b = unit / H, h = unit % H;
     const int64_t src = ((((int64_t)u * map.b1 + k) * nf + f) * map.b2 + l) * D + d;
     const int64_t dst = b * s0 + (map.row(f, k) + l - row0) * s1 + h * s2 + d;
-    El<E>::put(dk, dst, dKk[src]);
-    El<E>::put(dv, dst, dVk[src]);
+    const float4 x = *(const float4*)(dKk + src), y = *(const float4*)(dVk + src);
+    El<E>::put(dk, dst, x.x); El<E>::put(dk, dst + 1, x.y); El<E>::put(dk, dst + 2, x.z); El<E>::put(dk, dst + 3, x.w);
+    El<E>::put(dv, dst, y.x); El<E>::put(dv, dst + 1, y.y); El<E>::put(dv, dst + 2, y.z); El<E>::put(dv, dst + 3, y.w);
 }
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -427,7 +485,7 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     // 1. S1 = Qk Kk^T per (u, k)
     gemm(cx, false, true, AJ, NL, D, 1.f, 0.f, Qk_uk, Kk_uk, S1_uk, tE, tF, nuk);
     hipLaunchKernelGGL((softmax_right<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const float*)(ws + lay.S1f),
-                       (T*)(ws + lay.Rb), (float*)(ws + lay.c), AJ, nf, b2, s, nseg);
+                       (T*)(ws + lay.Rb), (float*)(ws + lay.c), b1, AJ, nf, b2, s, nseg);
     // 2, 3. Kbar, Y blocks = R block . K / V block per t
     gemm(cx, false, false, AJ, D, b2, 1.f, 0.f, Rb_t, Kk_t, Kbar_t, tE, tE, nt);
     gemm(cx, false, false, AJ, D, b2, 1.f, 0.f, Rb_t, Vk_t, Y_t, tE, tE, nt);
@@ -462,7 +520,7 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     gemm(cx, false, true, AJ, b2, D, 1.f, 0.f, dKbar_t, Kk_t, dRb_t, tE, tF, nt);
     gemm(cx, false, true, AJ, b2, D, 1.f, 1.f, dY_t, Vk_t, dRb_t, tE, tF, nt);
     hipLaunchKernelGGL((softmax_right_bwd<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const float*)(ws + lay.S1f),
-                       (const float*)(ws + lay.dRb), (const float*)(ws + lay.dc), (T*)(ws + lay.dS1), AJ, nf, b2, s, nseg);
+                       (const float*)(ws + lay.dRb), (const float*)(ws + lay.dc), (T*)(ws + lay.dS1), b1, AJ, nf, b2, s, nseg);
     // 10. dQ (right factor) = s dS1 K per (u, k);  11. dK = s dS1^T q per (u, k)
     gemm(cx, false, false, AJ, D, NL, s, 0.f, dS1_uk, Kk_uk, dQk_uk, tE, tF, nuk);
     gemm(cx, true, false, NL, D, AJ, s, 0.f, dS1_uk, Qk_uk, dKk_uk, tE, tF, nuk);
@@ -475,7 +533,7 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
         const int64_t tq = (int64_t)n * MQ * (D / 4);
         hipLaunchKernelGGL(scatter_dq, dim3((unsigned)((tq + 255) / 256)), dim3(256), 0, stream, (const float*)(ws + lay.dQa),
                            (const float*)(ws + lay.dQk), g.dq, g.dqs[0], g.dqs[1], g.dqs[2], p.qmap, na, H, D, p.unit0, tq);
-        const int64_t tk = (int64_t)n * b1 * (g.kv_f1 - g.kv_f0) * b2 * D;
+        const int64_t tk = (int64_t)n * b1 * (g.kv_f1 - g.kv_f0) * b2 * (D / 4);
         hipLaunchKernelGGL((scatter_dkv<E>), dim3((unsigned)((tk + 255) / 256)), dim3(256), 0, stream, (const float*)(ws + lay.dKk),
                            (const float*)(ws + lay.dVk), (T*)g.dk, (T*)g.dv, g.dks[0], g.dks[1], g.dks[2], p.kmap, nf, g.kv_f0, g.kv_f1,
                            g.dk_row0, H, D, p.unit0, tk);
@@ -499,6 +557,11 @@ size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits) {
 int launch_monarch_bwd_gemm(const MonarchBwdArgs& g, int dtype, int nunits, void* workspace, hipStream_t stream) {
     if (!blas_load()) {
         set_error("rocBLAS could not be loaded");
+        return SFM_ERR_UNSUPPORTED;
+    }
+    if (g.p.b2 > 64 * kSegPerLane || g.p.nf * g.p.b1 > 256 * kLeftPerThread) {
+        set_error("Monarch backward: b2=%d or rows=%d beyond the row kernels' limits (%d, %d)", g.p.b2, g.p.nf * g.p.b1,
+                  64 * kSegPerLane, 256 * kLeftPerThread);
         return SFM_ERR_UNSUPPORTED;
     }
     if (dtype == SFM_F32) return run<float>(g, nunits, workspace, stream);
