@@ -88,6 +88,9 @@ class AttentionFlags:
         self.w_reduce = _env_int("MONARCH_ATTN_W_REDUCE", 1)
         self.use_framewise = bool(_env_int("MONARCH_ATTN_FRAMEWISE", 0))
         self.disable_monarch = bool(_env_int("DISABLE_MONARCH_ATTN", 0))
+        # no counterpart in the reference: keep a windowed KV cache (local_attn_size != -1) as a ring instead of
+        # shifting it down on every eviction (cache_step_ring)
+        self.ring_cache = bool(_env_int("SFM_RING_KV_CACHE", 0))
         layers = os.getenv("MONARCH_ATTN_DISABLE_LAYERS")
         if layers is not None and block_num is not None and block_num in [int(x) for x in layers.split(",")]:
             self.disable_monarch = True
@@ -150,6 +153,24 @@ def cache_step(kv_cache, current_start, num_new, frame_seqlen, local_attn_size, 
     return roll, cache_start, local_start - cache_start, local_end - cache_start, current_end
 
 
+def cache_step_ring(kv_cache, current_start, num_new, frame_seqlen, sink_size):
+    """Windowed cache kept as a ring: the chunk at global tokens [current_start, current_start + num_new) is
+    written over the oldest chunk after the sink frames instead of shifting the window down
+    (causal_model.py:912-926 does the shift with a copy).  Attention over the cache is a sum over its rows, so
+    the order in which block-frames sit in it does not change the result; the rotary phase is in the rows.
+    Chunks must arrive in order (a re-run of the latest chunk lands in the same slot).
+    Returns (write_start, view_len, current_end), or None when chunks would straddle the end of the ring."""
+    cache_len = kv_cache["k"].shape[1]
+    sink = sink_size * frame_seqlen
+    ring = cache_len - sink
+    current_end = current_start + num_new
+    if current_end <= cache_len:                       # still filling: positions are the global ones
+        return current_start, current_end, current_end
+    if ring <= 0 or ring % num_new or current_start < sink or (current_start - sink) % num_new:
+        return None
+    return sink + (current_start - sink) % ring, cache_len, current_end
+
+
 def cache_commit(kv_cache, current_end, local_end):
     """causal_model.py:1102-1103 (the reference stores the view-relative local end)."""
     kv_cache["_global_end"], kv_cache["_local_end"] = current_end, local_end
@@ -195,14 +216,23 @@ class CausalWanSelfAttention(nn.Module):
         if self._rope is None or self._rope.device != x.device:
             self._rope = self.ops.rope_table(d, x.device)
 
-        roll, cache_start, local_start, local_end, current_end = cache_step(
-            kv_cache, current_start, s, frame_seqlen, self.local_attn_size, self.sink_size, self.max_attention_size)
-        if roll[2] > 0:      # window eviction (causal_model.py:919-922)
-            src, dst, ln = roll
-            for key in ("k", "v"):
-                kv_cache[key][:, dst:dst + ln] = kv_cache[key][:, src:src + ln].clone()
-
-        view_len = local_end
+        ring = None
+        if fl.ring_cache and self.local_attn_size != -1 and kv_cache.get("_ring", True):
+            ring = cache_step_ring(kv_cache, current_start, s, frame_seqlen, self.sink_size)
+            if ring is None and kv_cache.get("_ring"):
+                raise ValueError("ring KV cache: chunk sizes changed so that a chunk would straddle the end of the ring")
+            kv_cache["_ring"] = ring is not None
+        if ring is not None:
+            write_start, view_len, current_end = ring
+            cache_start, local_start, local_end = 0, write_start, write_start + s
+        else:
+            roll, cache_start, local_start, local_end, current_end = cache_step(
+                kv_cache, current_start, s, frame_seqlen, self.local_attn_size, self.sink_size, self.max_attention_size)
+            if roll[2] > 0:      # window eviction (causal_model.py:919-922)
+                src, dst, ln = roll
+                for key in ("k", "v"):
+                    kv_cache[key][:, dst:dst + ln] = kv_cache[key][:, src:src + ln].clone()
+            view_len = local_end
         is_init = fl.use_dense_init and view_len == 3 * frame_seqlen
         dense = fl.disable_monarch or is_init
         f_tied = 1 if fl.use_framewise else 3

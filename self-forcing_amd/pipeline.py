@@ -126,6 +126,7 @@ class CausalInferencePipeline(nn.Module):
             c["local_end_index"] = torch.tensor([0], dtype=torch.long, device=device)
             c["_global_end"] = c["_local_end"] = 0
             c.pop("_written", None)
+            c.pop("_ring", None)
 
     def _next_seed(self):
         if self.seeds is None:

@@ -71,3 +71,23 @@ def test_single_forward_matches_closely():
     # layer-0 cache rows (prologue output of the first layer) agree to one bf16 step
     assert max_abs(kv_d[0]["k"][:, :936], kv_r[0]["k"][:, :936]) <= 2 ** -5
     assert torch.equal(kv_d[0]["v"][:, 936:].cpu(), kv_r[0]["v"][:, 936:])
+
+
+def test_windowed_rollout_with_ring_cache_matches_shifting_cache_on_cpu():
+    """3 chunks through a 6-frame window: the GPU keeps the cache as a ring, the CPU reference run shifts it
+    down as the reference does; the third chunk evicts the first."""
+    torch.manual_seed(0)
+    ref = cm.CausalWanModel(ops=OracleOps(), attention_flags=dict(use_framewise=True), local_attn_size=6, **CFG)
+    ref.init_weights(zero_head=False)
+    ref = ref.to(torch.bfloat16).eval()
+    dev = cm.CausalWanModel(attention_flags=dict(use_framewise=True, ring_cache=True), local_attn_size=6, **CFG).to(torch.bfloat16).eval()
+    dev.load_state_dict(ref.state_dict())
+    g = torch.Generator().manual_seed(0)
+    noise = torch.randn(1, 9, 16, 12, 104, generator=g).to(torch.bfloat16)
+    ctx = torch.randn(1, 16, 64, generator=g).to(torch.bfloat16)
+    out_ref = pl.CausalInferencePipeline(pl.WanDiffusionWrapper(ref), frame_hw=(6, 52), local_attn_size=6).inference(noise, ctx)
+    pipe = pl.CausalInferencePipeline(pl.WanDiffusionWrapper(dev.to("cuda:0")), frame_hw=(6, 52), local_attn_size=6)
+    out = pipe.inference(noise.to("cuda:0"), ctx.to("cuda:0"))
+    assert pipe.kv_cache1[0]["_ring"] and pipe.kv_cache1[0]["_local_end"] == 3 * 312      # third chunk wrapped to the start
+    for c in range(3):
+        assert _cos(out[:, 3 * c:3 * c + 3], out_ref[:, 3 * c:3 * c + 3]) > 0.995

@@ -112,3 +112,45 @@ def test_patchify_equals_conv3d_and_unpatchify_inverts():
     assert u.shape == (2, 16, 3, 4, 6)
     # token (f,h,w), patch offset (q,r), channel c lands at [c, f, 2h+q, 2w+r]
     assert u[1, 5, 2, 3, 4] == y[1, (2 * 2 + 1) * 3 + 2].view(1, 2, 2, 16)[0, 1, 0, 5]
+
+
+@pytest.mark.parametrize("local_attn,sink,monarch", [(6, 0, True), (9, 3, True), (6, 0, False)])
+def test_ring_cache_gives_the_windowed_rollout_of_the_shifting_cache(local_attn, sink, monarch):
+    """5 chunks of 3 frames through a window of `local_attn` frames (the first `sink` pinned): the cache kept as a
+    ring against the reference's shift-down eviction (causal_model.py:912-926).  Same rows, other order in the
+    cache: results agree up to the order of float32 sums."""
+    outs = []
+    for ring in (False, True):
+        flags = dict(use_framewise=True, ring_cache=ring) if monarch else dict(disable_monarch=True, ring_cache=ring)
+        torch.manual_seed(0)
+        m = cm.CausalWanModel(ops=OracleOps(), attention_flags=flags, local_attn_size=local_attn, sink_size=sink, **TINY)
+        m.init_weights(zero_head=False)
+        gen = pl.WanDiffusionWrapper(m.float().eval())
+        pipe = pl.CausalInferencePipeline(gen, frame_hw=(2, 3), local_attn_size=local_attn)
+        g = torch.Generator().manual_seed(3)
+        noise = torch.randn(1, 15, 16, 4, 6, generator=g)
+        ctx = torch.randn(1, 5, 32, generator=g)
+        outs.append(pipe.inference(noise, ctx))
+        assert pipe.kv_cache1[0].get("_ring", False) == ring
+    assert torch.isfinite(outs[0]).all() and outs[0].abs().sum() > 0
+    assert torch.allclose(outs[0], outs[1], atol=2e-5, rtol=1e-4)
+    # the first two chunks fit the window; later ones differ from an unbounded cache, so eviction did happen
+    assert not torch.allclose(outs[0][:, 9:], _unbounded(noise, ctx)[:, 9:], atol=1e-3)
+
+
+def _unbounded(noise, ctx):
+    torch.manual_seed(0)
+    m = cm.CausalWanModel(ops=OracleOps(), attention_flags=dict(use_framewise=True), **{**TINY, "total_seq_len": 15 * 6})
+    m.init_weights(zero_head=False)
+    pipe = pl.CausalInferencePipeline(pl.WanDiffusionWrapper(m.float().eval()), frame_hw=(2, 3), num_cache_frames=15)
+    return pipe.inference(noise, ctx)
+
+
+def test_ring_cache_falls_back_when_chunks_would_straddle_the_ring():
+    kv = {"k": torch.zeros(1, 4 * 6, 1, 8)}           # window of 4 frames, chunks of 3: 4 % 3 != 0
+    assert cm.cache_step_ring(kv, 0, 18, 6, 0) == (0, 18, 18)
+    assert cm.cache_step_ring(kv, 18, 18, 6, 0) is None
+    kv = {"k": torch.zeros(1, 9 * 6, 1, 8)}           # 3 sink frames + ring of 6
+    assert cm.cache_step_ring(kv, 54, 18, 6, 3) == (18, 54, 72)
+    assert cm.cache_step_ring(kv, 72, 18, 6, 3) == (36, 54, 90)
+    assert cm.cache_step_ring(kv, 90, 18, 6, 3) == (18, 54, 108)
