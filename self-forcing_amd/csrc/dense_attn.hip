@@ -5,10 +5,13 @@
 // (wan/modules/attn_patch.py:20-110).
 //
 // MFMA kernel (bf16 / fp16, head_dim 64 or 128): workgroup = 128 queries of one (batch, head),
-// wave = 32 queries.  Per 64-key tile (K row-major and V^T staged once in LDS):
+// wave = 32 queries.  Per 64-key tile (K and V rows staged once in LDS, row-major, 16-byte chunks
+// XOR-swizzled):
 //     S^T[l, q] = K[l,:] . Q[q,:]          online softmax per query column (lane)
-//     O^T[d, q] += V^T[d, l] P^T[l, q]     P^T is fed from the accumulator layout (perm_row)
-// The next tile's K/V rows are prefetched into registers while the current one is consumed.
+//     O^T[d, q] += V^T[d, l] P^T[l, q]     V^T comes from transposing LDS reads (ds_read_tr16_b64), P^T from the
+//                                          accumulator layout (perm_row)
+// Two LDS buffers: the next tile's rows are fetched into registers while the current one is consumed and
+// written to the other buffer at the end of the iteration, so there is one barrier per tile.
 
 #include "sfm_common.hpp"
 
@@ -16,15 +19,27 @@ namespace sfm {
 
 template <int D>
 struct DnLds {
-    static constexpr int kRowPitch = D + 8;
-    static constexpr int kTPitch = 72;
-    static constexpr int kKrow = 0;
-    static constexpr int kVT = 64 * kRowPitch;
-    static constexpr int kTiles = kVT + D * kTPitch;
-    static constexpr int kStage = 4 * 32 * kRowPitch;
-    static constexpr int kTotal = kTiles > kStage ? kTiles : kStage;
-    static constexpr size_t bytes() { return 2 * (size_t)kTotal; }
+    static constexpr int kCPR = D / 8;                  // 16-byte chunks per row
+    static constexpr int kPitch = 2 * D;                // bytes per row
+    static constexpr int kMat = 64 * kPitch;            // one 64-row tile
+    static constexpr int kBuf = 2 * kMat;               // K tile, V tile
+    static constexpr int kStage = 4 * 32 * (2 * D + 16);   // output staging, 4 waves x 32 rows
+    static constexpr int kTotal = 2 * kBuf > kStage ? 2 * kBuf : kStage;
+    // chunk c of row r sits at chunk position c ^ swz(r); depends on r mod 16 only
+    static __device__ __forceinline__ int swz(int r) {
+        return D >= 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
+    }
 };
+
+typedef short dn_s16x4 __attribute__((ext_vector_type(4)));
+
+// Transposing LDS read: within each group of 16 lanes, lane i receives element i % 4 of the 8 bytes addressed
+// by lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12.  With lane s of a group addressing row s / 4, columns
+// 4 (s % 4) .. + 3 of a 4 x 16 block, lane i ends up with column i of the four rows.
+__device__ __forceinline__ u32x2 dn_read_tr(const char* lds, uint32_t off) {
+    dn_s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((dn_s16x4 __attribute__((address_space(3)))*)(lds + off));
+    return __builtin_bit_cast(u32x2, v);
+}
 
 template <class E, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void dense_fwd_kernel(sfm_dense_desc p, const uint16_t* __restrict__ q,
@@ -32,16 +47,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                                                         const uint16_t* __restrict__ vp, uint16_t* __restrict__ out,
                                                         float* __restrict__ lse) {
     using L = DnLds<D>;
-    constexpr int DS = D / 16, DT = D / 32, DP = D / 2;
-    __shared__ __attribute__((aligned(16))) uint16_t lds[L::kTotal];
+    constexpr int DS = D / 16, DT = D / 32;
+    extern __shared__ __attribute__((aligned(256))) char lds[];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, m = lane & 31, hf = lane >> 5;
     const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
     const int q0 = blockIdx.x * 128 + wave * 32;
     const int nq = p.q_tokens, nk = p.kv_tokens;
 
-    const uint16_t* kg = kp + (int64_t)b * p.k_stride[0] + (int64_t)h * p.k_stride[2];
-    const uint16_t* vg = vp + (int64_t)b * p.v_stride[0] + (int64_t)h * p.v_stride[2];
+    const char* kg = (const char*)(kp + (int64_t)b * p.k_stride[0] + (int64_t)h * p.k_stride[2]);
+    const char* vg = (const char*)(vp + (int64_t)b * p.v_stride[0] + (int64_t)h * p.v_stride[2]);
+    const uint32_t krs = (uint32_t)p.k_stride[1] * 2, vrs = (uint32_t)p.v_stride[1] * 2;     // row strides in bytes
 
     // query operand (B of the logits MFMA): lane (m, hf) holds Q[q0 + m][16 ds + 8 hf + 0..7]
     u32x4 qb[DS];
@@ -52,50 +68,54 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
     }
 
-    constexpr int kTasks = 8 * DP;                 // (sh, dword column) staging tasks per matrix
-    constexpr int kPer = (kTasks + 255) / 256;     // 2 for D=128, 1 for D=64
-    uint32_t pk[kPer][8], pv[kPer][8];
+    // staging: thread `tid` moves chunks tid, tid + 256, ... of the K tile and the same ones of the V tile.
+    // LDS position P (16-byte units) holds global chunk (P % kCPR) ^ swz(row) of row P / kCPR.  Rows past the
+    // last key repeat the last key (their logits are masked).
+    constexpr int kCh = 64 * L::kCPR / 256;            // 4 for D = 128, 2 for D = 64
+    int srow[kCh];
+    uint32_t scol[kCh];
+#pragma unroll
+    for (int i = 0; i < kCh; ++i) {
+        const int P = tid + i * 256;
+        srow[i] = P / L::kCPR;
+        scol[i] = (uint32_t)(((P % L::kCPR) ^ L::swz(srow[i])) * 16);
+    }
+    u32x4 sk[kCh], sv[kCh];
     auto prefetch = [&](int l0) {
+        const int last = nk - 1 - l0;                  // >= 0
 #pragma unroll
-        for (int t = 0; t < kPer; ++t) {
-            int task = tid + t * 256;
-            if (task < kTasks) {
-                int pc = task % DP, sh = task / DP;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    int l = l0 + perm_row(sh >> 1, sh & 1, e);
-                    uint32_t kk = 0, vv = 0;
-                    if (l < nk) {
-                        kk = *(const uint32_t*)(kg + (int64_t)l * p.k_stride[1] + 2 * pc);
-                        vv = *(const uint32_t*)(vg + (int64_t)l * p.v_stride[1] + 2 * pc);
-                    }
-                    pk[t][e] = kk;
-                    pv[t][e] = vv;
-                }
-            }
+        for (int i = 0; i < kCh; ++i) {
+            const uint32_t r = (uint32_t)(l0 + min(srow[i], last));
+            sk[i] = *(const u32x4*)(kg + (size_t)r * krs + scol[i]);
+            sv[i] = *(const u32x4*)(vg + (size_t)r * vrs + scol[i]);
         }
     };
-    auto commit = [&]() {
+    auto commit = [&](uint32_t buf) {
 #pragma unroll
-        for (int t = 0; t < kPer; ++t) {
-            int task = tid + t * 256;
-            if (task < kTasks) {
-                int pc = task % DP, sh = task / DP;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    int l = perm_row(sh >> 1, sh & 1, e);
-                    *(uint32_t*)(lds + L::kKrow + l * L::kRowPitch + 2 * pc) = pk[t][e];
-                }
-                u32x4 lo, hi;
-                lo.x = lo16x2(pv[t][0], pv[t][1]); lo.y = lo16x2(pv[t][2], pv[t][3]);
-                lo.z = lo16x2(pv[t][4], pv[t][5]); lo.w = lo16x2(pv[t][6], pv[t][7]);
-                hi.x = hi16x2(pv[t][0], pv[t][1]); hi.y = hi16x2(pv[t][2], pv[t][3]);
-                hi.z = hi16x2(pv[t][4], pv[t][5]); hi.w = hi16x2(pv[t][6], pv[t][7]);
-                *(u32x4*)(lds + L::kVT + (2 * pc) * L::kTPitch + sh * 8) = lo;
-                *(u32x4*)(lds + L::kVT + (2 * pc + 1) * L::kTPitch + sh * 8) = hi;
-            }
+        for (int i = 0; i < kCh; ++i) {
+            *(u32x4*)(lds + buf + (tid + i * 256) * 16) = sk[i];
+            *(u32x4*)(lds + buf + L::kMat + (tid + i * 256) * 16) = sv[i];
         }
     };
+
+    // logits: A operand = K rows; lane (m, hf) reads chunk 2 ds + hf of row 32 t + m
+    const uint32_t sA0 = (uint32_t)m * L::kPitch + (uint32_t)((hf ^ L::swz(m)) << 4);
+    // output: A operand = V^T.  For head-dim rows 32 dt + 0..31 and contraction step st lane (m, hf) needs keys
+    // l = 16 st + 4 hf + {0..3} and + 8 + {0..3} (the order in which the logits' accumulators hold l) of
+    // head-dim column 32 dt + m: two transposing reads.
+    uint32_t trA[DT][2];
+    {
+        const int s16 = lane & 15, g16 = lane >> 4;
+        const int rl = 4 * hf + (s16 >> 2);
+        const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int r = rl + 8 * half, c = 4 * dt + cl;
+                trA[dt][half] = L::kMat + (uint32_t)r * L::kPitch + (uint32_t)((c ^ L::swz(r)) << 4) + (uint32_t)(s16 & 1) * 8;
+            }
+    }
 
     f32x16 oacc[DT];
 #pragma unroll
@@ -107,23 +127,48 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int ntile = (nk + 63) / 64;
 
     prefetch(0);
+    commit(0);
     for (int tile = 0; tile < ntile; ++tile) {
-        lds_barrier();                   // everyone is done reading the previous tile
-        commit();
+        const uint32_t buf = (uint32_t)(tile & 1) * L::kBuf;
+        lds_barrier();                   // this tile is in LDS; the other buffer is free again
         if (tile + 1 < ntile) prefetch(64 * (tile + 1));
-        lds_barrier();                   // tile visible; the prefetch stays in flight
 
+        // LDS reads are issued a batch ahead of the MFMAs that use them (the fences keep that order)
         f32x16 s[2];
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int v = 0; v < 16; ++v) s[t][v] = 0.f;
-            const uint16_t* arow = lds + L::kKrow + (32 * t + m) * L::kRowPitch + 8 * hf;
+        const uint32_t sA = sA0 + buf;
+        constexpr int kB = 2;
+        u32x4 sa[2][kB][2];
+        auto load_s = [&](int ds0, u32x4 (*dst)[2]) {
 #pragma unroll
-            for (int ds = 0; ds < DS; ++ds) {
-                u32x4 a = *(const u32x4*)(arow + 16 * ds);
-                s[t] = E::mfma32(a, qb[ds], s[t]);
+            for (int i = 0; i < kB; ++i)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) dst[i][t] = *(const u32x4*)(lds + ((sA ^ (uint32_t)((ds0 + i) << 5)) + t * 32 * L::kPitch));
+        };
+        u32x4 ops[2][4];
+        auto load_ops = [&](int dt, u32x4* dst) {
+            const uint32_t a0 = trA[dt][0] + buf, a1 = trA[dt][1] + buf;
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                const u32x2 lo = dn_read_tr(lds, a0 + st * 16 * L::kPitch);
+                const u32x2 hi = dn_read_tr(lds, a1 + st * 16 * L::kPitch);
+                dst[st] = u32x4{lo.x, lo.y, hi.x, hi.y};
             }
+        };
+        load_s(0, sa[0]);
+#pragma unroll
+        for (int bt = 0; bt < DS / kB; ++bt) {
+            if (bt + 1 < DS / kB) load_s((bt + 1) * kB, sa[(bt + 1) & 1]);
+            else load_ops(0, ops[0]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < kB; ++i)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) s[t] = E::mfma32(sa[bt & 1][i][t], qb[bt * kB + i], s[t]);
+            __builtin_amdgcn_sched_barrier(0);
         }
         // online softmax in base 2; the scale is folded into the exponent argument (one fma per logit)
         const int lrem = nk - 64 * tile;           // valid keys in this tile (>= 1)
@@ -174,13 +219,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         lrun += psum;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            const uint16_t* arow = lds + L::kVT + (32 * dt + m) * L::kTPitch + 8 * hf;
+            if (dt + 1 < DT) load_ops(dt + 1, ops[(dt + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int st = 0; st < 4; ++st) {
-                u32x4 a = *(const u32x4*)(arow + 16 * st);
-                oacc[dt] = E::mfma32(a, pb[st], oacc[dt]);
-            }
+            for (int st = 0; st < 4; ++st) oacc[dt] = E::mfma32(ops[dt & 1][st], pb[st], oacc[dt]);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        if (tile + 1 < ntile) commit(buf ^ L::kBuf);
     }
 
     const float ltot = xhalf_sum(lrun);
@@ -189,7 +234,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         lse[((int64_t)b * p.H + h) * nq + q0 + m] = (mrun + log2f(ltot)) * kLn2;
 
     __syncthreads();                                   // tiles are dead; reuse LDS as output stage
-    uint16_t* stage = lds + wave * 32 * L::kRowPitch;
+    constexpr int kSP = D + 8;                         // u16 per staged row
+    uint16_t* stage = (uint16_t*)lds + wave * 32 * kSP;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -197,7 +243,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             u32x2 w;
             w.x = pack2<E>(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
             w.y = pack2<E>(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
-            *(u32x2*)(stage + m * L::kRowPitch + 32 * dt + 8 * g + 4 * hf) = w;
+            *(u32x2*)(stage + m * kSP + 32 * dt + 8 * g + 4 * hf) = w;
         }
     __syncthreads();
     {
@@ -206,7 +252,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int c = lane; c < 32 * CH; c += 64) {
             int r = c / CH, ch = c % CH;
             if (q0 + r < nq) {
-                u32x4 w = *(const u32x4*)(stage + r * L::kRowPitch + ch * 8);
+                u32x4 w = *(const u32x4*)(stage + r * kSP + ch * 8);
                 *(u32x4*)(og + (int64_t)(q0 + r) * p.o_stride[1] + ch * 8) = w;
             }
         }
@@ -291,16 +337,25 @@ int launch_dense(const sfm_dense_desc& d, const void* q, const void* k, const vo
     const bool mfma = (d.dtype == SFM_BF16 || d.dtype == SFM_F16) && (d.D == 64 || d.D == 128);
     if (mfma) {
         dim3 grid((d.q_tokens + 127) / 128, d.B * d.H);
+        const size_t ldsb = d.D == 128 ? DnLds<128>::kTotal : DnLds<64>::kTotal;
+        if (ldsb > 64 * 1024) {
+            const void* fn = d.dtype == SFM_BF16 ? (const void*)dense_fwd_kernel<BF16, 128> : (const void*)dense_fwd_kernel<F16, 128>;
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsb);
+            if (e != hipSuccess) {
+                set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+                return SFM_ERR_HIP;
+            }
+        }
         const uint16_t* qq = (const uint16_t*)q;
         const uint16_t* kk = (const uint16_t*)k;
         const uint16_t* vv = (const uint16_t*)v;
         uint16_t* oo = (uint16_t*)out;
         if (d.dtype == SFM_BF16) {
-            if (d.D == 128) hipLaunchKernelGGL((dense_fwd_kernel<BF16, 128>), grid, dim3(256), 0, stream, d, qq, kk, vv, oo, lse);
-            else hipLaunchKernelGGL((dense_fwd_kernel<BF16, 64>), grid, dim3(256), 0, stream, d, qq, kk, vv, oo, lse);
+            if (d.D == 128) hipLaunchKernelGGL((dense_fwd_kernel<BF16, 128>), grid, dim3(256), ldsb, stream, d, qq, kk, vv, oo, lse);
+            else hipLaunchKernelGGL((dense_fwd_kernel<BF16, 64>), grid, dim3(256), ldsb, stream, d, qq, kk, vv, oo, lse);
         } else {
-            if (d.D == 128) hipLaunchKernelGGL((dense_fwd_kernel<F16, 128>), grid, dim3(256), 0, stream, d, qq, kk, vv, oo, lse);
-            else hipLaunchKernelGGL((dense_fwd_kernel<F16, 64>), grid, dim3(256), 0, stream, d, qq, kk, vv, oo, lse);
+            if (d.D == 128) hipLaunchKernelGGL((dense_fwd_kernel<F16, 128>), grid, dim3(256), ldsb, stream, d, qq, kk, vv, oo, lse);
+            else hipLaunchKernelGGL((dense_fwd_kernel<F16, 64>), grid, dim3(256), ldsb, stream, d, qq, kk, vv, oo, lse);
         }
     } else {
         dim3 grid(d.q_tokens, d.B * d.H);

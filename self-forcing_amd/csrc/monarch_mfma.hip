@@ -3,15 +3,16 @@
 // Two kernels per pass over a group of (batch x head) units:
 //
 //  step 1 (right factor; replaces _al_cl_y_fwd, wan/modules/monarch_attn.py:109-253)
-//      workgroup = (unit, a-chunk, kv block-frame f, a range of block rows k)
-//      for each k: stage K[f,k,:,:], V[f,k,:,:] in LDS once (row-major K for the logits,
-//      transposed K^T / V^T for the contractions), and for ALL query block-frames of the chunk
+//      work item = tile (unit, key block row k, kv block-frame f) against all (a, j) columns of a chunk of query
+//      block-frames; one workgroup per CU, each taking an equal contiguous share of the tile list.
+//      per tile: stage K[f,k,:,:], V[f,k,:,:] in LDS once (row-major K for the logits, transposed K^T / V^T for
+//      the contractions), and for ALL columns of the chunk
 //          S^T[l,(a,j)] = K[f,k,l,:] . Q[a,k,j,:]           (MFMA, wave = 32 (a,j) columns)
 //          R = softmax_l(s S)       cl = sum_l R log2 R      (registers + one cross-half shuffle)
 //          Kbar^T = K^T R^T,  Y^T = V^T R^T                  (MFMA; R^T is fed straight from the
 //                                                             accumulator layout, see perm_row)
-//      rows Kbar[a,j,(f,k),:], Y[a,j,(f,k),:] go to the workspace through an LDS transpose so
-//      that every global store is a full 128-byte line.
+//      rows Kbar[a,j,(f,k),:], Y[a,j,(f,k),:] go to the workspace straight from the accumulators: one
+//      v_permlane32_swap per dword pair leaves 8 consecutive head-dim elements per lane (16-byte stores).
 //
 //  step 2 (left factor; replaces _z_fwd, monarch_attn.py:698-842)
 //      wave = (unit, a, j): streams its contiguous Kbar / Y rows once,
