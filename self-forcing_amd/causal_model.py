@@ -205,6 +205,20 @@ class CausalWanSelfAttention(nn.Module):
         self.norm_q = WanRMSNorm(dim, eps=eps)
         self.norm_k = WanRMSNorm(dim, eps=eps)
         self._rope = None
+        self._qkv = None
+
+    def _project_qkv(self, x):
+        """q, k, v projections as one GEMM over the concatenated weights (the parameters stay the reference's
+        three Linear layers; the concatenation is rebuilt when one of them changes).  The three results are
+        column slices of one [B, S, 3C] tensor, which the prologue reads through its row stride."""
+        ws = (self.q.weight, self.k.weight, self.v.weight)
+        key = tuple((w.data_ptr(), w._version) for w in ws) + (x.dtype, x.device)
+        if self._qkv is None or self._qkv[0] != key:
+            with torch.no_grad():
+                self._qkv = (key, torch.cat(ws, 0).contiguous(), torch.cat((self.q.bias, self.k.bias, self.v.bias), 0).contiguous())
+        y = torch.nn.functional.linear(x, self._qkv[1], self._qkv[2])
+        c = self.dim
+        return y[..., :c], y[..., c:2 * c], y[..., 2 * c:]
 
     def forward(self, x, grid, kv_cache, current_start=0):
         """x [B, S, C] with S = F*h*w tokens of grid = (F, h, w); kv_cache: the reference's per-layer dict."""
@@ -239,7 +253,8 @@ class CausalWanSelfAttention(nn.Module):
         # dense attention keeps the cache in token order (causal_model.py:961-962), Monarch in block order
         tiling = (1, 1, 1) if dense else (f_tied, fl.h_reduce, fl.w_reduce)
 
-        q = self.ops.qk_prologue(self.q(x), self.k(x), self.v(x), self.norm_q.weight, self.norm_k.weight, n, grid,
+        xq, xk, xv = self._project_qkv(x) if not torch.is_grad_enabled() else (self.q(x), self.k(x), self.v(x))
+        q = self.ops.qk_prologue(xq, xk, xv, self.norm_q.weight, self.norm_k.weight, n, grid,
                                  current_start // frame_seqlen, self._rope, kv_cache["k"], kv_cache["v"],
                                  cache_start + local_start, *tiling, eps=self.eps)
         k_view = kv_cache["k"][:, cache_start:cache_start + view_len]
