@@ -176,7 +176,10 @@ int sfm_qk_prologue(const sfm_prologue_desc* desc, const void* xq, const void* x
  *   scale/shift + (row / rows_per_frame) * mod_stride (wan/modules/causal_model.py:1179-1183, 1198-1201), or,
  *   when weight/bias are given (scale = shift = NULL), the affine LayerNorm of norm3 (causal_model.py:1194).
  * sfm_gate_residual: x += y * gate[f] in place (causal_model.py:1189, 1203-1204); gate = NULL gives x += y.
- * sfm_rms_norm: WanRMSNorm (wan/modules/model.py:462-478). */
+ * sfm_rms_norm: WanRMSNorm (wan/modules/model.py:462-478).
+ * sfm_gate_residual_ln: sfm_gate_residual followed by sfm_ln_modulate of the updated rows in one pass (the residual
+ *   update and the next sub-layer's norm, causal_model.py:1189+1194, 1196+1198): x is updated in place, out gets the
+ *   normalised rows. */
 int sfm_ln_modulate(int32_t dtype, int64_t rows, int32_t C, float eps, const void* x, int64_t x_stride, void* y,
                     int64_t y_stride, const void* scale, const void* shift, int64_t mod_stride, int32_t rows_per_frame,
                     const void* weight, const void* bias, void* stream);
@@ -184,6 +187,10 @@ int sfm_gate_residual(int32_t dtype, int64_t rows, int32_t C, void* x, int64_t x
                       const void* gate, int64_t mod_stride, int32_t rows_per_frame, void* stream);
 int sfm_rms_norm(int32_t dtype, int64_t rows, int32_t C, float eps, const void* x, int64_t x_stride, void* y,
                  int64_t y_stride, const void* weight, void* stream);
+int sfm_gate_residual_ln(int32_t dtype, int64_t rows, int32_t C, float eps, void* x, int64_t x_stride, const void* y,
+                         int64_t y_stride, const void* gate, int64_t gate_stride, int32_t gate_rows_per_frame, void* out,
+                         int64_t out_stride, const void* scale, const void* shift, int64_t mod_stride, int32_t rows_per_frame,
+                         const void* weight, const void* bias, void* stream);
 
 /* Thread-local description of the last error returned on this thread ("" if none). */
 const char* sfm_last_error(void);

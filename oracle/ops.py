@@ -54,6 +54,12 @@ class OracleOps:
         nf = gate.shape[1]
         return x + (y.unflatten(1, (nf, x.shape[1] // nf)) * gate).flatten(1, 2)
 
+    def gate_residual_ln(self, x, y, gate, eps, scale=None, shift=None, weight=None, bias=None):
+        x = self.gate_residual(x, y, gate)
+        if weight is not None:
+            return x, self.ln_affine(x, weight, bias, eps)
+        return x, self.ln_modulate(x, scale, shift, eps)
+
     def linear_gelu(self, x, linear):
         return torch.nn.functional.gelu(linear(x), approximate='tanh')
 

@@ -59,6 +59,29 @@ def gate_residual_(x, y, gate=None):
     return x
 
 
+def gate_residual_ln_(x, y, gate=None, scale=None, shift=None, weight=None, bias=None, eps=1e-6):
+    """x += y * gate in place (gate=None: x += y), then returns (x, LayerNorm(x) * (1 + scale) + shift), or the
+    affine LayerNorm when weight / bias are given: one pass over the rows instead of two kernels."""
+    rows, C, xs = _rows(x)
+    _, _, ys = _rows(y)
+    g, gms, grpf = (None, 0, 1) if gate is None else _mod(gate, x)
+    out = torch.empty_like(x, memory_format=torch.contiguous_format)
+    if weight is None:
+        sc, ms, rpf = _mod(scale, x)
+        sh, ms2, _ = _mod(shift, x)
+        if ms2 != ms:
+            sc, sh = sc.contiguous(), sh.contiguous()
+            ms = sc.stride(1)
+        mod = (sc.data_ptr(), sh.data_ptr(), ms, rpf, None, None)
+    else:
+        mod = (None, None, 0, 1, weight.data_ptr(), bias.data_ptr())
+    with torch.cuda.device(x.device):
+        _l.check(_l.load().sfm_gate_residual_ln(_DT[x.dtype], rows, C, eps, x.data_ptr(), xs, y.data_ptr(), ys,
+                                                None if g is None else g.data_ptr(), gms, grpf, out.data_ptr(), C, *mod,
+                                                _stream(x)))
+    return x, out
+
+
 def rms_norm(x, weight, eps=1e-6):
     rows, C, xs = _rows(x)
     y = torch.empty_like(x, memory_format=torch.contiguous_format)

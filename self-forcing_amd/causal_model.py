@@ -64,6 +64,10 @@ class HipAttentionOps:
     def rms_norm(self, x, weight, eps):
         return _blk.rms_norm(x, weight, eps)
 
+    def gate_residual_ln(self, x, y, gate, eps, scale=None, shift=None, weight=None, bias=None):
+        """(x + y * gate, norm of that sum): residual update and the next sub-layer's LayerNorm in one kernel."""
+        return _blk.gate_residual_ln_(x, y if y.stride(2) == 1 else y.contiguous(), gate, scale, shift, weight, bias, eps)
+
     def linear_gelu(self, x, linear):
         """GELU(tanh)(x W^T + b) with the activation applied in the GEMM's epilogue (hipBLASLt through
         torch's addmm-with-activation); the reference runs Linear and nn.GELU(approximate='tanh') apart
@@ -317,13 +321,12 @@ class CausalWanAttentionBlock(nn.Module):
         ops = self.ops
         e = (self.modulation.unsqueeze(1) + e).chunk(6, dim=2)
         y = self.self_attn(ops.ln_modulate(x, e[1], e[0], self.eps), grid, kv_cache, current_start)
-        x = ops.gate_residual(x, y, e[2])
         if isinstance(self.norm3, nn.Identity):
-            xn = x
+            x = xn = ops.gate_residual(x, y, e[2])
         else:
-            xn = ops.ln_affine(x, self.norm3.weight, self.norm3.bias, self.eps)
-        x = ops.gate_residual(x, self.cross_attn(xn, context, crossattn_cache))
-        y = self.ffn[2](ops.linear_gelu(ops.ln_modulate(x, e[4], e[3], self.eps), self.ffn[0]))
+            x, xn = ops.gate_residual_ln(x, y, e[2], self.eps, weight=self.norm3.weight, bias=self.norm3.bias)
+        x, xn = ops.gate_residual_ln(x, self.cross_attn(xn, context, crossattn_cache), None, self.eps, scale=e[4], shift=e[3])
+        y = self.ffn[2](ops.linear_gelu(xn, self.ffn[0]))
         return ops.gate_residual(x, y, e[5])
 
 

@@ -5,8 +5,10 @@
 //                   and no modulation (norm3, causal_model.py:1194)
 //   gate_residual   x += y * gate[frame]                                          (causal_model.py:1189, 1203-1204)
 //   rms_norm        y = (x * rsqrt(mean(x^2) + eps)).type_as(x) * w               (WanRMSNorm, model.py:462-478)
+//   gate_residual_ln  gate_residual followed by ln_modulate of the updated row, one pass over it
 //
-// One workgroup per token row (C <= 8192).  Statistics in fp32; the reference's rounding points are kept:
+// One wave per token row for the normalisations (C <= 8192; the row stays in registers, sums by lane shuffles,
+// no barrier), one workgroup per row for the residual.  Statistics in fp32; the reference's rounding points are kept:
 // every eager op of the reference rounds to the tensor dtype, so the kernels round after the same steps
 // (LayerNorm output, 1 + scale, the product, the sum; y * gate, x + ...).
 
@@ -48,43 +50,38 @@ template <class E> struct V8_16 {
 template <> struct V8<BF16> : V8_16<BF16> {};
 template <> struct V8<F16> : V8_16<F16> {};
 
-constexpr int kMaxChunks = 4;   // 256 threads x 4 chunks x 8 elements = 8192 channels
-
-__device__ __forceinline__ float block_sum(float v, float* red) {
+__device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float s = red[0] + red[1] + red[2] + red[3];
-    __syncthreads();
-    return s;
+    return v;
 }
 
 // x [rows, C] (row stride xs), scale/shift [B, F, C] addressed through (row -> frame) = row / rows_per_frame,
-// with element strides ms (between frames); weight/bias [C] or nullptr.
-template <typename T>
+// with element strides ms (between frames); weight/bias [C] or nullptr.  NT = 8-element chunks per lane.
+template <typename T, int NT>
 __global__ __launch_bounds__(256) void ln_modulate_kernel(const void* x, int64_t xs, void* y, int64_t ys, int C, float eps,
                                                           const void* scale, const void* shift, int64_t ms,
-                                                          int rows_per_frame, const void* weight, const void* bias) {
+                                                          int rows_per_frame, const void* weight, const void* bias, int64_t rows) {
     using V = V8<T>;
-    __shared__ float red[4];
-    const int row = blockIdx.x, tid = threadIdx.x, nch = C / 8;
-    float v[kMaxChunks][8];
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63, nch = C / 8;
+    float v[NT][8];
     float sum = 0.f;
 #pragma unroll
-    for (int t = 0; t < kMaxChunks; ++t) {
-        const int ch = tid + t * 256;
+    for (int t = 0; t < NT; ++t) {
+        const int ch = lane + t * 64;
         if (ch < nch) {
-            V::load(x, (int64_t)row * xs + ch * 8, v[t]);
+            V::load(x, row * xs + ch * 8, v[t]);
 #pragma unroll
             for (int i = 0; i < 8; ++i) sum += v[t][i];
         }
     }
-    const float mean = block_sum(sum, red) / C;
+    const float mean = wave_sum(sum) / C;
     float sq = 0.f;
 #pragma unroll
-    for (int t = 0; t < kMaxChunks; ++t) {
-        const int ch = tid + t * 256;
+    for (int t = 0; t < NT; ++t) {
+        const int ch = lane + t * 64;
         if (ch < nch) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -93,11 +90,11 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const void* x, int64_t
             }
         }
     }
-    const float rstd = 1.0f / sqrtf(block_sum(sq, red) / C + eps);
-    const int64_t moff = (int64_t)(row / rows_per_frame) * ms;
+    const float rstd = 1.0f / sqrtf(wave_sum(sq) / C + eps);
+    const int64_t moff = (row / rows_per_frame) * ms;
 #pragma unroll
-    for (int t = 0; t < kMaxChunks; ++t) {
-        const int ch = tid + t * 256;
+    for (int t = 0; t < NT; ++t) {
+        const int ch = lane + t * 64;
         if (ch < nch) {
             float o[8];
             if (weight != nullptr) {
@@ -117,7 +114,87 @@ __global__ __launch_bounds__(256) void ln_modulate_kernel(const void* x, int64_t
                     o[i] = V::rnd(n * g) + sh[i];
                 }
             }
-            V::store(y, (int64_t)row * ys + ch * 8, o);
+            V::store(y, row * ys + ch * 8, o);
+        }
+    }
+}
+
+// x += y * gate (gate = nullptr: x += y), written back, then out = the LayerNorm variant of ln_modulate_kernel
+// applied to the updated (rounded) row, which never leaves the registers in between.
+template <typename T, int NT>
+__global__ __launch_bounds__(256) void gate_residual_ln_kernel(void* x, int64_t xs, const void* yv, int64_t ys, const void* gate,
+                                                               int64_t gms, int g_rows_per_frame, void* out, int64_t os, int C,
+                                                               float eps, const void* scale, const void* shift, int64_t ms,
+                                                               int rows_per_frame, const void* weight, const void* bias, int64_t rows) {
+    using V = V8<T>;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63, nch = C / 8;
+    const int64_t goff = gate != nullptr ? (row / g_rows_per_frame) * gms : 0;
+    float v[NT][8];
+    float sum = 0.f;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int ch = lane + t * 64;
+        if (ch < nch) {
+            float b[8], g[8];
+            V::load(x, row * xs + ch * 8, v[t]);
+            V::load(yv, row * ys + ch * 8, b);
+            if (gate != nullptr) {
+                V::load(gate, goff + ch * 8, g);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+#pragma clang fp contract(off)      // two eager ops in the reference: no fma
+                    float prod = b[i] * g[i];
+                    v[t][i] = V::rnd(v[t][i] + V::rnd(prod));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[t][i] = V::rnd(v[t][i] + b[i]);
+            }
+            V::store(x, row * xs + ch * 8, v[t]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sum += v[t][i];
+        }
+    }
+    const float mean = wave_sum(sum) / C;
+    float sq = 0.f;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int ch = lane + t * 64;
+        if (ch < nch) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float d = v[t][i] - mean;
+                sq += d * d;
+            }
+        }
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(sq) / C + eps);
+    const int64_t moff = (row / rows_per_frame) * ms;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int ch = lane + t * 64;
+        if (ch < nch) {
+            float o[8];
+            if (weight != nullptr) {
+                float w[8], b[8];
+                V::load(weight, ch * 8, w);
+                V::load(bias, ch * 8, b);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) o[i] = (v[t][i] - mean) * rstd * w[i] + b[i];
+            } else {
+                float sc[8], sh[8];
+                V::load(scale, moff + ch * 8, sc);
+                V::load(shift, moff + ch * 8, sh);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    float n = V::rnd((v[t][i] - mean) * rstd);
+                    float g = V::rnd(1.0f + sc[i]);
+                    o[i] = V::rnd(n * g) + sh[i];
+                }
+            }
+            V::store(out, row * os + ch * 8, o);
         }
     }
 }
@@ -148,33 +225,34 @@ __global__ __launch_bounds__(256) void gate_residual_kernel(void* x, int64_t xs,
     }
 }
 
-template <typename T>
+template <typename T, int NT>
 __global__ __launch_bounds__(256) void rms_norm_kernel(const void* x, int64_t xs, void* y, int64_t ys, int C, float eps,
-                                                       const void* weight) {
+                                                       const void* weight, int64_t rows) {
     using V = V8<T>;
-    __shared__ float red[4];
-    const int row = blockIdx.x, tid = threadIdx.x, nch = C / 8;
-    float v[kMaxChunks][8];
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63, nch = C / 8;
+    float v[NT][8];
     float sq = 0.f;
 #pragma unroll
-    for (int t = 0; t < kMaxChunks; ++t) {
-        const int ch = tid + t * 256;
+    for (int t = 0; t < NT; ++t) {
+        const int ch = lane + t * 64;
         if (ch < nch) {
-            V::load(x, (int64_t)row * xs + ch * 8, v[t]);
+            V::load(x, row * xs + ch * 8, v[t]);
 #pragma unroll
             for (int i = 0; i < 8; ++i) sq += v[t][i] * v[t][i];
         }
     }
-    const float r = 1.0f / sqrtf(block_sum(sq, red) / C + eps);
+    const float r = 1.0f / sqrtf(wave_sum(sq) / C + eps);
 #pragma unroll
-    for (int t = 0; t < kMaxChunks; ++t) {
-        const int ch = tid + t * 256;
+    for (int t = 0; t < NT; ++t) {
+        const int ch = lane + t * 64;
         if (ch < nch) {
             float w[8], o[8];
             V::load(weight, ch * 8, w);
 #pragma unroll
             for (int i = 0; i < 8; ++i) o[i] = V::rnd(v[t][i] * r) * w[i];
-            V::store(y, (int64_t)row * ys + ch * 8, o);
+            V::store(y, row * ys + ch * 8, o);
         }
     }
 }
@@ -195,11 +273,36 @@ static int finish() {
     return SFM_OK;
 }
 
+// wave-per-row kernels: 4 rows per workgroup, NT = chunks of 8 elements per lane (3 covers C <= 1536, 10 C <= 5120)
+#define SFM_DISPATCH_ROWS(dtype, KERNEL, C, rows, stream, ...)                                                      \
+    do {                                                                                                            \
+        const dim3 grid((unsigned)(((rows) + 3) / 4));                                                              \
+        const int nt_ = ((C) / 8 + 63) / 64;                                                                        \
+        if (nt_ <= 3) SFM_DISPATCH_NT(dtype, KERNEL, 3, grid, stream, __VA_ARGS__);                                 \
+        else if (nt_ <= 10) SFM_DISPATCH_NT(dtype, KERNEL, 10, grid, stream, __VA_ARGS__);                          \
+        else SFM_DISPATCH_NT(dtype, KERNEL, 16, grid, stream, __VA_ARGS__);                                         \
+    } while (0)
+#define SFM_DISPATCH_NT(dtype, KERNEL, NT, grid, stream, ...)                                                       \
+    do {                                                                                                            \
+        if ((dtype) == SFM_BF16) hipLaunchKernelGGL((KERNEL<BF16, NT>), grid, dim3(256), 0, stream, __VA_ARGS__);   \
+        else if ((dtype) == SFM_F16) hipLaunchKernelGGL((KERNEL<F16, NT>), grid, dim3(256), 0, stream, __VA_ARGS__); \
+        else hipLaunchKernelGGL((KERNEL<float, NT>), grid, dim3(256), 0, stream, __VA_ARGS__);                      \
+    } while (0)
+
 int launch_ln_modulate(int dtype, int64_t rows, int C, float eps, const void* x, int64_t xs, void* y, int64_t ys,
                        const void* scale, const void* shift, int64_t ms, int rows_per_frame, const void* weight,
                        const void* bias, hipStream_t stream) {
-    SFM_DISPATCH(dtype, ln_modulate_kernel, dim3((unsigned)rows), stream, x, xs, y, ys, C, eps, scale, shift, ms,
-                 rows_per_frame, weight, bias);
+    SFM_DISPATCH_ROWS(dtype, ln_modulate_kernel, C, rows, stream, x, xs, y, ys, C, eps, scale, shift, ms, rows_per_frame,
+                      weight, bias, rows);
+    return finish();
+}
+
+int launch_gate_residual_ln(int dtype, int64_t rows, int C, float eps, void* x, int64_t xs, const void* y, int64_t ys,
+                            const void* gate, int64_t gms, int g_rows_per_frame, void* out, int64_t os, const void* scale,
+                            const void* shift, int64_t ms, int rows_per_frame, const void* weight, const void* bias,
+                            hipStream_t stream) {
+    SFM_DISPATCH_ROWS(dtype, gate_residual_ln_kernel, C, rows, stream, x, xs, y, ys, gate, gms, g_rows_per_frame, out, os, C, eps,
+                      scale, shift, ms, rows_per_frame, weight, bias, rows);
     return finish();
 }
 
@@ -211,7 +314,7 @@ int launch_gate_residual(int dtype, int64_t rows, int C, void* x, int64_t xs, co
 
 int launch_rms_norm(int dtype, int64_t rows, int C, float eps, const void* x, int64_t xs, void* y, int64_t ys,
                     const void* weight, hipStream_t stream) {
-    SFM_DISPATCH(dtype, rms_norm_kernel, dim3((unsigned)rows), stream, x, xs, y, ys, C, eps, weight);
+    SFM_DISPATCH_ROWS(dtype, rms_norm_kernel, C, rows, stream, x, xs, y, ys, C, eps, weight, rows);
     return finish();
 }
 

@@ -29,6 +29,10 @@ bool monarch_generic_supported(const MonarchArgs& a);
 int launch_ln_modulate(int dtype, int64_t rows, int C, float eps, const void* x, int64_t xs, void* y, int64_t ys,
                        const void* scale, const void* shift, int64_t ms, int rows_per_frame, const void* weight,
                        const void* bias, hipStream_t stream);
+int launch_gate_residual_ln(int dtype, int64_t rows, int C, float eps, void* x, int64_t xs, const void* y, int64_t ys,
+                            const void* gate, int64_t gms, int g_rows_per_frame, void* out, int64_t os, const void* scale,
+                            const void* shift, int64_t ms, int rows_per_frame, const void* weight, const void* bias,
+                            hipStream_t stream);
 int launch_gate_residual(int dtype, int64_t rows, int C, void* x, int64_t xs, const void* y, int64_t ys,
                          const void* gate, int64_t ms, int rows_per_frame, hipStream_t stream);
 int launch_rms_norm(int dtype, int64_t rows, int C, float eps, const void* x, int64_t xs, void* y, int64_t ys,
@@ -195,7 +199,7 @@ using namespace sfm;
 
 extern "C" {
 
-int sfm_version(void) { return 3; }
+int sfm_version(void) { return 4; }
 
 const char* sfm_last_error(void) { return g_err; }
 
@@ -738,6 +742,34 @@ int sfm_ln_modulate(int32_t dtype, int64_t rows, int32_t C, float eps, const voi
     }
     return launch_ln_modulate(dtype, rows, C, eps, x, x_stride, y, y_stride, scale, shift, mod_stride,
                               affine ? 1 : rows_per_frame, weight, bias, (hipStream_t)stream);
+}
+
+int sfm_gate_residual_ln(int32_t dtype, int64_t rows, int32_t C, float eps, void* x, int64_t x_stride, const void* y,
+                         int64_t y_stride, const void* gate, int64_t gate_stride, int32_t gate_rows_per_frame, void* out,
+                         int64_t out_stride, const void* scale, const void* shift, int64_t mod_stride, int32_t rows_per_frame,
+                         const void* weight, const void* bias, void* stream) {
+    int rc = check_rows(dtype, rows, C, x_stride, y_stride);
+    if (!rc) rc = check_rows(dtype, rows, C, x_stride, out_stride);
+    if (rc) return rc;
+    const bool affine = weight != nullptr || bias != nullptr;
+    if (!x || !y || !out || (affine && (!weight || !bias)) || (!affine && (!scale || !shift))) {
+        set_error("x, y, out and either (scale, shift) or (weight, bias) must be non-NULL");
+        return SFM_ERR_NULL;
+    }
+    const int esz = dtype == SFM_F32 ? 4 : 2;
+    if ((gate && (gate_rows_per_frame < 1 || gate_stride < 0 || (gate_stride * esz) % 16)) ||
+        (!affine && (rows_per_frame < 1 || mod_stride < 0 || (mod_stride * esz) % 16))) {
+        set_error("rows_per_frame must be >= 1 and modulation strides multiples of 16 bytes");
+        return SFM_ERR_STRIDE;
+    }
+    if (!aligned16(x) || !aligned16(y) || !aligned16(out) || !aligned16(gate) || !aligned16(scale) || !aligned16(shift) ||
+        !aligned16(weight) || !aligned16(bias)) {
+        set_error("tensors must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    return launch_gate_residual_ln(dtype, rows, C, eps, x, x_stride, y, y_stride, gate, gate_stride, gate ? gate_rows_per_frame : 1,
+                                   out, out_stride, scale, shift, mod_stride, affine ? 1 : rows_per_frame, weight, bias,
+                                   (hipStream_t)stream);
 }
 
 int sfm_gate_residual(int32_t dtype, int64_t rows, int32_t C, void* x, int64_t x_stride, const void* y, int64_t y_stride,

@@ -39,6 +39,16 @@ def test_ln_modulate_gate_residual_rms(dtype, B, F, fs, C):
     got = blk.gate_residual_(xd.clone(), yd, chd[2])
     assert torch.equal(got.cpu(), ref)                     # no statistics involved: bit exact
     assert torch.equal(blk.gate_residual_(xd.clone(), yd).cpu(), x + y)
+    # residual update + the next norm in one kernel: the updated rows bit exact, the norm as the separate kernels
+    for gate, gate_d in ((ch[2], chd[2]), (None, None)):
+        xr, nr = o.gate_residual_ln(x, y, gate, 1e-6, scale=ch[4], shift=ch[3])
+        xg, ng = blk.gate_residual_ln_(xd.clone(), yd, gate_d, scale=chd[4], shift=chd[3], eps=1e-6)
+        assert torch.equal(xg.cpu(), xr)
+        _check(ng, nr, dtype)
+    xr, nr = o.gate_residual_ln(x, y, ch[2], 1e-6, weight=w, bias=b)
+    xg, ng = blk.gate_residual_ln_(xd.clone(), yd, chd[2], weight=w.to(DEV), bias=b.to(DEV), eps=1e-6)
+    assert torch.equal(xg.cpu(), xr)
+    _check(ng, nr, dtype)
 
 
 def test_block_ops_reject_bad_layouts():
