@@ -56,6 +56,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int lane = tid & 63;
     const int m = lane & 31;
     const int hf = lane >> 5;
+    const uint32_t piece = (uint32_t)(4 * ((m >> 3) & 1) + 2 * ((m >> 4) & 1) + hf) * 16;   // see the output stores of step 1
 
     uint16_t* const lds = lds_all + grp * L::kElems;
     uint16_t* const lds_krow = lds;                                  // [64][D+8]
@@ -174,7 +175,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     // addresses).  The number of stores between a prefetch and the wait for it is then the same on
     // every path, so that wait leaves the stores in flight instead of draining them.
     u32x4 qb[DS];                                          // logits operand (B): this lane's query row
-    uint32_t crow = 0;                                     // byte offset of this lane's scratch row in its (f, k) slab
+    uint32_t crow[4] = {0, 0, 0, 0};                       // byte offsets in the (f, k) slab of the four scratch rows this lane stores to
     uint32_t cloff = 0;                                    // same for cl
     int qkey = -1;
 
@@ -214,8 +215,13 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds) asm volatile("" : "+v"(qb[ds]));
-            crow = ((uint32_t)(ca * b2 + cj) * p.ws_aj * D + 8 * hf) * 2;
             cloff = (uint32_t)(ca * b2 + cj) * p.ws_aj * 4;
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                const int sg = min(wave * 32 + (m & 7) + 8 * rb, cur.ncols - 1);
+                const int sa = sg / b2;
+                crow[rb] = (uint32_t)((cur.a0 + sa) * b2 + (sg - sa * b2)) * p.ws_aj * (D * 2) + piece;
+            }
         }
         {
             // the tile after this one; past the end of the share the current tile is loaded again and dropped
@@ -286,33 +292,61 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         // contractions with K^T then V^T, 32 head-dim columns at a time.  A 32 x 32 accumulator tile holds,
         // per lane (column c, half hf), head-dim 8g + 4hf + 0..3 for g = 0..3; swapping the g-odd dwords of the
         // lower half with the g-even dwords of the upper half (v_permlane32_swap) leaves 8 consecutive
-        // elements per lane, i.e. 16-byte stores with the two halves of a row side by side.
+        // elements per lane: the 16-byte piece 4 dt + 2 gp + hf of column c's 2D-byte scratch row.  Two more
+        // exchanges, over a pair of head-dim blocks, trade lane bit 4 for gp (v_permlane16_swap) and lane
+        // bit 3 for the block within the pair (a rotation by 8 within rows of 16 lanes).  Afterwards a lane
+        // holds, for each of the four row groups rb, the piece 4 (dt0 + bit 3) + 2 bit 4 + hf of column
+        // (c & 7) + 8 rb, so that one store instruction writes 128 contiguous bytes of each of 8 rows.
 #pragma unroll
         for (int which = 0; which < 2; ++which) {
             const uint16_t* tbase = which == 0 ? lds_kt : lds_vt;
             char* og = (char*)(which == 0 ? p.kbar : p.y) + (size_t)srow * (D * 2);
 #pragma unroll
-            for (int dt = 0; dt < D / 32; ++dt) {
-                f32x16 acc;
+            for (int dp = 0; dp < D / 64; ++dp) {
+                uint32_t w[2][2][4];             // [block in pair][gp][dword]
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-                const uint16_t* arow = tbase + (32 * dt + m) * L::kTPitch + 8 * hf;
+                for (int dl = 0; dl < 2; ++dl) {
+                    const int dt = 2 * dp + dl;
+                    f32x16 acc;
 #pragma unroll
-                for (int st = 0; st < 4; ++st) {
-                    if (st < 2 * NT) {
-                        u32x4 a = *(const u32x4*)(arow + 16 * st);
-                        acc = E::mfma32(a, pb[st], acc);
+                    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+                    const uint16_t* arow = tbase + (32 * dt + m) * L::kTPitch + 8 * hf;
+#pragma unroll
+                    for (int st = 0; st < 4; ++st) {
+                        if (st < 2 * NT) {
+                            u32x4 a = *(const u32x4*)(arow + 16 * st);
+                            acc = E::mfma32(a, pb[st], acc);
+                        }
+                    }
+#pragma unroll
+                    for (int gp = 0; gp < 2; ++gp) {
+                        const int g0 = 2 * gp, g1 = 2 * gp + 1;
+                        auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 0], acc[4 * g0 + 1]),
+                                                                   pack2<E>(acc[4 * g1 + 0], acc[4 * g1 + 1]), false, false);
+                        auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 2], acc[4 * g0 + 3]),
+                                                                   pack2<E>(acc[4 * g1 + 2], acc[4 * g1 + 3]), false, false);
+                        w[dl][gp][0] = rx[0]; w[dl][gp][1] = ry[0]; w[dl][gp][2] = rx[1]; w[dl][gp][3] = ry[1];
+                    }
+                    // lane bit 4 <-> gp: slot 0 then holds rows (c & 15), slot 1 rows (c & 15) + 16
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        auto r = __builtin_amdgcn_permlane16_swap(w[dl][0][q], w[dl][1][q], false, false);
+                        w[dl][0][q] = r[0]; w[dl][1][q] = r[1];
                     }
                 }
+                // lane bit 3 <-> block within the pair
 #pragma unroll
-                for (int gp = 0; gp < 2; ++gp) {
-                    const int g0 = 2 * gp, g1 = 2 * gp + 1;
-                    auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 0], acc[4 * g0 + 1]),
-                                                               pack2<E>(acc[4 * g1 + 0], acc[4 * g1 + 1]), false, false);
-                    auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 2], acc[4 * g0 + 3]),
-                                                               pack2<E>(acc[4 * g1 + 2], acc[4 * g1 + 3]), false, false);
-                    u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
-                    *(u32x4*)(og + crow + (32 * dt + 16 * gp) * 2) = w;
+                for (int r4 = 0; r4 < 2; ++r4) {
+                    u32x4 lo, hi;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t a = w[0][r4][q], b = w[1][r4][q];
+                        // row_ror:8 within 16 lanes; bank mask 0xc writes lanes 8..15 of a row, 0x3 lanes 0..7
+                        lo[q] = (uint32_t)__builtin_amdgcn_update_dpp((int)a, (int)b, 0x128, 0xf, 0xc, false);
+                        hi[q] = (uint32_t)__builtin_amdgcn_update_dpp((int)b, (int)a, 0x128, 0xf, 0x3, false);
+                    }
+                    *(u32x4*)(og + crow[2 * r4 + 0] + 128 * dp) = lo;
+                    *(u32x4*)(og + crow[2 * r4 + 1] + 128 * dp) = hi;
                 }
             }
         }
