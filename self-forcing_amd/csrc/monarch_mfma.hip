@@ -345,8 +345,11 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                         lo[q] = (uint32_t)__builtin_amdgcn_update_dpp((int)a, (int)b, 0x128, 0xf, 0xc, false);
                         hi[q] = (uint32_t)__builtin_amdgcn_update_dpp((int)b, (int)a, 0x128, 0xf, 0x3, false);
                     }
-                    *(u32x4*)(og + crow[2 * r4 + 0] + 128 * dp) = lo;
-                    *(u32x4*)(og + crow[2 * r4 + 1] + 128 * dp) = hi;
+// Non-temporal: the rows are read exactly once, by step 2, after the whole grid has finished.
+                    // Ordinary stores leave them dirty in the caches and their write-back then competes with
+                    // step 2's reads (measured at 4680 x 32760, 12 heads: step 1 +15 us, step 2 -45 us).
+                    __builtin_nontemporal_store(lo, (u32x4*)(og + crow[2 * r4 + 0] + 128 * dp));
+                    __builtin_nontemporal_store(hi, (u32x4*)(og + crow[2 * r4 + 1] + 128 * dp));
                 }
             }
         }
