@@ -5,13 +5,14 @@
 // (wan/modules/attn_patch.py:20-110).
 //
 // MFMA kernel (bf16 / fp16, head_dim 64 or 128): workgroup = 128 queries of one (batch, head),
-// wave = 32 queries.  Per 64-key tile (K and V rows staged once in LDS, row-major, 16-byte chunks
-// XOR-swizzled):
+// wave = 32 queries.  Per 64-key tile (K and V rows in LDS, row-major, 16-byte chunks XOR-swizzled):
 //     S^T[l, q] = K[l,:] . Q[q,:]          online softmax per query column (lane)
 //     O^T[d, q] += V^T[d, l] P^T[l, q]     V^T comes from transposing LDS reads (ds_read_tr16_b64), P^T from the
 //                                          accumulator layout (perm_row)
-// Two LDS buffers: the next tile's rows are fetched into registers while the current one is consumed and
-// written to the other buffer at the end of the iteration, so there is one barrier per tile.
+// Tiles go from global memory straight into LDS (global_load_lds_dwordx4), two K and two V buffers, one
+// barrier per tile.  A wave's matrix and vector work are interleaved in its instruction stream: the logits of
+// tile n + 1 are contracted while the exponentials of tile n are taken, and the maximum of tile n + 1 is reduced
+// while tile n's P V products run.
 
 #include "sfm_common.hpp"
 
@@ -22,9 +23,9 @@ struct DnLds {
     static constexpr int kCPR = D / 8;                  // 16-byte chunks per row
     static constexpr int kPitch = 2 * D;                // bytes per row
     static constexpr int kMat = 64 * kPitch;            // one 64-row tile
-    static constexpr int kBuf = 2 * kMat;               // K tile, V tile
+    static constexpr int kK = 0, kV = 2 * kMat;         // K tiles 0/1, then V tiles 0/1
     static constexpr int kStage = 4 * 32 * (2 * D + 16);   // output staging, 4 waves x 32 rows
-    static constexpr int kTotal = 2 * kBuf > kStage ? 2 * kBuf : kStage;
+    static constexpr int kTotal = 4 * kMat > kStage ? 4 * kMat : kStage;
     // chunk c of row r sits at chunk position c ^ swz(r); depends on r mod 16 only
     static __device__ __forceinline__ int swz(int r) {
         return D >= 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
@@ -41,6 +42,15 @@ __device__ __forceinline__ u32x2 dn_read_tr(const char* lds, uint32_t off) {
     return __builtin_bit_cast(u32x2, v);
 }
 
+// 16 bytes per lane from global memory into LDS without passing through registers: lane i of the wave reads
+// base + off (off per lane, unsigned 32 bit) and writes LDS bytes [lds_addr + 16 i, + 16).  `base` and `lds_addr`
+// are the same in every lane.  The load counts in vmcnt like any other; the compiler does not know that it
+// writes LDS, so the code that reads the tile waits (dn_wait_tiles) and synchronises explicitly.
+__device__ __forceinline__ void dn_load_lds16(const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void dn_wait_tiles() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 template <class E, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void dense_fwd_kernel(sfm_dense_desc p, const uint16_t* __restrict__ q,
                                                         const uint16_t* __restrict__ kp,
@@ -49,8 +59,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     using L = DnLds<D>;
     constexpr int DS = D / 16, DT = D / 32;
     extern __shared__ __attribute__((aligned(256))) char lds[];
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, m = lane & 31, hf = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
     const int q0 = blockIdx.x * 128 + wave * 32;
     const int nq = p.q_tokens, nk = p.kv_tokens;
@@ -66,36 +78,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const uint16_t* qrow = q + (int64_t)b * p.q_stride[0] + (int64_t)qi * p.q_stride[1] + (int64_t)h * p.q_stride[2] + 8 * hf;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) asm volatile("" : "+v"(qb[ds]));      // loaded before any tile is awaited
     }
 
-    // staging: thread `tid` moves chunks tid, tid + 256, ... of the K tile and the same ones of the V tile.
-    // LDS position P (16-byte units) holds global chunk (P % kCPR) ^ swz(row) of row P / kCPR.  Rows past the
-    // last key repeat the last key (their logits are masked).
+    // staging: thread `tid` moves chunks tid, tid + 256, ... of a tile.  LDS position P (16-byte units) holds
+    // global chunk (P % kCPR) ^ swz(row) of row P / kCPR; a wave's 64 positions are contiguous.  Chunk i of a
+    // thread is kRPC rows below chunk i - 1 in the same (swizzled) column, so one per-thread byte offset serves
+    // all of them and everything else (tile, i) goes into the scalar base address.
     constexpr int kCh = 64 * L::kCPR / 256;            // 4 for D = 128, 2 for D = 64
-    int srow[kCh];
-    uint32_t scol[kCh];
+    constexpr int kRPC = 256 / L::kCPR;                // rows between a thread's consecutive chunks (multiple of 16)
+    const int srow = tid / L::kCPR;
+    const uint32_t scol = (uint32_t)(((tid % L::kCPR) ^ L::swz(srow)) * 16);
+    const uint32_t koff = (uint32_t)srow * krs + scol, voff = (uint32_t)srow * vrs + scol;
+    // full tile
+    auto stage = [&](const char* g, uint32_t rs, uint32_t off, int tile, uint32_t dst) {
 #pragma unroll
-    for (int i = 0; i < kCh; ++i) {
-        const int P = tid + i * 256;
-        srow[i] = P / L::kCPR;
-        scol[i] = (uint32_t)(((P % L::kCPR) ^ L::swz(srow[i])) * 16);
-    }
-    u32x4 sk[kCh], sv[kCh];
-    auto prefetch = [&](int l0) {
-        const int last = nk - 1 - l0;                  // >= 0
-#pragma unroll
-        for (int i = 0; i < kCh; ++i) {
-            const uint32_t r = (uint32_t)(l0 + min(srow[i], last));
-            sk[i] = *(const u32x4*)(kg + (size_t)r * krs + scol[i]);
-            sv[i] = *(const u32x4*)(vg + (size_t)r * vrs + scol[i]);
-        }
+        for (int i = 0; i < kCh; ++i)
+            dn_load_lds16(g + (size_t)(tile * 64 + i * kRPC) * rs, off, lds0 + dst + (uint32_t)(i * 256 + wave * 64) * 16);
     };
-    auto commit = [&](uint32_t buf) {
+    // possibly ragged tile: rows past the last key repeat the last key (their logits are masked)
+    auto stage_clamped = [&](const char* g, uint32_t rs, int tile, uint32_t dst) {
+        const char* base = g + (size_t)tile * 64 * rs;
+        const int last = nk - 1 - 64 * tile;           // >= 0
 #pragma unroll
-        for (int i = 0; i < kCh; ++i) {
-            *(u32x4*)(lds + buf + (tid + i * 256) * 16) = sk[i];
-            *(u32x4*)(lds + buf + L::kMat + (tid + i * 256) * 16) = sv[i];
-        }
+        for (int i = 0; i < kCh; ++i)
+            dn_load_lds16(base, (uint32_t)min(srow + i * kRPC, last) * rs + scol, lds0 + dst + (uint32_t)(i * 256 + wave * 64) * 16);
     };
 
     // logits: A operand = K rows; lane (m, hf) reads chunk 2 ds + hf of row 32 t + m
@@ -103,18 +111,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // output: A operand = V^T.  For head-dim rows 32 dt + 0..31 and contraction step st lane (m, hf) needs keys
     // l = 16 st + 4 hf + {0..3} and + 8 + {0..3} (the order in which the logits' accumulators hold l) of
     // head-dim column 32 dt + m: two transposing reads.
-    uint32_t trA[DT][2];
+    // Head-dim block dt only changes chunk bits 2..3 of the (swizzled) chunk index: address ^ (dt << 6).
+    uint32_t trA[2];
     {
         const int s16 = lane & 15, g16 = lane >> 4;
         const int rl = 4 * hf + (s16 >> 2);
         const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int r = rl + 8 * half, c = 4 * dt + cl;
-                trA[dt][half] = L::kMat + (uint32_t)r * L::kPitch + (uint32_t)((c ^ L::swz(r)) << 4) + (uint32_t)(s16 & 1) * 8;
-            }
+        for (int half = 0; half < 2; ++half) {
+            const int r = rl + 8 * half;
+            trA[half] = (uint32_t)r * L::kPitch + (uint32_t)((cl ^ L::swz(r)) << 4) + (uint32_t)(s16 & 1) * 8;
+        }
     }
 
     f32x16 oacc[DT];
@@ -125,108 +132,165 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     float mrun = -INFINITY, lrun = 0.f;            // running max (scaled, base-2 units) and sum
     const float sc2 = p.sm_scale * kLog2e;
     const int ntile = (nk + 63) / 64;
+    const int lrem = nk - 64 * (ntile - 1);        // valid keys of the last tile (1..64)
 
-    prefetch(0);
-    commit(0);
-    for (int tile = 0; tile < ntile; ++tile) {
-        const uint32_t buf = (uint32_t)(tile & 1) * L::kBuf;
-        lds_barrier();                   // this tile is in LDS; the other buffer is free again
-        if (tile + 1 < ntile) prefetch(64 * (tile + 1));
+    // Both phases of an iteration are sequences of steps, one MFMA each, with the step's A operand read from
+    // LDS kAhead steps earlier into a ring of registers and a slice of the vector work beside it.
+    constexpr int NA = 2 * DS;                     // logits steps: (ds, t) = (j / 2, j % 2)
+    constexpr int NP = 4 * DT;                     // output steps: (dt, st) = (j / 4, j % 4)
+    constexpr int kVA = 32 / NA;                   // logits per lane exponentiated beside one logits step
+    constexpr int kVP = 32 / NP;                   // logits per lane reduced beside one output step
+    constexpr int kAhead = 3, kRing = kAhead + 1;
 
-        // LDS reads are issued a batch ahead of the MFMAs that use them (the fences keep that order)
-        f32x16 s[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) s[t][v] = 0.f;
-        const uint32_t sA = sA0 + buf;
-        constexpr int kB = 2;
-        u32x4 sa[2][kB][2];
-        auto load_s = [&](int ds0, u32x4 (*dst)[2]) {
-#pragma unroll
-            for (int i = 0; i < kB; ++i)
-#pragma unroll
-                for (int t = 0; t < 2; ++t) dst[i][t] = *(const u32x4*)(lds + ((sA ^ (uint32_t)((ds0 + i) << 5)) + t * 32 * L::kPitch));
-        };
-        u32x4 ops[2][4];
-        auto load_ops = [&](int dt, u32x4* dst) {
-            const uint32_t a0 = trA[dt][0] + buf, a1 = trA[dt][1] + buf;
-#pragma unroll
-            for (int st = 0; st < 4; ++st) {
-                const u32x2 lo = dn_read_tr(lds, a0 + st * 16 * L::kPitch);
-                const u32x2 hi = dn_read_tr(lds, a1 + st * 16 * L::kPitch);
-                dst[st] = u32x4{lo.x, lo.y, hi.x, hi.y};
-            }
-        };
-        load_s(0, sa[0]);
-#pragma unroll
-        for (int bt = 0; bt < DS / kB; ++bt) {
-            if (bt + 1 < DS / kB) load_s((bt + 1) * kB, sa[(bt + 1) & 1]);
-            else load_ops(0, ops[0]);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 0; i < kB; ++i)
-#pragma unroll
-                for (int t = 0; t < 2; ++t) s[t] = E::mfma32(sa[bt & 1][i][t], qb[bt * kB + i], s[t]);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // online softmax in base 2; the scale is folded into the exponent argument (one fma per logit)
-        const int lrem = nk - 64 * tile;           // valid keys in this tile (>= 1)
-        if (lrem < 64) {                           // ragged last tile only (wave-uniform)
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    int l = 32 * t + 8 * (v >> 2) + 4 * hf + (v & 3);
-                    s[t][v] = l < lrem ? s[t][v] : kMaskLogit;
-                }
-        }
-        float mx = s[0][0];
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[t][v]);
-        mx = xhalf_max(mx) * sc2;
-        const float mnew = fmaxf(mrun, mx);
-        float psum = 0.f;
+    // `kbuf` / `vbuf` are constants, so that they and the row offsets go into the instructions' offset fields
+    auto read_k = [&](uint32_t kbuf, int j) -> u32x4 {
+        return *(const u32x4*)(lds + (sA0 ^ (uint32_t)((j >> 1) << 5)) + kbuf + (j & 1) * 32 * L::kPitch);
+    };
+    auto read_v = [&](uint32_t vbuf, int j) -> u32x4 {
+        const u32x2 lo = dn_read_tr(lds + (trA[0] ^ (uint32_t)((j >> 2) << 6)), vbuf + (j & 3) * 16 * L::kPitch);
+        const u32x2 hi = dn_read_tr(lds + (trA[1] ^ (uint32_t)((j >> 2) << 6)), vbuf + (j & 3) * 16 * L::kPitch);
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+    };
+    auto mask_tail = [&](f32x16* s) {              // logits of the keys past the end of a ragged last tile
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                float e = fast_exp2(fmaf(s[t][v], sc2, -mnew));
-                psum += e;
-                s[t][v] = e;
+                const int l = 32 * t + 8 * (v >> 2) + 4 * hf + (v & 3);
+                s[t][v] = l < lrem ? s[t][v] : kMaskLogit;
             }
-        u32x4 pb[4];
+    };
+    // value i (0..31) of a lane's logits, in the order the P^T operands take them
+#define DN_SVAL(s, i) s[(i) >> 4][(i) & 15]
+
+    f32x16 sbuf[2][2];                             // logits of tile n in sbuf[n & 1]
+    u32x4 ring[kRing];                             // A operands on their way from LDS
+    u32x4 pb[4];
+
+    // ---- prologue: tile 0 (and K of tile 1) into LDS, logits and maximum of tile 0
+    stage_clamped(kg, krs, 0, L::kK);
+    stage_clamped(vg, vrs, 0, L::kV);
+    if (ntile > 1) stage_clamped(kg, krs, 1, L::kK + L::kMat);
+    dn_wait_tiles();
 #pragma unroll
-        for (int st = 0; st < 4; ++st) {
-            const int t = st >> 1, v0 = 8 * (st & 1);
-            pb[st].x = pack2<E>(s[t][v0 + 0], s[t][v0 + 1]);
-            pb[st].y = pack2<E>(s[t][v0 + 2], s[t][v0 + 3]);
-            pb[st].z = pack2<E>(s[t][v0 + 4], s[t][v0 + 5]);
-            pb[st].w = pack2<E>(s[t][v0 + 6], s[t][v0 + 7]);
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sbuf[0][t][v] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NA; ++j) sbuf[0][j & 1] = E::mfma32(read_k(L::kK, j), qb[j >> 1], sbuf[0][j & 1]);
+    if (ntile == 1 && lrem < 64) mask_tail(sbuf[0]);
+    {
+        float mx = sbuf[0][0][0];
+#pragma unroll
+        for (int i = 1; i < 32; ++i) mx = fmaxf(mx, DN_SVAL(sbuf[0], i));
+        mrun = xhalf_max(mx) * sc2;
+    }
+
+    // One iteration consumes tile n (logits in sbuf[n & 1], maximum already folded into mrun) and, unless it is
+    // the last one, produces the logits of tile n + 1.  PAR = n & 1 fixes every LDS buffer at compile time.
+    // kind 0: the last tile; 1: any other tile; 2: a tile at least three before the last one (the tiles it
+    // fetches are full ones: no tests, no clamping)
+    auto iteration = [&](int n, auto par_c, auto kind_c) {
+        constexpr int PAR = decltype(par_c)::value, kind = decltype(kind_c)::value;
+        constexpr bool has_next = kind != 0;
+        constexpr uint32_t kbuf = L::kK + (uint32_t)(PAR ^ 1) * L::kMat;     // K of tile n + 1; K of n + 2 goes where K of n was
+        constexpr uint32_t vbuf = L::kV + (uint32_t)PAR * L::kMat;           // V of tile n; V of n + 1 goes to the other one
+        f32x16* scur = sbuf[PAR];
+        f32x16* snext = sbuf[PAR ^ 1];
+        dn_wait_tiles();                 // K(n+1) and V(n) are in LDS; the buffers of K(n) and V(n-1) are free
+        if (kind == 2) {
+            stage(kg, krs, koff, n + 2, L::kK + (uint32_t)PAR * L::kMat);
+            stage(vg, vrs, voff, n + 1, L::kV + (uint32_t)(PAR ^ 1) * L::kMat);
+        } else if (kind == 1) {
+            // only the last tile can be ragged
+            if (n + 3 < ntile) stage(kg, krs, koff, n + 2, L::kK + (uint32_t)PAR * L::kMat);
+            else if (n + 3 == ntile) stage_clamped(kg, krs, n + 2, L::kK + (uint32_t)PAR * L::kMat);
+            if (n + 2 < ntile) stage(vg, vrs, voff, n + 1, L::kV + (uint32_t)(PAR ^ 1) * L::kMat);
+            else stage_clamped(vg, vrs, n + 1, L::kV + (uint32_t)(PAR ^ 1) * L::kMat);
         }
-        // rescale the running output only when some query of the wave raised its maximum
-        if (__builtin_amdgcn_ballot_w64(mnew > mrun) != 0) {
-            const float alpha = fast_exp2(mrun - mnew);
-            lrun *= alpha;
+
+        // phase A: logits of tile n + 1 beside the exponentials of tile n
+        float psum = 0.f;
+        if (has_next) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
-            mrun = mnew;
+                for (int v = 0; v < 16; ++v) snext[t][v] = 0.f;
+#pragma unroll
+            for (int j = 0; j < kAhead; ++j) ring[j % kRing] = read_k(kbuf, j);
+        } else {
+#pragma unroll
+            for (int j = 0; j < kAhead; ++j) ring[(NA + j) % kRing] = read_v(vbuf, j);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < NA; ++j) {
+            if (has_next) {
+                const int ja = j + kAhead;
+                if (ja < NA) ring[ja % kRing] = read_k(kbuf, ja);
+                else ring[ja % kRing] = read_v(vbuf, ja - NA);
+                snext[j & 1] = E::mfma32(ring[j % kRing], qb[j >> 1], snext[j & 1]);
+            }
+#pragma unroll
+            for (int i = kVA * j; i < kVA * (j + 1); ++i) {
+                const float e = fast_exp2(fmaf(DN_SVAL(scur, i), sc2, -mrun));
+                psum += e;
+                DN_SVAL(scur, i) = e;
+            }
+#pragma unroll
+            for (int i = kVA * j; i < kVA * (j + 1); i += 2) pb[i >> 3][(i >> 1) & 3] = pack2<E>(DN_SVAL(scur, i), DN_SVAL(scur, i + 1));
+            __builtin_amdgcn_sched_barrier(0);
         }
         lrun += psum;
+        if (kind == 1) {
+            if (n + 2 == ntile && lrem < 64) mask_tail(snext);
+        }
+
+        // phase B: P V of tile n beside the maximum of tile n + 1
+        float mx = has_next ? snext[0][0] : 0.f;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            if (dt + 1 < DT) load_ops(dt + 1, ops[(dt + 1) & 1]);
-            __builtin_amdgcn_sched_barrier(0);
+        for (int j = 0; j < NP; ++j) {
+            if (j + kAhead < NP) ring[(NA + j + kAhead) % kRing] = read_v(vbuf, j + kAhead);
+            oacc[j >> 2] = E::mfma32(ring[(NA + j) % kRing], pb[j & 3], oacc[j >> 2]);
+            if (has_next) {
 #pragma unroll
-            for (int st = 0; st < 4; ++st) oacc[dt] = E::mfma32(ops[dt & 1][st], pb[st], oacc[dt]);
+                for (int i = kVP * j; i < kVP * (j + 1); ++i) mx = fmaxf(mx, DN_SVAL(snext, i));
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (tile + 1 < ntile) commit(buf ^ L::kBuf);
+        if (has_next) {
+            // rescale the running output only when some query of the wave raised its maximum
+            const float mnew = fmaxf(mrun, xhalf_max(mx) * sc2);
+            if (__builtin_amdgcn_ballot_w64(mnew > mrun) != 0) {
+                const float alpha = fast_exp2(mrun - mnew);
+                lrun *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
+                mrun = mnew;
+            }
+        }
+    };
+    using c0 = std::integral_constant<int, 0>;
+    using c1 = std::integral_constant<int, 1>;
+    using c2 = std::integral_constant<int, 2>;
+    int n = 0;
+    for (; n + 4 < ntile; n += 2) {
+        iteration(n, c0{}, c2{});
+        iteration(n + 1, c1{}, c2{});
     }
+    for (; n + 2 < ntile; n += 2) {                // at most once
+        iteration(n, c0{}, c1{});
+        iteration(n + 1, c1{}, c1{});
+    }
+    if (n + 1 < ntile) {
+        iteration(n, c0{}, c1{});
+        iteration(n + 1, c1{}, c0{});
+    } else {
+        iteration(n, c0{}, c0{});
+    }
+#undef DN_SVAL
 
     const float ltot = xhalf_sum(lrun);
     const float inv = 1.f / ltot;
@@ -235,7 +299,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     __syncthreads();                                   // tiles are dead; reuse LDS as output stage
     constexpr int kSP = D + 8;                         // u16 per staged row
-    uint16_t* stage = (uint16_t*)lds + wave * 32 * kSP;
+    uint16_t* stage_o = (uint16_t*)lds + wave * 32 * kSP;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -243,7 +307,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             u32x2 w;
             w.x = pack2<E>(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
             w.y = pack2<E>(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
-            *(u32x2*)(stage + m * kSP + 32 * dt + 8 * g + 4 * hf) = w;
+            *(u32x2*)(stage_o + m * kSP + 32 * dt + 8 * g + 4 * hf) = w;
         }
     __syncthreads();
     {
@@ -252,7 +316,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int c = lane; c < 32 * CH; c += 64) {
             int r = c / CH, ch = c % CH;
             if (q0 + r < nq) {
-                u32x4 w = *(const u32x4*)(stage + r * kSP + ch * 8);
+                u32x4 w = *(const u32x4*)(stage_o + r * kSP + ch * 8);
                 *(u32x4*)(og + (int64_t)(q0 + r) * p.o_stride[1] + ch * 8) = w;
             }
         }
