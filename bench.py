@@ -133,6 +133,11 @@ def op_level(torch, sfa, args):
         torch.cuda.synchronize()
         bwd_ms = (time.perf_counter() - t0) * 1e3
 
+    # what the matrix pipes sustain on this machine (independent MFMAs only), to read the dense figure against
+    probe = C.c_float(0)
+    L.check(lib.sfm_probe_mfma_bf16(20000, stream, C.byref(probe)))
+    dense_tfl = DENSE_FLOPS / (dense_ms * 1e-3) / 1e12
+
     if args.copy_probe:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -150,8 +155,8 @@ def op_level(torch, sfa, args):
                          "kernel_ms": {"monarch_step1": s1_ms, "monarch_step2": s2_ms}},
         "monarch_bwd": {"workload": "gradients of q and of all 21 cached K/V frames at the same shape (fp32 kernels)",
                         "ms_per_call": bwd_ms},
-        "dense_fallback": {"ms_per_call": dense_ms, "tflops": DENSE_FLOPS / (dense_ms * 1e-3) / 1e12,
-                           "mfma_frac": DENSE_FLOPS / (dense_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS},
+        "dense_fallback": {"ms_per_call": dense_ms, "tflops": dense_tfl, "mfma_frac": dense_tfl / MFMA_BF16_PEAK_TFLOPS,
+                           "mfma_probe_tflops": probe.value, "frac_of_probe": dense_tfl / probe.value},
         "roofline": {"kernel": "monarch_step1_kernel (configs[1] shape)", "bound": "hbm", "achieved": s1_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s1_gbs / HBM_PEAK_GBS,
                      "algorithmic_bytes": STEP1_BYTES, "traffic": MEASURED_TRAFFIC["monarch_step1_kernel"]},

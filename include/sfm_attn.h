@@ -192,6 +192,11 @@ int sfm_gate_residual_ln(int32_t dtype, int64_t rows, int32_t C, float eps, void
                          int64_t out_stride, const void* scale, const void* shift, int64_t mod_stride, int32_t rows_per_frame,
                          const void* weight, const void* bias, void* stream);
 
+/* Measurement aid with no counterpart in the reference: runs a stream of independent 32x32x16 bf16 MFMAs (two waves
+ * per SIMD, `iters` x 16 per wave) on `stream`, waits for it and returns the sustained rate in TFLOP/s.  bench.py
+ * reports the dense kernel against it beside the nominal peak. */
+int sfm_probe_mfma_bf16(int32_t iters, void* stream, float* tflops);
+
 /* Thread-local description of the last error returned on this thread ("" if none). */
 const char* sfm_last_error(void);
 

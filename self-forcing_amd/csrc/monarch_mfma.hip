@@ -560,7 +560,7 @@ bool monarch_mfma_supported(int dtype, int D, int b2) {
     return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 >= 1 && b2 <= 64;
 }
 
-static int cu_count() {
+int cu_count() {
     static thread_local int cached_dev = -1, cached = 0;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 256;

@@ -1,0 +1,84 @@
+// Measurement aid: what the matrix pipes of this device sustain on a stream of independent bf16 MFMAs.
+// bench.py reports the dense kernel against this figure next to the nominal peak.
+
+#include <hip/hip_runtime.h>
+
+#include "sfm_attn.h"
+#include "sfm_common.hpp"
+
+// External linkage, so that the store in the kernel (and with it the MFMA chain) cannot be dropped as unobservable.
+__device__ float sfm_probe_sink[1];
+
+namespace sfm {
+namespace {
+
+__global__ __launch_bounds__(256) void mfma_probe_kernel(int iters) {
+    f32x16 acc[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[a][v] = 0.f;
+    // operands: pseudo-random bf16 values of either sign with magnitudes in [0.125, 2), one set per chain (what the
+    // pipes sustain depends on the data: all-small operands toggle few bits and clock higher)
+    auto rnd16 = [](uint32_t h) {
+        h *= 2654435761u;
+        h ^= h >> 15;
+        h *= 2246822519u;
+        h ^= h >> 13;
+        return (uint32_t)(((h & 1u) << 15) | ((0x7cu + ((h >> 1) & 3u)) << 7) | ((h >> 3) & 0x7fu));
+    };
+    auto rnd32 = [&](uint32_t h) { return rnd16(2 * h) | (rnd16(2 * h + 1) << 16); };
+    u32x4 x[4], y;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        const uint32_t h = (threadIdx.x * 4 + a) * 4;
+        x[a] = u32x4{rnd32(h), rnd32(h + 1), rnd32(h + 2), rnd32(h + 3)};
+    }
+    y = u32x4{rnd32(77777 + threadIdx.x * 4), rnd32(77778 + threadIdx.x * 4), rnd32(77779 + threadIdx.x * 4), rnd32(77780 + threadIdx.x * 4)};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int a = 0; a < 4; ++a) acc[a] = BF16::mfma32(x[a], y, acc[a]);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s += acc[a][v];
+    if (s == 12345.678f) sfm_probe_sink[0] = s;                 // keeps the accumulators alive; never true in practice
+}
+
+}  // namespace
+}  // namespace sfm
+
+extern "C" int sfm_probe_mfma_bf16(int32_t iters, void* stream, float* tflops) {
+    using namespace sfm;
+    if (iters < 1 || iters > (1 << 20) || tflops == nullptr) {
+        set_error("sfm_probe_mfma_bf16: iters must be in [1, 2^20] and tflops non-null");
+        return SFM_ERR_RANGE;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int wgs = 2 * cu_count();                          // two waves per SIMD
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        set_error("sfm_probe_mfma_bf16: hipEventCreate failed");
+        return SFM_ERR_HIP;
+    }
+    hipLaunchKernelGGL(mfma_probe_kernel, dim3(wgs), dim3(256), 0, st, iters);          // warm-up
+    hipEventRecord(e0, st);
+    hipLaunchKernelGGL(mfma_probe_kernel, dim3(wgs), dim3(256), 0, st, iters);
+    hipEventRecord(e1, st);
+    hipError_t e = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    if (e != hipSuccess || ms <= 0.f) {
+        set_error("sfm_probe_mfma_bf16: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    const double flops = (double)wgs * 4 * (double)iters * 16 * (2.0 * 32 * 32 * 16);
+    *tflops = (float)(flops / (ms * 1e-3) / 1e12);
+    return SFM_OK;
+}

@@ -180,5 +180,6 @@ size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits);
 int launch_monarch_bwd_gemm(const MonarchBwdArgs& g, int dtype, int nunits, void* workspace, hipStream_t stream);
 
 void set_error(const char* fmt, ...);
+int cu_count();                                  // compute units of the current device (cached per thread)
 
 }  // namespace sfm

@@ -159,3 +159,11 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(L, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         L.load()
+
+
+def test_mfma_probe_rejects_bad_arguments_before_any_launch():
+    lib = L.load()
+    out = C.c_float(0)
+    assert lib.sfm_probe_mfma_bf16(0, None, C.byref(out)) == -4
+    assert lib.sfm_probe_mfma_bf16(100, None, None) == -4
+    assert b"iters" in lib.sfm_last_error()

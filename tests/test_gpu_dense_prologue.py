@@ -123,3 +123,13 @@ def test_prologue_then_monarch_c2_pipeline():
     assert_close_16bit(out[:, :, heads], ref, torch.bfloat16)
     dn = sfa.attention.attention(qd, kc, vc)
     print(f"C2 monarch vs dense: max-abs {max_abs(out, dn):.3e}")
+
+
+@pytest.mark.gpu
+def test_mfma_probe_reports_a_rate():
+    import ctypes as C
+    from self_forcing_amd import lib as L
+    lib = L.load()
+    out = C.c_float(0)
+    L.check(lib.sfm_probe_mfma_bf16(2000, None, C.byref(out)))
+    assert 10.0 < out.value < 5000.0       # TFLOP/s; the nominal peak is 2500
