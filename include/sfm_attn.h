@@ -192,6 +192,26 @@ int sfm_gate_residual_ln(int32_t dtype, int64_t rows, int32_t C, float eps, void
                          int64_t out_stride, const void* scale, const void* shift, int64_t mod_stride, int32_t rows_per_frame,
                          const void* weight, const void* bias, void* stream);
 
+typedef struct sfm_conv_desc {
+    int32_t dtype;            /* SFM_BF16 | SFM_F16 */
+    int32_t T, H, W;          /* output frames, rows, columns */
+    int32_t Cin, Cout;        /* Cin a multiple of 32 */
+    int32_t Cout_pad;         /* rows per tap in `wt`: a multiple of 32, >= Cout (rows past Cout are never stored) */
+    int32_t kt, kh, kw;       /* kt in 1..3; kh = kw in {1, 3} */
+    int32_t up2x;             /* 1: the input is at half resolution and is upsampled x2 (nearest) on the fly */
+    int32_t reserved;
+    int64_t x_stride[3];      /* frame, row, column strides of the padded input, in elements (channels contiguous) */
+    int64_t y_stride[3];      /* same for the output */
+} sfm_conv_desc;
+
+/* Channels-last convolution of the streaming VAE decoder: the nn.Conv3d / nn.Conv2d calls of wan/modules/vae.py
+ * (CausalConv3d :17-36; the 3x3 conv after the nearest x2 upsampling :76-79; residual, head and shortcut
+ * convolutions :186-220, :423-472).  `x` is the input with its kt - 1 history (or zero) frames in front and,
+ * for a 3x3 spatial kernel, a one-pixel zero border, i.e. [T + kt - 1][H + kh - 1][W + kw - 1][Cin] (with up2x:
+ * [T + kt - 1][H/2 + 2][W/2 + 2][Cin]); `wt` is the weight as [kt][kh][kw][Cout_pad][Cin]; `bias` (fp32, [Cout])
+ * may be NULL; `y` is [T][H][W][Cout].  One call's input must stay below 4 GiB. */
+int sfm_conv3d_cl(const sfm_conv_desc* desc, const void* x, const void* wt, const float* bias, void* y, void* stream);
+
 /* Measurement aid with no counterpart in the reference: runs a stream of independent 32x32x16 bf16 MFMAs (two waves
  * per SIMD, `iters` x 16 per wave) on `stream`, waits for it and returns the sustained rate in TFLOP/s.  bench.py
  * reports the dense kernel against it beside the nominal peak. */

@@ -8,7 +8,8 @@ reference's module names:
     attention.attention / attention.full_attention_with_kv_cache
     prologue.qk_prologue / prologue.rope_table
     causal_model.CausalWanModel (+ self-attention, block, head), pipeline.CausalInferencePipeline
+    vae_decode.WanVAEDecoder (streaming latent -> pixel decode; torch convolutions only)
 """
-from . import lib, monarch_attn, attention, prologue, causal_model, pipeline  # noqa: F401
+from . import lib, monarch_attn, attention, prologue, causal_model, pipeline, vae_decode  # noqa: F401
 
-__all__ = ["lib", "monarch_attn", "attention", "prologue", "causal_model", "pipeline"]
+__all__ = ["lib", "monarch_attn", "attention", "prologue", "causal_model", "pipeline", "vae_decode"]

@@ -1,0 +1,68 @@
+"""Channels-last convolutions of the streaming VAE decoder on the HIP library (`sfm_conv3d_cl`).
+
+Activations are [T, H, W, C] tensors (one video; channels contiguous).  Weights are re-laid out once per module
+as [kt, kh, kw, Cout_pad, Cin] and cached on it.  The reference's modules are nn.Conv3d / nn.Conv2d on
+[B, C, T, H, W] (wan/modules/vae.py:17-36, :76-79)."""
+import ctypes as C
+
+import torch
+
+from . import lib as L
+
+_DT = {torch.bfloat16: L.SFM_BF16, torch.float16: L.SFM_F16}
+
+
+def prepared(conv, dtype, device):
+    """(wt [kt,kh,kw,Cout_pad,Cin_pad], bias fp32 or None, kt, k) of an nn.Conv3d / nn.Conv2d, cached on the module.
+    Cin is padded with zero weights to a multiple of 32, Cout with zero rows to a multiple of 32."""
+    key = (dtype, str(device), conv.weight._version, conv.weight.data_ptr())
+    hit = getattr(conv, "_sfm_cl", None)
+    if hit is not None and hit[0] == key:
+        return hit[1]
+    w = conv.weight.detach()
+    if w.dim() == 4:                                   # Conv2d: one frame
+        w = w.unsqueeze(2)
+    cout, cin, kt, kh, kw = w.shape
+    cin_p, cout_p = (cin + 31) // 32 * 32, (cout + 31) // 32 * 32
+    wt = torch.zeros(kt, kh, kw, cout_p, cin_p, dtype=dtype, device=device)
+    wt[:, :, :, :cout, :cin] = w.permute(2, 3, 4, 0, 1).to(device=device, dtype=dtype)
+    bias = conv.bias.detach().to(device=device, dtype=torch.float32).contiguous() if conv.bias is not None else None
+    out = (wt.contiguous(), bias, kt, kh, cout, cin, cin_p, cout_p)
+    conv._sfm_cl = (key, out)
+    return out
+
+
+def conv_cl(x, conv, history=None, up2x=False):
+    """x [T, H, W, Cin] -> [T, H', W', Cout] for a causal Conv3d (kt - 1 frames of `history`, zeros where it is
+    shorter) or a Conv2d applied per frame; with up2x the nearest x2 upsampling in front of a 3x3 Conv2d is folded
+    into the convolution (H' = 2 H, W' = 2 W)."""
+    if x.dtype not in _DT:
+        raise TypeError(f"conv_cl: dtype {x.dtype} (bf16 or fp16 only)")
+    wt, bias, kt, k, cout, cin, cin_p, cout_p = prepared(conv, x.dtype, x.device)
+    T, H, W, _ = x.shape
+    past = kt - 1
+    pad = (k - 1) // 2
+    if past == 0 and pad == 0 and cin_p == cin and x.is_contiguous():
+        xp = x
+    else:
+        xp = torch.zeros(T + past, H + 2 * pad, W + 2 * pad, cin_p, dtype=x.dtype, device=x.device)
+        if history is not None and past > 0:
+            n = min(history.shape[0], past)
+            xp[past - n:past, pad:pad + H, pad:pad + W, :cin] = history[-n:]
+        xp[past:, pad:pad + H, pad:pad + W, :cin] = x
+    Ho, Wo = (2 * H, 2 * W) if up2x else (H, W)
+    y = torch.empty(T, Ho, Wo, cout, dtype=x.dtype, device=x.device)
+    d = L.ConvDesc()
+    d.dtype = _DT[x.dtype]
+    d.T, d.H, d.W = T, Ho, Wo
+    d.Cin, d.Cout, d.Cout_pad = cin_p, cout, cout_p
+    d.kt, d.kh, d.kw = kt, k, k
+    d.up2x = 1 if up2x else 0
+    for i in range(3):
+        d.x_stride[i] = xp.stride(i)
+        d.y_stride[i] = y.stride(i)
+    lib = L.load()
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    L.check(lib.sfm_conv3d_cl(C.byref(d), xp.data_ptr(), wt.data_ptr(), bias.data_ptr() if bias is not None else None,
+                              y.data_ptr(), stream))
+    return y

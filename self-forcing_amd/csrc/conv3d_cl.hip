@@ -1,0 +1,280 @@
+// Channels-last 3-D convolution as an implicit GEMM on gfx950 MFMA (bf16 / fp16), for the streaming VAE decoder
+// (replaces the nn.Conv3d / nn.Conv2d calls of wan/modules/vae.py:17-36, :76-97, :186-220, :423-472).
+//
+//   y[t, h, w, co] = bias[co] + sum_{dt, dh, dw, ci}  wt[dt, dh, dw, co, ci] * xp[t + dt, h' + dh, w' + dw, ci]
+//
+// xp is the input with its zero (or history) frames and its zero border already in place, so the kernel has no
+// bounds tests; with `up2x` it is the half-resolution tensor and (h', w') = the row / column of xp that the
+// nearest-neighbour x2 upsampling would have copied (vae.py:57-63, :77-79), i.e. the upsampled tensor is
+// never materialised.
+//
+// GEMM view: M = output channels (A operand, rows of wt with ci contiguous), N = output voxels (B operand, rows of
+// xp), K = taps x input channels, walked one tap and 32 channels at a time.  Each K step stages 64-byte rows
+// (32 channels) of both operands straight into LDS (global_load_lds_dwordx4), four rows to a 256-byte line with
+// the rows of a line rotated by the line index so that operand reads are conflict-free; two stage buffers, one
+// barrier per stage.  A wave owns CB x 32 output channels by 64 voxels; accumulators leave through the same
+// half-swap as the attention kernels (8 consecutive channels = 16 bytes per lane and voxel).
+
+#include <hip/hip_runtime.h>
+
+#include "sfm_attn.h"
+#include "sfm_common.hpp"
+
+namespace sfm {
+namespace {
+
+constexpr int kKC = 32;                      // input channels per stage
+constexpr int kRowBytes = kKC * 2;           // one staged row
+
+struct ConvArgs {
+    const char* x;            // padded input, channels-last
+    const char* wt;           // [taps][Cout_pad][Cin] (ci contiguous)
+    const float* bias;        // [Cout] or null
+    char* y;
+    int T, H, W;              // output grid
+    int Cin, Cout, Cout_pad;
+    int kt, kh, kw;
+    int up2x;
+    int64_t xs_t, xs_h, xs_w; // input strides in elements (channel stride 1)
+    int64_t ys_t, ys_h, ys_w; // output strides in elements
+    int64_t voxels;           // T * H * W
+};
+
+// byte offset of chunk c (16 bytes) of row r in a tile of 64-byte rows
+__device__ __forceinline__ uint32_t tile_off(int r, int c) {
+    const int line = r >> 2;
+    return (uint32_t)(line * 256 + (((r & 3) ^ (line & 3)) << 6) + (c << 4));
+}
+
+__device__ __forceinline__ void cv_load_lds16(const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void cv_wait_stage() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// CB: 32-channel blocks per wave; WN: waves along the output channels (the other 4 / WN waves split the voxels).
+template <class E, int CB, int WN>
+__global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
+    constexpr int WM = 4 / WN;
+    constexpr int kVox = 64 * WM;                         // voxels per workgroup
+    constexpr int kCo = 32 * CB * WN;                     // output channels per workgroup
+    constexpr int kCoRows = (kCo + 63) / 64 * 64;         // weight rows staged (whole groups of 16 per wave)
+    constexpr int kRows = kCoRows + kVox;
+    constexpr int kStage = kRows * kRowBytes;
+    constexpr int kGroups = kRows / 16;                   // 16-row groups, one load instruction each
+    constexpr int kPerWave = kGroups / 4;
+    static_assert(kGroups % 4 == 0, "rows must split evenly over the waves");
+    extern __shared__ __attribute__((aligned(256))) char lds[];
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
+
+    const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave % WN, wm = wave / WN;
+    const int64_t v0 = (int64_t)blockIdx.x * kVox;
+    const int co0 = blockIdx.y * kCo;
+
+    // ---- what this lane stages: for each of the wave's row groups one 16-byte chunk of one row
+    // lane -> (line, quarter, chunk) of the group's 1 KB; the row sitting in that quarter is quarter ^ line
+    const int g_line = lane >> 4, g_q = (lane >> 2) & 3, g_c = lane & 3;
+    const int g_row = g_line * 4 + (g_q ^ g_line);
+    // weights: byte offset of the row (without tap and channel step); voxels: byte offset of the voxel's first tap
+    // (with up2x only its frame: rows and columns depend on the tap through the halving and are added per stage)
+    uint32_t src_off[kPerWave];
+    int vh[kPerWave], vw[kPerWave];
+#pragma unroll
+    for (int i = 0; i < kPerWave; ++i) {
+        const int row = (i * 4 + wave) * 16 + g_row;
+        vh[i] = vw[i] = 0;
+        if (row < kCoRows) {                              // wave-uniform: a group is all weights or all voxels
+            const int co = min(co0 + row, p.Cout_pad - 1);
+            src_off[i] = (uint32_t)(co * p.Cin * 2 + g_c * 16);
+        } else {
+            const int64_t v = min(v0 + (row - kCoRows), p.voxels - 1);   // rows past the end repeat the last voxel
+            const int w = (int)(v % p.W);
+            const int64_t r = v / p.W;
+            const int h = (int)(r % p.H), t = (int)(r / p.H);
+            vh[i] = h;
+            vw[i] = w;
+            const int64_t e = p.up2x ? t * p.xs_t : t * p.xs_t + h * p.xs_h + w * p.xs_w;
+            src_off[i] = (uint32_t)(e * 2 + g_c * 16);
+        }
+    }
+
+    const int cin_steps = p.Cin / kKC;
+    const int taps = p.kt * p.kh * p.kw;
+    const int nstage = taps * cin_steps;
+
+    auto stage = [&](int s, uint32_t buf) {
+        const int tap = s / cin_steps, cs = s - tap * cin_steps;
+        const int dw = tap % p.kw;
+        const int r = tap / p.kw;
+        const int dh = r % p.kh, dt = r / p.kh;
+        const char* wbase = p.wt + ((size_t)tap * p.Cout_pad * p.Cin + (size_t)cs * kKC) * 2;
+        const char* xbase = p.x + ((size_t)dt * p.xs_t + (size_t)cs * kKC) * 2;
+        if (!p.up2x) xbase += ((size_t)dh * p.xs_h + (size_t)dw * p.xs_w) * 2;
+#pragma unroll
+        for (int i = 0; i < kPerWave; ++i) {
+            const uint32_t dst = lds0 + buf + (uint32_t)(i * 4 + wave) * 1024;
+            if ((i * 4 + wave) * 16 < kCoRows) {
+                cv_load_lds16(wbase, src_off[i], dst);
+            } else if (!p.up2x) {
+                cv_load_lds16(xbase, src_off[i], dst);
+            } else {
+                const int hh = ((vh[i] + dh - 1) >> 1) + 1, ww = ((vw[i] + dw - 1) >> 1) + 1;
+                cv_load_lds16(xbase, src_off[i] + (uint32_t)((hh * p.xs_h + ww * p.xs_w) * 2), dst);
+            }
+        }
+    };
+
+    f32x16 acc[CB][2];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int vb = 0; vb < 2; ++vb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[cb][vb][v] = 0.f;
+
+    // operand read offsets within a stage: row r0 + m, chunk 2 ks + hf
+    uint32_t a_off[CB], b_off[2];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) a_off[cb] = tile_off(32 * (cb + CB * wn) + m, hf);
+#pragma unroll
+    for (int vb = 0; vb < 2; ++vb) b_off[vb] = tile_off(kCoRows + 64 * wm + 32 * vb + m, hf);
+
+    stage(0, 0);
+    for (int s = 0; s < nstage; ++s) {
+        const uint32_t buf = (uint32_t)(s & 1) * kStage;
+        cv_wait_stage();                                   // stage s is in LDS; the other buffer is free
+        if (s + 1 < nstage) stage(s + 1, buf ^ kStage);
+#pragma unroll
+        for (int ks = 0; ks < kKC / 16; ++ks) {
+            u32x4 a[CB], b[2];
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) a[cb] = *(const u32x4*)(lds + buf + a_off[cb] + ks * 32);
+#pragma unroll
+            for (int vb = 0; vb < 2; ++vb) b[vb] = *(const u32x4*)(lds + buf + b_off[vb] + ks * 32);
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int vb = 0; vb < 2; ++vb) acc[cb][vb] = E::mfma32(a[cb], b[vb], acc[cb][vb]);
+        }
+    }
+
+    // ---- epilogue: lane (m, hf) of block (cb, vb) holds voxel 32 vb + m, channels 8 g + 4 hf + (v & 3)
+#pragma unroll
+    for (int vb = 0; vb < 2; ++vb) {
+        const int64_t v = v0 + 64 * wm + 32 * vb + m;
+        const bool vok = v < p.voxels;
+        const int64_t vc = vok ? v : 0;
+        const int w = (int)(vc % p.W);
+        const int64_t r = vc / p.W;
+        const int h = (int)(r % p.H), t = (int)(r / p.H);
+        char* yrow = p.y + (t * p.ys_t + h * p.ys_h + w * p.ys_w) * 2;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            const int cbase = co0 + 32 * (cb + CB * wn);
+            if (p.bias != nullptr) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int co = cbase + 8 * (e >> 2) + 4 * hf + (e & 3);
+                    acc[cb][vb][e] += co < p.Cout ? p.bias[co] : 0.f;
+                }
+            }
+            if (cbase + 32 <= p.Cout) {
+#pragma unroll
+                for (int gp = 0; gp < 2; ++gp) {
+                    const int g0 = 2 * gp, g1 = 2 * gp + 1;
+                    auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[cb][vb][4 * g0 + 0], acc[cb][vb][4 * g0 + 1]),
+                                                               pack2<E>(acc[cb][vb][4 * g1 + 0], acc[cb][vb][4 * g1 + 1]), false, false);
+                    auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[cb][vb][4 * g0 + 2], acc[cb][vb][4 * g0 + 3]),
+                                                               pack2<E>(acc[cb][vb][4 * g1 + 2], acc[cb][vb][4 * g1 + 3]), false, false);
+                    u32x4 o = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+                    if (vok) *(u32x4*)(yrow + (cbase + 16 * gp + 8 * hf) * 2) = o;
+                }
+            } else {
+                // a partial last block (e.g. the 3 channels of the decoder's head): element stores
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int co = cbase + 8 * (e >> 2) + 4 * hf + (e & 3);
+                    if (vok && co < p.Cout) *(uint16_t*)(yrow + co * 2) = E::from_float(acc[cb][vb][e]);
+                }
+            }
+        }
+    }
+}
+
+template <class E, int CB, int WN>
+int launch_cfg(const ConvArgs& a, hipStream_t st) {
+    constexpr int kVox = 64 * (4 / WN), kCo = 32 * CB * WN, kCoRows = (kCo + 63) / 64 * 64;
+    constexpr int ldsb = 2 * (kCoRows + kVox) * kRowBytes;
+    dim3 grid((unsigned)((a.voxels + kVox - 1) / kVox), (unsigned)((a.Cout_pad + kCo - 1) / kCo));
+    hipLaunchKernelGGL((conv3d_cl_kernel<E, CB, WN>), grid, dim3(256), ldsb, st, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("sfm_conv3d_cl: launch failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+template <class E>
+int launch_dtype(const ConvArgs& a, hipStream_t st) {
+    if (a.Cout_pad % 192 == 0) return launch_cfg<E, 3, 2>(a, st);
+    if (a.Cout_pad % 96 == 0) return launch_cfg<E, 3, 1>(a, st);
+    return launch_cfg<E, 1, 1>(a, st);                    // Cout_pad a multiple of 32
+}
+
+}  // namespace
+}  // namespace sfm
+
+extern "C" int sfm_conv3d_cl(const sfm_conv_desc* d, const void* x, const void* wt, const float* bias, void* y, void* stream) {
+    using namespace sfm;
+    if (d == nullptr || x == nullptr || wt == nullptr || y == nullptr) {
+        set_error("sfm_conv3d_cl: null argument");
+        return SFM_ERR_NULL;
+    }
+    if (d->dtype != SFM_BF16 && d->dtype != SFM_F16) {
+        set_error("sfm_conv3d_cl: dtype %d (need SFM_BF16 or SFM_F16)", d->dtype);
+        return SFM_ERR_DTYPE;
+    }
+    if (d->T < 1 || d->H < 1 || d->W < 1 || d->Cin < 32 || d->Cin % 32 != 0 || d->Cout < 1 || d->Cout_pad < d->Cout ||
+        d->Cout_pad % 32 != 0 || d->kt < 1 || d->kt > 3 || (d->kh != 1 && d->kh != 3) || d->kh != d->kw) {
+        set_error("sfm_conv3d_cl: T,H,W >= 1, Cin a multiple of 32, Cout_pad >= Cout a multiple of 32, kt in 1..3, kh = kw in {1, 3}");
+        return SFM_ERR_SHAPE;
+    }
+    if (d->up2x && (d->kh != 3 || d->H % 2 != 0 || d->W % 2 != 0)) {
+        set_error("sfm_conv3d_cl: up2x needs a 3x3 spatial kernel and even H, W");
+        return SFM_ERR_SHAPE;
+    }
+    for (int i = 0; i < 3; ++i) {
+        // whole 32-channel blocks leave as 16-byte stores, a partial last block element by element
+        if (d->x_stride[i] < d->Cin || d->x_stride[i] % 8 != 0 || d->y_stride[i] < d->Cout || (d->Cout >= 32 && d->y_stride[i] % 8 != 0)) {
+            set_error("sfm_conv3d_cl: strides must be at least the channel count and (input always, output when Cout >= 32) multiples of 8 elements");
+            return SFM_ERR_STRIDE;
+        }
+    }
+    // extents of the padded input the kernel will touch, in elements, must fit the 32-bit lane offsets
+    const int64_t hin = (d->up2x ? d->H / 2 : d->H) + (d->kh - 1), win = (d->up2x ? d->W / 2 : d->W) + (d->kw - 1);
+    const int64_t span = ((int64_t)(d->T + d->kt - 2) * d->x_stride[0] + (hin - 1) * d->x_stride[1] + (win - 1) * d->x_stride[2] + d->Cin) * 2;
+    if (span >= ((int64_t)1 << 32) || (int64_t)d->Cout_pad * d->Cin * 2 >= ((int64_t)1 << 32)) {
+        set_error("sfm_conv3d_cl: the input of one call must stay below 4 GiB (%lld bytes)", (long long)span);
+        return SFM_ERR_RANGE;
+    }
+    if ((((uintptr_t)x | (uintptr_t)wt) & 15) || ((uintptr_t)y & (d->Cout >= 32 ? 15 : 1))) {
+        set_error("sfm_conv3d_cl: x, wt, y must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    ConvArgs a;
+    a.x = (const char*)x;
+    a.wt = (const char*)wt;
+    a.bias = bias;
+    a.y = (char*)y;
+    a.T = d->T; a.H = d->H; a.W = d->W;
+    a.Cin = d->Cin; a.Cout = d->Cout; a.Cout_pad = d->Cout_pad;
+    a.kt = d->kt; a.kh = d->kh; a.kw = d->kw;
+    a.up2x = d->up2x;
+    a.xs_t = d->x_stride[0]; a.xs_h = d->x_stride[1]; a.xs_w = d->x_stride[2];
+    a.ys_t = d->y_stride[0]; a.ys_h = d->y_stride[1]; a.ys_w = d->y_stride[2];
+    a.voxels = (int64_t)d->T * d->H * d->W;
+    hipStream_t st = (hipStream_t)stream;
+    return d->dtype == SFM_BF16 ? launch_dtype<BF16>(a, st) : launch_dtype<F16>(a, st);
+}

@@ -20,8 +20,14 @@ ERR_NAMES = {
 SYMBOLS = [
     "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
-    "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm", "sfm_probe_mfma_bf16", "sfm_last_error", "sfm_version",
+    "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm", "sfm_probe_mfma_bf16", "sfm_conv3d_cl", "sfm_last_error", "sfm_version",
 ]
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [("dtype", C.c_int32), ("T", C.c_int32), ("H", C.c_int32), ("W", C.c_int32), ("Cin", C.c_int32),
+                ("Cout", C.c_int32), ("Cout_pad", C.c_int32), ("kt", C.c_int32), ("kh", C.c_int32), ("kw", C.c_int32),
+                ("up2x", C.c_int32), ("reserved", C.c_int32), ("x_stride", C.c_int64 * 3), ("y_stride", C.c_int64 * 3)]
 
 
 class Tiling(C.Structure):
@@ -95,6 +101,7 @@ def load():
     lib.sfm_gate_residual_ln.argtypes = [C.c_int32, I64, C.c_int32, C.c_float, P, I64, P, I64, P, I64, C.c_int32, P, I64, P, P, I64,
                                          C.c_int32, P, P, P]
     lib.sfm_rms_norm.argtypes = [C.c_int32, I64, C.c_int32, C.c_float, P, I64, P, I64, P, P]
+    lib.sfm_conv3d_cl.argtypes = [C.POINTER(ConvDesc), P, P, P, P, P]
     lib.sfm_probe_mfma_bf16.argtypes = [C.c_int32, P, C.POINTER(C.c_float)]
     for name in SYMBOLS:
         if name not in ("sfm_version", "sfm_last_error"):

@@ -137,8 +137,14 @@ class CausalInferencePipeline(nn.Module):
         return s
 
     @torch.no_grad()
-    def inference(self, noise, prompt_embeds, profile=False):
-        """noise [B, F, C, H, W]; prompt_embeds [B, L_text, text_dim].  Returns latents [B, F, C, H, W]."""
+    def inference(self, noise, prompt_embeds, profile=False, vae=None, on_pixels=None):
+        """noise [B, F, C, H, W]; prompt_embeds [B, L_text, text_dim].  Returns latents [B, F, C, H, W].
+
+        With `vae` (a vae_decode.WanVAEDecoder) every chunk is decoded as soon as it is clean, continuing one
+        decode stream (the demo's chunk-by-chunk decode, demo.py:406-441); the pixel chunks [B, T', 3, 8H, 8W]
+        go to `on_pixels(chunk_index, pixels)` if given, else they are concatenated and returned as a second
+        value.  The reference's offline pipeline decodes the finished video in one go instead
+        (pipeline/causal_inference.py:265): call `vae.decode_to_pixel(latents)` on the result for that."""
         B, num_frames, C, H, W = noise.shape
         assert num_frames % self.num_frame_per_block == 0
         num_blocks = num_frames // self.num_frame_per_block
@@ -151,7 +157,9 @@ class CausalInferencePipeline(nn.Module):
             self._reset_caches(noise.device)
         self.last_chunk_ms = []
         start_frame = 0
-        for _ in range(num_blocks):
+        decode_state = vae.new_state() if vae is not None else None
+        pixels = []
+        for block in range(num_blocks):
             nf = self.num_frame_per_block
             if profile:
                 torch.cuda.synchronize(noise.device)
@@ -171,12 +179,20 @@ class CausalInferencePipeline(nn.Module):
                         flat, eps, next_t * torch.ones([B * nf], device=noise.device, dtype=torch.long)
                     ).unflatten(0, denoised.shape[:2])
             output[:, start_frame:start_frame + nf] = denoised
+            if vae is not None:
+                px = vae.decode_to_pixel(denoised, use_cache=True, state=decode_state)
+                if on_pixels is not None:
+                    on_pixels(block, px)
+                else:
+                    pixels.append(px)
             ctx_t = torch.ones([B, nf], device=noise.device, dtype=torch.int64) * self.context_noise
             self.generator(denoised, cond, ctx_t, self.kv_cache1, self.crossattn_cache, cur)
             if profile:
                 torch.cuda.synchronize(noise.device)
                 self.last_chunk_ms.append((time.perf_counter() - t0) * 1e3)
             start_frame += nf
+        if vae is not None and on_pixels is None:
+            return output, torch.cat(pixels, dim=1)
         return output
 
 

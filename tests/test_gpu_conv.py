@@ -1,0 +1,69 @@
+"""GPU parity of the channels-last convolution kernel (`sfm_conv3d_cl` through conv_ops.conv_cl) against torch's
+fp32 convolution of the same 16-bit operands: the shapes of the streaming VAE decoder (causal 3x3x3 with and
+without history, the (3,1,1) temporal convolution, the 3x3 convolution behind the nearest x2 upsampling, the
+16-channel input and the 3-channel head), ragged tile edges, both 16-bit types."""
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from self_forcing_amd import conv_ops as co
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # cin, cout, kt, k, T, H, W, up2x, history frames, dtype
+    (96, 96, 3, 3, 2, 5, 7, False, 2, torch.bfloat16),
+    (192, 192, 3, 3, 3, 6, 10, False, 1, torch.bfloat16),
+    (192, 384, 3, 3, 1, 4, 9, False, 0, torch.bfloat16),
+    (384, 768, 3, 1, 2, 5, 6, False, 2, torch.bfloat16),
+    (16, 384, 3, 3, 1, 6, 8, False, 0, torch.bfloat16),
+    (96, 3, 3, 3, 4, 9, 13, False, 2, torch.bfloat16),
+    (384, 192, 1, 3, 2, 5, 6, True, 0, torch.bfloat16),
+    (192, 96, 1, 3, 3, 4, 7, True, 0, torch.bfloat16),
+    (96, 96, 3, 3, 3, 33, 41, False, 2, torch.float16),
+    (64, 64, 3, 3, 1, 1, 1, False, 0, torch.float16),
+    (96, 96, 3, 3, 2, 16, 16, False, 2, torch.bfloat16),          # 512 voxels: exactly two workgroup tiles
+]
+
+
+@pytest.mark.parametrize("cin,cout,kt,k,T,H,W,up2x,hist,dt", CASES)
+def test_conv_cl_matches_fp32_convolution(cin, cout, kt, k, T, H, W, up2x, hist, dt):
+    torch.manual_seed(cin * 7 + cout + T)
+    conv = (nn.Conv2d(cin, cout, 3, padding=1) if kt == 1 else nn.Conv3d(cin, cout, (kt, k, k))).cuda().to(dt)
+    x = torch.randn(T, H, W, cin, device="cuda").to(dt)
+    h = torch.randn(hist, H, W, cin, device="cuda").to(dt) if hist else None
+    y = co.conv_cl(x, conv, h, up2x)
+    wf, bf = conv.weight.float(), conv.bias.float()
+    if kt == 1:
+        z = x.float().permute(0, 3, 1, 2)
+        if up2x:
+            z = F.interpolate(z, scale_factor=2.0, mode="nearest")
+        ref = F.conv2d(z, wf, bf, padding=1).permute(0, 2, 3, 1)
+    else:
+        xf = x.float().permute(3, 0, 1, 2).unsqueeze(0)
+        if h is not None:
+            xf = torch.cat([h.float().permute(3, 0, 1, 2).unsqueeze(0), xf], 2)
+        xf = F.pad(xf, (k // 2, k // 2, k // 2, k // 2, (kt - 1) - (xf.shape[2] - T), 0))
+        ref = F.conv3d(xf, wf, bf)[0].permute(1, 2, 3, 0)
+    assert y.shape == ref.shape
+    # fp32 accumulation of 16-bit products, one rounding of the result
+    tol = (2.0 ** -8 if dt == torch.bfloat16 else 2.0 ** -11) * max(1.0, ref.abs().max().item()) * 1.01
+    assert (y.float() - ref).abs().max().item() <= tol
+
+
+def test_conv_cl_rejects_bad_arguments():
+    import ctypes as C
+    from self_forcing_amd import lib as L
+    lib = L.load()
+    d = L.ConvDesc()
+    d.dtype, d.T, d.H, d.W, d.Cin, d.Cout, d.Cout_pad, d.kt, d.kh, d.kw = L.SFM_BF16, 1, 4, 4, 48, 32, 32, 3, 3, 3
+    buf = torch.zeros(1 << 16, dtype=torch.bfloat16, device="cuda")
+    for i in range(3):
+        d.x_stride[i] = d.y_stride[i] = 64
+    assert lib.sfm_conv3d_cl(C.byref(d), buf.data_ptr(), buf.data_ptr(), None, buf.data_ptr(), None) == -3      # Cin % 32
+    d.Cin = 64
+    d.x_stride[2] = 60
+    assert lib.sfm_conv3d_cl(C.byref(d), buf.data_ptr(), buf.data_ptr(), None, buf.data_ptr(), None) == -5      # stride
+    d.x_stride[2] = 64
+    assert lib.sfm_conv3d_cl(C.byref(d), None, buf.data_ptr(), None, buf.data_ptr(), None) == -1
