@@ -212,6 +212,13 @@ typedef struct sfm_conv_desc {
  * may be NULL; `y` is [T][H][W][Cout].  One call's input must stay below 4 GiB. */
 int sfm_conv3d_cl(const sfm_conv_desc* desc, const void* x, const void* wt, const float* bias, void* y, void* stream);
 
+/* RMS norm over the channels with optional SiLU for channels-last activations [T][H][W][C]: y = x / max(|x|_2, 1e-12)
+ * * sqrt(C) * gamma, then y * sigmoid(y) if act != 0 (wan/modules/vae.py:39-54 and the nn.SiLU that follows it in
+ * :192-197, :418-420).  fp32 inside, one rounding.  Strides in elements (frame, row, column); x and y may be views
+ * into larger buffers (e.g. the interior of the next convolution's padded input).  gamma has the dtype of x. */
+int sfm_vae_norm_act(int32_t dtype, int32_t T, int32_t H, int32_t W, int32_t C, int32_t act, const void* x,
+                     const int64_t x_stride[3], const void* gamma, void* y, const int64_t y_stride[3], void* stream);
+
 /* Measurement aid with no counterpart in the reference: runs a stream of independent 32x32x16 bf16 MFMAs (two waves
  * per SIMD, `iters` x 16 per wave) on `stream`, waits for it and returns the sustained rate in TFLOP/s.  bench.py
  * reports the dense kernel against it beside the nominal peak. */

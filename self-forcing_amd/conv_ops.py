@@ -32,24 +32,47 @@ def prepared(conv, dtype, device):
     return out
 
 
-def conv_cl(x, conv, history=None, up2x=False):
+def norm_act(x, gamma, act, out=None):
+    """RMS norm over the channels of x [T, H, W, C] (+ SiLU if act) on the HIP library; `out` may be a strided view
+    (e.g. the interior of a padded convolution input)."""
+    T, H, W, Cn = x.shape
+    if out is None:
+        out = torch.empty_like(x)
+    g = gamma.detach().reshape(-1).to(device=x.device, dtype=x.dtype).contiguous()
+    if x.stride(3) != 1 or out.stride(3) != 1:
+        raise ValueError("norm_act: channels must be contiguous")
+    S3 = C.c_int64 * 3
+    lib = L.load()
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    L.check(lib.sfm_vae_norm_act(_DT[x.dtype], T, H, W, Cn, 1 if act else 0, x.data_ptr(), S3(*x.stride()[:3]), g.data_ptr(),
+                                 out.data_ptr(), S3(*out.stride()[:3]), stream))
+    return out
+
+
+def conv_cl(x, conv, history=None, up2x=False, norm=None, want_tail=False):
     """x [T, H, W, Cin] -> [T, H', W', Cout] for a causal Conv3d (kt - 1 frames of `history`, zeros where it is
     shorter) or a Conv2d applied per frame; with up2x the nearest x2 upsampling in front of a 3x3 Conv2d is folded
-    into the convolution (H' = 2 H, W' = 2 W)."""
+    into the convolution (H' = 2 H, W' = 2 W).  With norm = (gamma, act) the convolution's input is
+    norm_act(x, gamma, act), written straight into the padded buffer.  With want_tail the last two frames of the
+    (history + input) sequence come back as well: what the next call of a stream passes as `history`."""
     if x.dtype not in _DT:
         raise TypeError(f"conv_cl: dtype {x.dtype} (bf16 or fp16 only)")
     wt, bias, kt, k, cout, cin, cin_p, cout_p = prepared(conv, x.dtype, x.device)
     T, H, W, _ = x.shape
     past = kt - 1
     pad = (k - 1) // 2
-    if past == 0 and pad == 0 and cin_p == cin and x.is_contiguous():
+    if past == 0 and pad == 0 and cin_p == cin and x.is_contiguous() and norm is None:
         xp = x
     else:
         xp = torch.zeros(T + past, H + 2 * pad, W + 2 * pad, cin_p, dtype=x.dtype, device=x.device)
         if history is not None and past > 0:
             n = min(history.shape[0], past)
             xp[past - n:past, pad:pad + H, pad:pad + W, :cin] = history[-n:]
-        xp[past:, pad:pad + H, pad:pad + W, :cin] = x
+        inner = xp[past:, pad:pad + H, pad:pad + W, :cin]
+        if norm is None:
+            inner.copy_(x)
+        else:
+            norm_act(x, norm[0], norm[1], out=inner)
     Ho, Wo = (2 * H, 2 * W) if up2x else (H, W)
     y = torch.empty(T, Ho, Wo, cout, dtype=x.dtype, device=x.device)
     d = L.ConvDesc()
@@ -65,4 +88,7 @@ def conv_cl(x, conv, history=None, up2x=False):
     stream = torch.cuda.current_stream(x.device).cuda_stream
     L.check(lib.sfm_conv3d_cl(C.byref(d), xp.data_ptr(), wt.data_ptr(), bias.data_ptr() if bias is not None else None,
                               y.data_ptr(), stream))
+    if want_tail:
+        n = min(2, T + past)
+        return y, xp[T + past - n:, pad:pad + H, pad:pad + W, :cin].clone()
     return y

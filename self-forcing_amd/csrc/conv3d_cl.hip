@@ -223,6 +223,78 @@ int launch_dtype(const ConvArgs& a, hipStream_t st) {
     return launch_cfg<E, 1, 1>(a, st);                    // Cout_pad a multiple of 32
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// RMS norm over the channels, optional SiLU (vae.py:39-54 + nn.SiLU of :192-197, :418-420), channels-last, fp32
+// inside, one rounding at the end.  GL lanes share a voxel (8 channels each, the first C / 8 of them active).
+// ------------------------------------------------------------------------------------------------
+struct NormArgs {
+    const char* x;
+    char* y;
+    const uint16_t* gamma;
+    int T, H, W, C, act;
+    int64_t xs_t, xs_h, xs_w, ys_t, ys_h, ys_w;
+    int64_t voxels;
+};
+
+template <class E, int GL>
+__global__ __launch_bounds__(256) void vae_norm_act_kernel(NormArgs p) {
+    const int tid = threadIdx.x;
+    const int sub = tid % GL;
+    const int64_t v = (int64_t)blockIdx.x * (256 / GL) + tid / GL;
+    const bool active = v < p.voxels && sub < p.C / 8;
+    const int64_t vc = v < p.voxels ? v : p.voxels - 1;
+    const int w = (int)(vc % p.W);
+    const int64_t r = vc / p.W;
+    const int h = (int)(r % p.H), t = (int)(r / p.H);
+    u32x4 raw = {0u, 0u, 0u, 0u};
+    if (active) raw = *(const u32x4*)(p.x + (t * p.xs_t + h * p.xs_h + w * p.xs_w + sub * 8) * 2);
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = E::to_float((uint16_t)(raw[i] & 0xffffu));
+        f[2 * i + 1] = E::to_float((uint16_t)(raw[i] >> 16));
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss += f[i] * f[i];
+#pragma unroll
+    for (int o = GL / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, GL);
+    // x / max(|x|, 1e-12) * sqrt(C)  (F.normalize's clamp, vae.py:51-54)
+    const float inv = sqrtf((float)p.C) / fmaxf(sqrtf(ss), 1e-12f);
+    if (active) {
+        const u32x4 g = *(const u32x4*)(p.gamma + sub * 8);
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float a = f[2 * i] * inv * E::to_float((uint16_t)(g[i] & 0xffffu));
+            float b = f[2 * i + 1] * inv * E::to_float((uint16_t)(g[i] >> 16));
+            if (p.act) {
+                a = a / (1.f + __expf(-a));
+                b = b / (1.f + __expf(-b));
+            }
+            o[i] = pack2<E>(a, b);
+        }
+        *(u32x4*)(p.y + (t * p.ys_t + h * p.ys_h + w * p.ys_w + sub * 8) * 2) = o;
+    }
+}
+
+template <class E>
+int launch_norm(const NormArgs& a, hipStream_t st) {
+    const int lanes = a.C / 8;
+    const int gl = lanes <= 16 ? 16 : lanes <= 32 ? 32 : 64;
+    const unsigned blocks = (unsigned)((a.voxels + 256 / gl - 1) / (256 / gl));
+    if (gl == 16) hipLaunchKernelGGL((vae_norm_act_kernel<E, 16>), dim3(blocks), dim3(256), 0, st, a);
+    else if (gl == 32) hipLaunchKernelGGL((vae_norm_act_kernel<E, 32>), dim3(blocks), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((vae_norm_act_kernel<E, 64>), dim3(blocks), dim3(256), 0, st, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("sfm_vae_norm_act: launch failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
 }  // namespace
 }  // namespace sfm
 
@@ -277,4 +349,41 @@ extern "C" int sfm_conv3d_cl(const sfm_conv_desc* d, const void* x, const void* 
     a.voxels = (int64_t)d->T * d->H * d->W;
     hipStream_t st = (hipStream_t)stream;
     return d->dtype == SFM_BF16 ? launch_dtype<BF16>(a, st) : launch_dtype<F16>(a, st);
+}
+
+extern "C" int sfm_vae_norm_act(int32_t dtype, int32_t T, int32_t H, int32_t W, int32_t C, int32_t act, const void* x,
+                                const int64_t x_stride[3], const void* gamma, void* y, const int64_t y_stride[3], void* stream) {
+    using namespace sfm;
+    if (x == nullptr || y == nullptr || gamma == nullptr || x_stride == nullptr || y_stride == nullptr) {
+        set_error("sfm_vae_norm_act: null argument");
+        return SFM_ERR_NULL;
+    }
+    if (dtype != SFM_BF16 && dtype != SFM_F16) {
+        set_error("sfm_vae_norm_act: dtype %d (need SFM_BF16 or SFM_F16)", dtype);
+        return SFM_ERR_DTYPE;
+    }
+    if (T < 1 || H < 1 || W < 1 || C < 8 || C > 512 || C % 8 != 0) {
+        set_error("sfm_vae_norm_act: T,H,W >= 1 and C a multiple of 8 up to 512");
+        return SFM_ERR_SHAPE;
+    }
+    for (int i = 0; i < 3; ++i) {
+        if (x_stride[i] < C || x_stride[i] % 8 != 0 || y_stride[i] < C || y_stride[i] % 8 != 0) {
+            set_error("sfm_vae_norm_act: strides must be multiples of 8 elements and at least C");
+            return SFM_ERR_STRIDE;
+        }
+    }
+    if (((uintptr_t)x | (uintptr_t)y | (uintptr_t)gamma) & 15) {
+        set_error("sfm_vae_norm_act: x, y, gamma must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    NormArgs a;
+    a.x = (const char*)x;
+    a.y = (char*)y;
+    a.gamma = (const uint16_t*)gamma;
+    a.T = T; a.H = H; a.W = W; a.C = C; a.act = act;
+    a.xs_t = x_stride[0]; a.xs_h = x_stride[1]; a.xs_w = x_stride[2];
+    a.ys_t = y_stride[0]; a.ys_h = y_stride[1]; a.ys_w = y_stride[2];
+    a.voxels = (int64_t)T * H * W;
+    hipStream_t st = (hipStream_t)stream;
+    return dtype == SFM_BF16 ? launch_norm<BF16>(a, st) : launch_norm<F16>(a, st);
 }

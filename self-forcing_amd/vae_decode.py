@@ -10,9 +10,16 @@ Every temporal convolution is causal and keeps the last two input frames of the 
 decoder serves any number of independent streams.  The reference feeds the decoder one latent frame per
 call; the convolutions are causal, so a call may carry any number of frames and give the same result, and
 this decoder pushes a whole chunk through at once (only the very first frame of a stream goes alone: the
-temporal upsamplers skip it, vae.py:104-107).  The convolutions run in torch (MIOpen); nothing here needs
-the attention library.
+temporal upsamplers skip it, vae.py:104-107).
+
+Two execution paths share the parameters and the stream logic.  On the GPU in bf16 / fp16 a stream of one video
+runs channels-last ([T, H, W, C] activations): 3x3x3, (3,1,1) and upsampling convolutions go to the HIP
+implicit-GEMM kernel (`conv_ops.conv_cl`, which folds the nearest x2 upsampling into the convolution), 1x1
+convolutions are matrix products.  Anywhere else (CPU, fp32, batches, `SFM_VAE_TORCH_CONV=1`) the modules run as
+torch convolutions on [B, C, T, H, W].  A DecodeState stays with the path that started it.
 """
+import os
+
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
@@ -35,6 +42,7 @@ class DecodeState:
         self.tails = [None] * n_convs
         self.cursor = 0
         self.frames_in = 0
+        self.layout = None                  # "cl" (channels-last, HIP convolutions) or "ncthw" (torch), set by the first call
 
     def rewind(self):
         self.cursor = 0
@@ -78,6 +86,21 @@ class CausalConv3d(nn.Conv3d):
         state.tails[i] = tail
         return y
 
+    def stream_cl(self, x, state, norm=None):
+        """`stream` for channels-last activations [T, H, W, C]; with norm = (gamma, act) the convolution's input is
+        the RMS norm (+ SiLU) of x.  The tail kept is always two frames (a zero frame stands in before the stream
+        has two), which the convolution treats exactly like the reference's shorter cache plus zero padding."""
+        from . import conv_ops
+        i = state.take()
+        prev = state.tails[i]
+        y, tail = conv_ops.conv_cl(x, self, prev if isinstance(prev, torch.Tensor) else None, norm=norm, want_tail=True)
+        state.tails[i] = tail
+        return y
+
+    def pointwise_cl(self, x):
+        """A 1x1x1 convolution of channels-last activations: a matrix product over the channels."""
+        return F.linear(x, self.weight.view(self.out_channels, self.in_channels), self.bias)
+
 
 class RMS_norm(nn.Module):
     """x / |x|_2 over channels * sqrt(C) * gamma (vae.py:39-54)."""
@@ -89,6 +112,10 @@ class RMS_norm(nn.Module):
 
     def forward(self, x):
         return F.normalize(x, dim=1) * self.scale * self.gamma
+
+    def forward_cl(self, x, act=False):
+        from . import conv_ops
+        return conv_ops.norm_act(x.contiguous(), self.gamma, act)
 
 
 class _Nearest2x(nn.Module):
@@ -134,6 +161,26 @@ class Resample(nn.Module):
         return x.reshape(b, t, x.shape[1], 2 * h, 2 * w).permute(0, 2, 1, 3, 4)
 
 
+    def forward_cl(self, x, state):
+        """`forward` for channels-last activations [T, H, W, C]."""
+        from . import conv_ops
+        t, h, w, c = x.shape
+        if self.mode == "upsample3d":
+            i = state.take()
+            prev = state.tails[i]
+            if prev is None:
+                state.tails[i] = DecodeState.FIRST
+            else:
+                tail = x[-TAIL:].clone()
+                if tail.shape[0] < TAIL:
+                    head = prev[-1:] if isinstance(prev, torch.Tensor) else torch.zeros_like(tail)
+                    tail = torch.cat([head, tail], dim=0)
+                y = conv_ops.conv_cl(x, self.time_conv, prev if isinstance(prev, torch.Tensor) else None)
+                state.tails[i] = tail
+                x = torch.stack((y[..., :c], y[..., c:]), dim=1).reshape(2 * t, h, w, c)
+        return conv_ops.conv_cl(x, self.resample[1], None, up2x=True)
+
+
 class ResidualBlock(nn.Module):
     """norm, SiLU, conv, norm, SiLU, conv + shortcut (vae.py:186-220)."""
 
@@ -148,6 +195,13 @@ class ResidualBlock(nn.Module):
         skip = self.shortcut(x)
         for layer in self.residual:
             x = layer.stream(x, state) if isinstance(layer, CausalConv3d) else layer(x)
+        return x + skip
+
+    def forward_cl(self, x, state):
+        skip = self.shortcut.pointwise_cl(x) if isinstance(self.shortcut, CausalConv3d) else x
+        r = self.residual                       # norm, SiLU, conv, norm, SiLU, dropout(0), conv
+        x = r[2].stream_cl(x, state, norm=(r[0].gamma, True))
+        x = r[6].stream_cl(x, state, norm=(r[3].gamma, True))
         return x + skip
 
 
@@ -168,6 +222,13 @@ class AttentionBlock(nn.Module):
         o = F.scaled_dot_product_attention(qkv[:, 0:1], qkv[:, 1:2], qkv[:, 2:3])          # one head
         o = self.proj(o[:, 0].transpose(1, 2).reshape(b * t, c, h, w))
         return x + o.reshape(b, t, c, h, w).permute(0, 2, 1, 3, 4)
+
+    def forward_cl(self, x, state=None):
+        t, h, w, c = x.shape
+        qkv = F.linear(self.norm.forward_cl(x).reshape(t, h * w, c), self.to_qkv.weight.view(3 * c, c), self.to_qkv.bias)
+        q, k, v = (u.unsqueeze(1) for u in qkv.split(c, dim=-1))                           # [t, 1, hw, c]
+        o = F.scaled_dot_product_attention(q, k, v)[:, 0]
+        return x + F.linear(o, self.proj.weight.view(c, c), self.proj.bias).reshape(t, h, w, c)
 
 
 class Decoder3d(nn.Module):
@@ -201,6 +262,15 @@ class Decoder3d(nn.Module):
         x = self.head[1](self.head[0](x))
         return self.head[2].stream(x, state)
 
+    def forward_cl(self, x, state):
+        state.rewind()
+        x = self.conv1.stream_cl(x, state)
+        for layer in self.middle:
+            x = layer.forward_cl(x, state)
+        for layer in self.upsamples:
+            x = layer.forward_cl(x, state)
+        return self.head[2].stream_cl(x, state, norm=(self.head[0].gamma, True))
+
 
 class WanVAEDecoder(nn.Module):
     """`conv2` + `decoder` of the reference's WanVAE_ (vae.py:486-513) with the latent statistics of
@@ -230,18 +300,37 @@ class WanVAEDecoder(nn.Module):
         self.load_state_dict(picked, strict=True)
 
     # ---- decoding ---------------------------------------------------------------------------------
+    def _channels_last(self, z, state):
+        """Whether this call runs on the HIP convolution path; a stream keeps the path it started with."""
+        if state.layout is None:
+            ok = (z.is_cuda and z.shape[0] == 1 and z.dtype in (torch.bfloat16, torch.float16)
+                  and os.environ.get("SFM_VAE_TORCH_CONV", "0") != "1")
+            state.layout = "cl" if ok else "ncthw"
+        if state.layout == "cl" and z.shape[0] != 1:
+            raise ValueError("a channels-last decode stream carries one video")
+        return state.layout == "cl"
+
     def _frames(self, z, state):
         """z: [B, C, t, h, w] un-normalised latents -> [B, 3, t', 8h, 8w]."""
-        x = self.conv2(z)
+        if self._channels_last(z, state):
+            x = self.conv2.pointwise_cl(z[0].permute(1, 2, 3, 0))                  # [t, h, w, C]
+            run, cat_dim = self.decoder.forward_cl, 0
+            pick = lambda a, b: x[a:b]
+        else:
+            x = self.conv2(z)
+            run, cat_dim = self.decoder, 2
+            pick = lambda a, b: x[:, :, a:b]
+        n = z.shape[2]
         outs = []
         start = 0
         if state.frames_in == 0:
-            outs.append(self.decoder(x[:, :, :1], state))
+            outs.append(run(pick(0, 1), state))
             start = 1
-        if x.shape[2] > start:
-            outs.append(self.decoder(x[:, :, start:], state))
-        state.frames_in += x.shape[2]
-        return outs[0] if len(outs) == 1 else torch.cat(outs, dim=2)
+        if n > start:
+            outs.append(run(pick(start, n), state))
+        state.frames_in += n
+        out = outs[0] if len(outs) == 1 else torch.cat(outs, dim=cat_dim)
+        return out.permute(3, 0, 1, 2).unsqueeze(0) if state.layout == "cl" else out
 
     @torch.no_grad()
     def decode_stream(self, latent, state):

@@ -67,3 +67,22 @@ def test_conv_cl_rejects_bad_arguments():
     assert lib.sfm_conv3d_cl(C.byref(d), buf.data_ptr(), buf.data_ptr(), None, buf.data_ptr(), None) == -5      # stride
     d.x_stride[2] = 64
     assert lib.sfm_conv3d_cl(C.byref(d), None, buf.data_ptr(), None, buf.data_ptr(), None) == -1
+
+
+@pytest.mark.parametrize("C_,act,dt", [(96, True, torch.bfloat16), (192, True, torch.bfloat16), (384, False, torch.bfloat16),
+                                      (384, True, torch.float16), (32, False, torch.float16)])
+def test_norm_act_matches_fp32(C_, act, dt):
+    torch.manual_seed(C_)
+    x = torch.randn(3, 5, 7, C_, device="cuda").to(dt)
+    x[0, 0, 0] = 0                                                     # an all-zero voxel stays zero (clamped norm)
+    gamma = (1.0 + 0.3 * torch.randn(C_, 1, 1, 1, device="cuda")).to(dt)
+    big = torch.zeros(5, 7, 9, C_ + 32, device="cuda", dtype=dt)
+    out = big[2:, 1:6, 1:8, :C_]                                       # a strided view, like a padded conv input
+    co.norm_act(x, gamma, act, out=out)
+    xf = x.float()
+    ref = F.normalize(xf, dim=-1) * C_ ** 0.5 * gamma.float().view(-1)
+    if act:
+        ref = F.silu(ref)
+    tol = (2.0 ** -8 if dt == torch.bfloat16 else 2.0 ** -11) * max(1.0, ref.abs().max().item()) * 1.01
+    assert (out.float() - ref).abs().max().item() <= tol
+    assert big[:2].abs().max() == 0 and big[:, 0].abs().max() == 0 and big[..., C_:].abs().max() == 0   # nothing outside the view

@@ -57,3 +57,21 @@ def test_chunked_stream_equals_one_shot_on_the_device():
     # same arithmetic, but the convolutions see other batch shapes: equal up to the library's algorithm choice
     assert (got - whole).abs().max() < 1e-1
     assert (got - whole).abs().mean() < 4e-3
+
+
+def test_torch_and_hip_convolution_paths_agree(monkeypatch):
+    m = _decoder(torch.bfloat16, seed=6)
+    g = torch.Generator().manual_seed(7)
+    lat = torch.randn(1, 3, 16, 6, 8, generator=g).to(torch.bfloat16).cuda()
+    st = m.new_state()
+    fast = m.decode_to_pixel(lat, use_cache=True, state=st)
+    assert st.layout == "cl"
+    monkeypatch.setenv("SFM_VAE_TORCH_CONV", "1")
+    st2 = m.new_state()
+    slow = m.decode_to_pixel(lat, use_cache=True, state=st2)
+    assert st2.layout == "ncthw"
+    want = ov.decode_to_pixel(lat.double().cpu(), {k: v.cpu() for k, v in m.state_dict().items()})
+    e_fast, e_slow = (fast.cpu().double() - want).abs(), (slow.cpu().double() - want).abs()
+    # the HIP path is held to the error of the library path (both bf16 with fp32 accumulation)
+    assert e_fast.max() < 6e-2 and e_fast.mean() < 8e-3, (e_fast.max().item(), e_fast.mean().item())
+    assert e_fast.mean() < 2.0 * e_slow.mean() + 1e-3
