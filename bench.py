@@ -175,6 +175,26 @@ def op_level(torch, sfa, args):
     }
 
 
+def vae_decode_leg(torch, sfa):
+    """Streaming decode of one video's latents (outside the headline metric, which excludes the VAE): random-init
+    decoder of the Wan 2.1 VAE shape, bf16, 21 latent frames in 7 chunks of 3 -> 81 frames of 480x832."""
+    vae = sfa.vae_decode.WanVAEDecoder().eval().to("cuda", torch.bfloat16)
+    g = torch.Generator().manual_seed(0)
+    lat = torch.randn(1, 21, 16, 60, 104, generator=g).to(torch.bfloat16).cuda()
+    sec = None
+    for _ in range(2):                         # the first pass warms up
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        st, frames = vae.new_state(), 0
+        for c in range(7):
+            frames += vae.decode_to_pixel(lat[:, 3 * c:3 * c + 3], use_cache=True, state=st).shape[1]
+        torch.cuda.synchronize()
+        sec = time.perf_counter() - t0
+    return {"workload": "WanVAEDecoder (dim 96, z 16), 21 latent frames 60x104 in 7 chunks -> 81 frames 480x832, bf16, "
+                        "HIP channels-last convolutions", "ms_per_video": sec * 1e3, "pixel_frames_per_s": frames / sec,
+            "latent_frames_per_s": 21.0 / sec}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -225,6 +245,7 @@ def main():
         del pipe, gen
         torch.cuda.empty_cache()
     rec.update(op_level(torch, sfa, args))
+    rec["vae_decode"] = vae_decode_leg(torch, sfa)
     if args.op_only:
         rec["metric"] = "Monarch attn ms/call, causal Wan-1.3B 480x832 chunk shape, bf16"
         rec["unit"], rec["higher_is_better"] = "ms/call", False
