@@ -51,8 +51,9 @@ __device__ __forceinline__ void cv_load_lds16(const char* base, uint32_t off, ui
 }
 __device__ __forceinline__ void cv_wait_stage() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// CB: 32-channel blocks per wave; WN: waves along the output channels (the other 4 / WN waves split the voxels).
-template <class E, int CB, int WN>
+// CB: 32-channel blocks per wave; WN: waves along the output channels (the other 4 / WN waves split the voxels);
+// UP: the input is at half resolution (nearest x2 upsampling folded into the addresses).
+template <class E, int CB, int WN, bool UP>
 __global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
     constexpr int WM = 4 / WN;
     constexpr int kVox = 64 * WM;                         // voxels per workgroup
@@ -60,9 +61,8 @@ __global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
     constexpr int kCoRows = (kCo + 63) / 64 * 64;         // weight rows staged (whole groups of 16 per wave)
     constexpr int kRows = kCoRows + kVox;
     constexpr int kStage = kRows * kRowBytes;
-    constexpr int kGroups = kRows / 16;                   // 16-row groups, one load instruction each
-    constexpr int kPerWave = kGroups / 4;
-    static_assert(kGroups % 4 == 0, "rows must split evenly over the waves");
+    constexpr int kWG = kCoRows / 64;                     // 16-row groups (one load instruction each) of weights per wave
+    constexpr int kVG = kVox / 64;                        // ... of voxels per wave
     extern __shared__ __attribute__((aligned(256))) char lds[];
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
 
@@ -76,51 +76,59 @@ __global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
     // lane -> (line, quarter, chunk) of the group's 1 KB; the row sitting in that quarter is quarter ^ line
     const int g_line = lane >> 4, g_q = (lane >> 2) & 3, g_c = lane & 3;
     const int g_row = g_line * 4 + (g_q ^ g_line);
-    // weights: byte offset of the row (without tap and channel step); voxels: byte offset of the voxel's first tap
-    // (with up2x only its frame: rows and columns depend on the tap through the halving and are added per stage)
-    uint32_t src_off[kPerWave];
-    int vh[kPerWave], vw[kPerWave];
+    uint32_t w_off[kWG];                                  // byte offset of the weight row (without tap and channel step)
+    uint32_t x_off[kVG];                                  // byte offset of the voxel's first tap (with UP: of its frame only)
+    int vh[kVG], vw[kVG];
 #pragma unroll
-    for (int i = 0; i < kPerWave; ++i) {
-        const int row = (i * 4 + wave) * 16 + g_row;
-        vh[i] = vw[i] = 0;
-        if (row < kCoRows) {                              // wave-uniform: a group is all weights or all voxels
-            const int co = min(co0 + row, p.Cout_pad - 1);
-            src_off[i] = (uint32_t)(co * p.Cin * 2 + g_c * 16);
-        } else {
-            const int64_t v = min(v0 + (row - kCoRows), p.voxels - 1);   // rows past the end repeat the last voxel
-            const int w = (int)(v % p.W);
-            const int64_t r = v / p.W;
-            const int h = (int)(r % p.H), t = (int)(r / p.H);
-            vh[i] = h;
-            vw[i] = w;
-            const int64_t e = p.up2x ? t * p.xs_t : t * p.xs_t + h * p.xs_h + w * p.xs_w;
-            src_off[i] = (uint32_t)(e * 2 + g_c * 16);
-        }
+    for (int i = 0; i < kWG; ++i) {
+        const int co = min(co0 + (i * 4 + wave) * 16 + g_row, p.Cout_pad - 1);
+        w_off[i] = (uint32_t)(co * p.Cin * 2 + g_c * 16);
+    }
+#pragma unroll
+    for (int i = 0; i < kVG; ++i) {
+        const int64_t v = min(v0 + (i * 4 + wave) * 16 + g_row, p.voxels - 1);       // rows past the end repeat the last voxel
+        const int w = (int)(v % p.W);
+        const int64_t r = v / p.W;
+        const int h = (int)(r % p.H), t = (int)(r / p.H);
+        vh[i] = h;
+        vw[i] = w;
+        const int64_t e = UP ? t * p.xs_t : t * p.xs_t + h * p.xs_h + w * p.xs_w;
+        x_off[i] = (uint32_t)(e * 2 + g_c * 16);
     }
 
     const int cin_steps = p.Cin / kKC;
-    const int taps = p.kt * p.kh * p.kw;
-    const int nstage = taps * cin_steps;
+    const int nstage = p.kt * p.kh * p.kw * cin_steps;
+    const size_t w_tap = (size_t)p.Cout_pad * p.Cin * 2;  // bytes between taps of wt
 
-    auto stage = [&](int s, uint32_t buf) {
-        const int tap = s / cin_steps, cs = s - tap * cin_steps;
-        const int dw = tap % p.kw;
-        const int r = tap / p.kw;
-        const int dh = r % p.kh, dt = r / p.kh;
-        const char* wbase = p.wt + ((size_t)tap * p.Cout_pad * p.Cin + (size_t)cs * kKC) * 2;
-        const char* xbase = p.x + ((size_t)dt * p.xs_t + (size_t)cs * kKC) * 2;
-        if (!p.up2x) xbase += ((size_t)dh * p.xs_h + (size_t)dw * p.xs_w) * 2;
+    // position of the stage being fetched, advanced without divisions
+    int f_cs = 0, f_dw = 0, f_dh = 0, f_dt = 0;
+    const char* f_w = p.wt;                               // weights of the current tap
+    auto stage = [&](uint32_t buf) {
+        const char* wbase = f_w + (size_t)f_cs * (kKC * 2);
+        const char* xbase = p.x + ((size_t)f_dt * p.xs_t + (size_t)f_cs * kKC) * 2;
+        if (!UP) xbase += ((size_t)f_dh * p.xs_h + (size_t)f_dw * p.xs_w) * 2;
 #pragma unroll
-        for (int i = 0; i < kPerWave; ++i) {
-            const uint32_t dst = lds0 + buf + (uint32_t)(i * 4 + wave) * 1024;
-            if ((i * 4 + wave) * 16 < kCoRows) {
-                cv_load_lds16(wbase, src_off[i], dst);
-            } else if (!p.up2x) {
-                cv_load_lds16(xbase, src_off[i], dst);
+        for (int i = 0; i < kWG; ++i) cv_load_lds16(wbase, w_off[i], lds0 + buf + (uint32_t)(i * 4 + wave) * 1024);
+#pragma unroll
+        for (int i = 0; i < kVG; ++i) {
+            const uint32_t dst = lds0 + buf + (uint32_t)(kCoRows / 16 + i * 4 + wave) * 1024;
+            if (!UP) {
+                cv_load_lds16(xbase, x_off[i], dst);
             } else {
-                const int hh = ((vh[i] + dh - 1) >> 1) + 1, ww = ((vw[i] + dw - 1) >> 1) + 1;
-                cv_load_lds16(xbase, src_off[i] + (uint32_t)((hh * p.xs_h + ww * p.xs_w) * 2), dst);
+                // tap d of output position o reads padded low-resolution index ((o + d - 1) >> 1) + 1
+                const int hh = ((vh[i] + f_dh - 1) >> 1) + 1, ww = ((vw[i] + f_dw - 1) >> 1) + 1;
+                cv_load_lds16(xbase, x_off[i] + (uint32_t)((hh * p.xs_h + ww * p.xs_w) * 2), dst);
+            }
+        }
+        if (++f_cs == cin_steps) {
+            f_cs = 0;
+            f_w += w_tap;
+            if (++f_dw == p.kw) {
+                f_dw = 0;
+                if (++f_dh == p.kh) {
+                    f_dh = 0;
+                    ++f_dt;
+                }
             }
         }
     };
@@ -140,11 +148,11 @@ __global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
 #pragma unroll
     for (int vb = 0; vb < 2; ++vb) b_off[vb] = tile_off(kCoRows + 64 * wm + 32 * vb + m, hf);
 
-    stage(0, 0);
+    stage(0);
     for (int s = 0; s < nstage; ++s) {
         const uint32_t buf = (uint32_t)(s & 1) * kStage;
         cv_wait_stage();                                   // stage s is in LDS; the other buffer is free
-        if (s + 1 < nstage) stage(s + 1, buf ^ kStage);
+        if (s + 1 < nstage) stage(buf ^ kStage);
 #pragma unroll
         for (int ks = 0; ks < kKC / 16; ++ks) {
             u32x4 a[CB], b[2];
@@ -207,7 +215,8 @@ int launch_cfg(const ConvArgs& a, hipStream_t st) {
     constexpr int kVox = 64 * (4 / WN), kCo = 32 * CB * WN, kCoRows = (kCo + 63) / 64 * 64;
     constexpr int ldsb = 2 * (kCoRows + kVox) * kRowBytes;
     dim3 grid((unsigned)((a.voxels + kVox - 1) / kVox), (unsigned)((a.Cout_pad + kCo - 1) / kCo));
-    hipLaunchKernelGGL((conv3d_cl_kernel<E, CB, WN>), grid, dim3(256), ldsb, st, a);
+    if (a.up2x) hipLaunchKernelGGL((conv3d_cl_kernel<E, CB, WN, true>), grid, dim3(256), ldsb, st, a);
+    else hipLaunchKernelGGL((conv3d_cl_kernel<E, CB, WN, false>), grid, dim3(256), ldsb, st, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("sfm_conv3d_cl: launch failed: %s", hipGetErrorString(e));
