@@ -3,6 +3,11 @@ import sys
 
 import pytest
 
+# The few tests that run torch's own convolutions on the GPU (the VAE decoder's library path) would otherwise spend
+# most of a minute in the convolution library's exhaustive algorithm search, and log every missing solver.
+os.environ.setdefault("MIOPEN_FIND_MODE", "2")
+os.environ.setdefault("MIOPEN_LOG_LEVEL", "1")
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
