@@ -209,8 +209,10 @@ typedef struct sfm_conv_desc {
  * convolutions :186-220, :423-472).  `x` is the input with its kt - 1 history (or zero) frames in front and,
  * for a 3x3 spatial kernel, a one-pixel zero border, i.e. [T + kt - 1][H + kh - 1][W + kw - 1][Cin] (with up2x:
  * [T + kt - 1][H/2 + 2][W/2 + 2][Cin]); `wt` is the weight as [kt][kh][kw][Cout_pad][Cin]; `bias` (fp32, [Cout])
- * may be NULL; `y` is [T][H][W][Cout].  One call's input must stay below 4 GiB. */
-int sfm_conv3d_cl(const sfm_conv_desc* desc, const void* x, const void* wt, const float* bias, void* y, void* stream);
+ * may be NULL; `res` (a residual input added to the result, the `x + h` of vae.py:220; same layout and strides as
+ * `y`) may be NULL; `y` is [T][H][W][Cout].  One call's input must stay below 4 GiB. */
+int sfm_conv3d_cl(const sfm_conv_desc* desc, const void* x, const void* wt, const float* bias, const void* res, void* y,
+                  void* stream);
 
 /* RMS norm over the channels with optional SiLU for channels-last activations [T][H][W][C]: y = x / max(|x|_2, 1e-12)
  * * sqrt(C) * gamma, then y * sigmoid(y) if act != 0 (wan/modules/vae.py:39-54 and the nn.SiLU that follows it in

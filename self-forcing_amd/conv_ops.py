@@ -49,11 +49,12 @@ def norm_act(x, gamma, act, out=None):
     return out
 
 
-def conv_cl(x, conv, history=None, up2x=False, norm=None, want_tail=False):
+def conv_cl(x, conv, history=None, up2x=False, norm=None, want_tail=False, res=None):
     """x [T, H, W, Cin] -> [T, H', W', Cout] for a causal Conv3d (kt - 1 frames of `history`, zeros where it is
     shorter) or a Conv2d applied per frame; with up2x the nearest x2 upsampling in front of a 3x3 Conv2d is folded
     into the convolution (H' = 2 H, W' = 2 W).  With norm = (gamma, act) the convolution's input is
-    norm_act(x, gamma, act), written straight into the padded buffer.  With want_tail the last two frames of the
+    norm_act(x, gamma, act), written straight into the padded buffer.  `res` [T, H', W', Cout] is added to the result
+    inside the kernel.  With want_tail the last two frames of the
     (history + input) sequence come back as well: what the next call of a stream passes as `history`."""
     if x.dtype not in _DT:
         raise TypeError(f"conv_cl: dtype {x.dtype} (bf16 or fp16 only)")
@@ -75,6 +76,10 @@ def conv_cl(x, conv, history=None, up2x=False, norm=None, want_tail=False):
             norm_act(x, norm[0], norm[1], out=inner)
     Ho, Wo = (2 * H, 2 * W) if up2x else (H, W)
     y = torch.empty(T, Ho, Wo, cout, dtype=x.dtype, device=x.device)
+    if res is not None and (res.shape != y.shape or res.dtype != y.dtype):
+        raise ValueError(f"conv_cl: res {tuple(res.shape)} {res.dtype} does not match the output {tuple(y.shape)} {y.dtype}")
+    if res is not None:
+        res = res.contiguous()
     d = L.ConvDesc()
     d.dtype = _DT[x.dtype]
     d.T, d.H, d.W = T, Ho, Wo
@@ -87,7 +92,7 @@ def conv_cl(x, conv, history=None, up2x=False, norm=None, want_tail=False):
     lib = L.load()
     stream = torch.cuda.current_stream(x.device).cuda_stream
     L.check(lib.sfm_conv3d_cl(C.byref(d), xp.data_ptr(), wt.data_ptr(), bias.data_ptr() if bias is not None else None,
-                              y.data_ptr(), stream))
+                              res.data_ptr() if res is not None else None, y.data_ptr(), stream))
     if want_tail:
         n = min(2, T + past)
         return y, xp[T + past - n:, pad:pad + H, pad:pad + W, :cin].clone()

@@ -1,7 +1,7 @@
 // Channels-last 3-D convolution as an implicit GEMM on gfx950 MFMA (bf16 / fp16), for the streaming VAE decoder
 // (replaces the nn.Conv3d / nn.Conv2d calls of wan/modules/vae.py:17-36, :76-97, :186-220, :423-472).
 //
-//   y[t, h, w, co] = bias[co] + sum_{dt, dh, dw, ci}  wt[dt, dh, dw, co, ci] * xp[t + dt, h' + dh, w' + dw, ci]
+//   y[t, h, w, co] = bias[co] + res[t, h, w, co] + sum_{dt, dh, dw, ci}  wt[dt, dh, dw, co, ci] * xp[t + dt, h' + dh, w' + dw, ci]
 //
 // xp is the input with its zero (or history) frames and its zero border already in place, so the kernel has no
 // bounds tests; with `up2x` it is the half-resolution tensor and (h', w') = the row / column of xp that the
@@ -30,6 +30,7 @@ struct ConvArgs {
     const char* x;            // padded input, channels-last
     const char* wt;           // [taps][Cout_pad][Cin] (ci contiguous)
     const float* bias;        // [Cout] or null
+    const char* res;          // residual input laid out like y, or null
     char* y;
     int T, H, W;              // output grid
     int Cin, Cout, Cout_pad;
@@ -180,6 +181,25 @@ __global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
             const int cbase = co0 + 32 * (cb + CB * wn);
+            if (p.res != nullptr && vok) {
+                // the block of the voxel that this lane completes: channels 8 g + 4 hf + 0..3
+                const char* rrow = p.res + (t * p.ys_t + h * p.ys_h + w * p.ys_w) * 2;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int co = cbase + 8 * g + 4 * hf;
+                    if (co + 4 <= p.Cout) {
+                        const u32x2 rv = *(const u32x2*)(rrow + co * 2);
+                        acc[cb][vb][4 * g + 0] += E::to_float((uint16_t)(rv.x & 0xffffu));
+                        acc[cb][vb][4 * g + 1] += E::to_float((uint16_t)(rv.x >> 16));
+                        acc[cb][vb][4 * g + 2] += E::to_float((uint16_t)(rv.y & 0xffffu));
+                        acc[cb][vb][4 * g + 3] += E::to_float((uint16_t)(rv.y >> 16));
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (co + e < p.Cout) acc[cb][vb][4 * g + e] += E::to_float(*(const uint16_t*)(rrow + (co + e) * 2));
+                    }
+                }
+            }
             if (p.bias != nullptr) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
@@ -307,7 +327,8 @@ int launch_norm(const NormArgs& a, hipStream_t st) {
 }  // namespace
 }  // namespace sfm
 
-extern "C" int sfm_conv3d_cl(const sfm_conv_desc* d, const void* x, const void* wt, const float* bias, void* y, void* stream) {
+extern "C" int sfm_conv3d_cl(const sfm_conv_desc* d, const void* x, const void* wt, const float* bias, const void* res, void* y,
+                             void* stream) {
     using namespace sfm;
     if (d == nullptr || x == nullptr || wt == nullptr || y == nullptr) {
         set_error("sfm_conv3d_cl: null argument");
@@ -340,7 +361,7 @@ extern "C" int sfm_conv3d_cl(const sfm_conv_desc* d, const void* x, const void* 
         set_error("sfm_conv3d_cl: the input of one call must stay below 4 GiB (%lld bytes)", (long long)span);
         return SFM_ERR_RANGE;
     }
-    if ((((uintptr_t)x | (uintptr_t)wt) & 15) || ((uintptr_t)y & (d->Cout >= 32 ? 15 : 1))) {
+    if ((((uintptr_t)x | (uintptr_t)wt) & 15) || (((uintptr_t)y | (uintptr_t)res) & (d->Cout >= 32 ? 15 : 1))) {
         set_error("sfm_conv3d_cl: x, wt, y must be 16-byte aligned");
         return SFM_ERR_ALIGN;
     }
@@ -348,6 +369,7 @@ extern "C" int sfm_conv3d_cl(const sfm_conv_desc* d, const void* x, const void* 
     a.x = (const char*)x;
     a.wt = (const char*)wt;
     a.bias = bias;
+    a.res = (const char*)res;
     a.y = (char*)y;
     a.T = d->T; a.H = d->H; a.W = d->W;
     a.Cin = d->Cin; a.Cout = d->Cout; a.Cout_pad = d->Cout_pad;

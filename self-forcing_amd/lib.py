@@ -101,7 +101,7 @@ def load():
     lib.sfm_gate_residual_ln.argtypes = [C.c_int32, I64, C.c_int32, C.c_float, P, I64, P, I64, P, I64, C.c_int32, P, I64, P, P, I64,
                                          C.c_int32, P, P, P]
     lib.sfm_rms_norm.argtypes = [C.c_int32, I64, C.c_int32, C.c_float, P, I64, P, I64, P, P]
-    lib.sfm_conv3d_cl.argtypes = [C.POINTER(ConvDesc), P, P, P, P, P]
+    lib.sfm_conv3d_cl.argtypes = [C.POINTER(ConvDesc), P, P, P, P, P, P]
     lib.sfm_vae_norm_act.argtypes = [C.c_int32] * 6 + [P, S3, P, P, S3, P]
     lib.sfm_probe_mfma_bf16.argtypes = [C.c_int32, P, C.POINTER(C.c_float)]
     for name in SYMBOLS:

@@ -86,14 +86,14 @@ class CausalConv3d(nn.Conv3d):
         state.tails[i] = tail
         return y
 
-    def stream_cl(self, x, state, norm=None):
+    def stream_cl(self, x, state, norm=None, res=None):
         """`stream` for channels-last activations [T, H, W, C]; with norm = (gamma, act) the convolution's input is
-        the RMS norm (+ SiLU) of x.  The tail kept is always two frames (a zero frame stands in before the stream
+        the RMS norm (+ SiLU) of x and `res` is added to the result.  The tail kept is always two frames (a zero frame stands in before the stream
         has two), which the convolution treats exactly like the reference's shorter cache plus zero padding."""
         from . import conv_ops
         i = state.take()
         prev = state.tails[i]
-        y, tail = conv_ops.conv_cl(x, self, prev if isinstance(prev, torch.Tensor) else None, norm=norm, want_tail=True)
+        y, tail = conv_ops.conv_cl(x, self, prev if isinstance(prev, torch.Tensor) else None, norm=norm, want_tail=True, res=res)
         state.tails[i] = tail
         return y
 
@@ -201,8 +201,7 @@ class ResidualBlock(nn.Module):
         skip = self.shortcut.pointwise_cl(x) if isinstance(self.shortcut, CausalConv3d) else x
         r = self.residual                       # norm, SiLU, conv, norm, SiLU, dropout(0), conv
         x = r[2].stream_cl(x, state, norm=(r[0].gamma, True))
-        x = r[6].stream_cl(x, state, norm=(r[3].gamma, True))
-        return x + skip
+        return r[6].stream_cl(x, state, norm=(r[3].gamma, True), res=skip)          # the residual sum happens in the kernel
 
 
 class AttentionBlock(nn.Module):

@@ -61,12 +61,24 @@ def test_conv_cl_rejects_bad_arguments():
     buf = torch.zeros(1 << 16, dtype=torch.bfloat16, device="cuda")
     for i in range(3):
         d.x_stride[i] = d.y_stride[i] = 64
-    assert lib.sfm_conv3d_cl(C.byref(d), buf.data_ptr(), buf.data_ptr(), None, buf.data_ptr(), None) == -3      # Cin % 32
+    assert lib.sfm_conv3d_cl(C.byref(d), buf.data_ptr(), buf.data_ptr(), None, None, buf.data_ptr(), None) == -3      # Cin % 32
     d.Cin = 64
     d.x_stride[2] = 60
-    assert lib.sfm_conv3d_cl(C.byref(d), buf.data_ptr(), buf.data_ptr(), None, buf.data_ptr(), None) == -5      # stride
+    assert lib.sfm_conv3d_cl(C.byref(d), buf.data_ptr(), buf.data_ptr(), None, None, buf.data_ptr(), None) == -5      # stride
     d.x_stride[2] = 64
-    assert lib.sfm_conv3d_cl(C.byref(d), None, buf.data_ptr(), None, buf.data_ptr(), None) == -1
+    assert lib.sfm_conv3d_cl(C.byref(d), None, buf.data_ptr(), None, None, buf.data_ptr(), None) == -1
+
+
+@pytest.mark.parametrize("cout", [96, 3])
+def test_conv_cl_adds_the_residual_input(cout):
+    torch.manual_seed(cout)
+    conv = nn.Conv3d(96, cout, 3).cuda().to(torch.bfloat16)
+    x = torch.randn(2, 6, 9, 96, device="cuda").to(torch.bfloat16)
+    res = torch.randn(2, 6, 9, cout, device="cuda").to(torch.bfloat16)
+    y = co.conv_cl(x, conv, None, res=res)
+    xf = F.pad(x.float().permute(3, 0, 1, 2).unsqueeze(0), (1, 1, 1, 1, 2, 0))
+    ref = F.conv3d(xf, conv.weight.float(), conv.bias.float())[0].permute(1, 2, 3, 0) + res.float()
+    assert (y.float() - ref).abs().max().item() <= 2.0 ** -8 * max(1.0, ref.abs().max().item()) * 1.01
 
 
 @pytest.mark.parametrize("C_,act,dt", [(96, True, torch.bfloat16), (192, True, torch.bfloat16), (384, False, torch.bfloat16),
