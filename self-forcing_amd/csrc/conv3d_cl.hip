@@ -101,34 +101,42 @@ __global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
     const int nstage = p.kt * p.kh * p.kw * cin_steps;
     const size_t w_tap = (size_t)p.Cout_pad * p.Cin * 2;  // bytes between taps of wt
 
-    // position of the stage being fetched, advanced without divisions
-    int f_cs = 0, f_dw = 0, f_dh = 0, f_dt = 0;
-    const char* f_w = p.wt;                               // weights of the current tap
+    // position of the stage being fetched: channel step, tap column, tap row; the source pointers move by precomputed
+    // deltas, so that issuing a stage costs a handful of scalar instructions
+    int f_cs = 0, f_dw = 0, f_dh = 0;
+    const char* f_w = p.wt;
+    const char* f_x = p.x;
+    const int64_t step_tap_w = (int64_t)w_tap - (int64_t)p.Cin * 2;                           // last channel step of a tap -> next tap's first
+    const int64_t step_dw = (UP ? 0 : p.xs_w * 2) - (int64_t)p.Cin * 2;                       // next tap column
+    const int64_t step_dh = UP ? 0 : (p.xs_h - (int64_t)p.kw * p.xs_w) * 2;                   // next tap row
+    const int64_t step_dt = (UP ? p.xs_t : p.xs_t - (int64_t)p.kh * p.xs_h) * 2;              // next tap frame
     auto stage = [&](uint32_t buf) {
-        const char* wbase = f_w + (size_t)f_cs * (kKC * 2);
-        const char* xbase = p.x + ((size_t)f_dt * p.xs_t + (size_t)f_cs * kKC) * 2;
-        if (!UP) xbase += ((size_t)f_dh * p.xs_h + (size_t)f_dw * p.xs_w) * 2;
+        const uint32_t mb = lds0 + buf + (uint32_t)wave * 1024;
 #pragma unroll
-        for (int i = 0; i < kWG; ++i) cv_load_lds16(wbase, w_off[i], lds0 + buf + (uint32_t)(i * 4 + wave) * 1024);
+        for (int i = 0; i < kWG; ++i) cv_load_lds16(f_w, w_off[i], mb + (uint32_t)i * 4096);
 #pragma unroll
         for (int i = 0; i < kVG; ++i) {
-            const uint32_t dst = lds0 + buf + (uint32_t)(kCoRows / 16 + i * 4 + wave) * 1024;
+            const uint32_t dst = mb + (uint32_t)(kCoRows / 16 + i * 4) * 1024;
             if (!UP) {
-                cv_load_lds16(xbase, x_off[i], dst);
+                cv_load_lds16(f_x, x_off[i], dst);
             } else {
                 // tap d of output position o reads padded low-resolution index ((o + d - 1) >> 1) + 1
                 const int hh = ((vh[i] + f_dh - 1) >> 1) + 1, ww = ((vw[i] + f_dw - 1) >> 1) + 1;
-                cv_load_lds16(xbase, x_off[i] + (uint32_t)((hh * p.xs_h + ww * p.xs_w) * 2), dst);
+                cv_load_lds16(f_x, x_off[i] + (uint32_t)((hh * p.xs_h + ww * p.xs_w) * 2), dst);
             }
         }
+        f_w += kKC * 2;
+        f_x += kKC * 2;
         if (++f_cs == cin_steps) {
             f_cs = 0;
-            f_w += w_tap;
+            f_w += step_tap_w;
+            f_x += step_dw;
             if (++f_dw == p.kw) {
                 f_dw = 0;
+                f_x += step_dh;
                 if (++f_dh == p.kh) {
                     f_dh = 0;
-                    ++f_dt;
+                    f_x += step_dt;
                 }
             }
         }
