@@ -244,6 +244,7 @@ def main():
         rec["ms_per_step"] = sec * 1e3
         del pipe, gen
         torch.cuda.empty_cache()
+        torch.cuda.tunable.tuning_enable(False)       # the legs below keep the selections made so far and tune nothing new
     rec.update(op_level(torch, sfa, args))
     rec["vae_decode"] = vae_decode_leg(torch, sfa)
     if args.op_only:
