@@ -91,3 +91,23 @@ def test_windowed_rollout_with_ring_cache_matches_shifting_cache_on_cpu():
     assert pipe.kv_cache1[0]["_ring"] and pipe.kv_cache1[0]["_local_end"] == 3 * 312      # third chunk wrapped to the start
     for c in range(3):
         assert _cos(out[:, 3 * c:3 * c + 3], out_ref[:, 3 * c:3 * c + 3]) > 0.995
+
+
+def test_pipeline_decodes_each_chunk_as_it_is_finished():
+    """inference(vae=...) hands every clean chunk to one decode stream; the pixels equal decoding the finished latents in
+    one go (pipeline/causal_inference.py:265) up to the convolution kernels' 16-bit rounding per call shape."""
+    from self_forcing_amd import vae_decode as vd
+    g = torch.Generator().manual_seed(0)
+    noise = torch.randn(1, 6, 16, 12, 104, generator=g).to(torch.bfloat16).to("cuda:0")
+    ctx = torch.randn(1, 16, 64, generator=g).to(torch.bfloat16).to("cuda:0")
+    _, dev_gen = _pair(use_framewise=True)
+    torch.manual_seed(3)
+    vae = vd.WanVAEDecoder(dim=32).eval().to("cuda:0", torch.bfloat16)
+    pipe = pl.CausalInferencePipeline(dev_gen, frame_hw=(6, 52), num_cache_frames=6)
+    latents, video = pipe.inference(noise, ctx, vae=vae)
+    assert video.shape == (1, 1 + 4 * 5, 3, 96, 832) and torch.isfinite(video).all()
+    whole = vae.decode_to_pixel(latents)
+    assert (video - whole).abs().max() < 5e-2 and (video - whole).abs().mean() < 3e-3
+    seen = []
+    pipe.inference(noise, ctx, vae=vae, on_pixels=lambda i, px: seen.append((i, px.shape[1])))
+    assert seen == [(0, 9), (1, 12)]

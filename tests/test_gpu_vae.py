@@ -75,3 +75,20 @@ def test_torch_and_hip_convolution_paths_agree(monkeypatch):
     # the HIP path is held to the error of the library path (both bf16 with fp32 accumulation)
     assert e_fast.max() < 6e-2 and e_fast.mean() < 8e-3, (e_fast.max().item(), e_fast.mean().item())
     assert e_fast.mean() < 2.0 * e_slow.mean() + 1e-3
+
+
+def test_fp16_decode_streams_on_the_hip_path():
+    """The demo runs its decoder in fp16 (demo.py:430)."""
+    m = _decoder(torch.float16, seed=8)
+    g = torch.Generator().manual_seed(9)
+    lat = torch.randn(1, 4, 16, 5, 7, generator=g).to(torch.float16)
+    want = ov.decode_to_pixel(lat.double(), {k: v.cpu() for k, v in m.state_dict().items()})
+    st, outs = m.new_state(), []
+    for t0, t1 in ((0, 1), (1, 4)):
+        outs.append(m.decode_to_pixel(lat[:, t0:t1].cuda(), use_cache=True, state=st))
+    assert st.layout == "cl"
+    got = torch.cat(outs, 1).cpu().double()
+    assert got.shape == want.shape == (1, 13, 3, 40, 56)
+    err = (got - want).abs()
+    assert err.max() < 1.5e-2 and err.mean() < 2e-3, (err.max().item(), err.mean().item())
+
