@@ -17,6 +17,8 @@
 //   dR = dKbar.K + dY.V + dc ln R            dS1 = R (dR - sum_l R dR)
 //   dQ = s dS2 Kbar + s dS1 K                dK = R^T dKbar + s dS1^T q         dV = R^T dY
 
+#include <cstdlib>
+
 #include "sfm_common.hpp"
 
 #include <dlfcn.h>
@@ -315,6 +317,29 @@ __global__ __launch_bounds__(256) void softmax_right_bwd(const float* S1, const 
     }
 }
 
+// The same with R read back (16 bit, row pitch 64, rows [t][aj]) instead of recomputed from the logits.
+template <typename E>
+__global__ __launch_bounds__(256) void softmax_right_bwd_r(const typename El<E>::type* Rb, const float* dRb, const float* dc,
+                                                           typename El<E>::type* dS1, int b1, int AJ, int nf, int b2, int64_t nseg) {
+    const int64_t seg = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (seg >= nseg) return;
+    const int lane = threadIdx.x & 63;
+    const int f = (int)(seg % nf);
+    const int64_t row = seg / nf;
+    const int aj = (int)(row % AJ);
+    const int64_t uk = row / AJ;
+    const int k = (int)(uk % b1);
+    const int64_t u = uk / b1;
+    const int64_t blk = (uk * nf + f) * AJ + aj;
+    const float dcv = dc[(u * AJ + aj) * ((int64_t)nf * b1) + (int64_t)k * nf + f];
+    const bool in = lane < b2;                          // b2 <= 64 on this path
+    const float r = in ? El<E>::get(Rb, blk * 64 + lane) : 0.f;
+    float gv = in ? dRb[blk * b2 + lane] : 0.f;
+    if (r > 0.f) gv += dcv * __logf(r);                 // dR + dc ln R
+    const float dot = wave_sum(r * gv);
+    if (in) El<E>::put(dS1, seg * b2 + lane, r * (gv - dot));
+}
+
 // dq[token row of (a, i, j)] = dQa[u][aj][i][:] (left factor) + dQk[u][i][aj][:] (right factor)
 __global__ __launch_bounds__(256) void scatter_dq(const float* dQa, const float* dQk, float* dq, int64_t s0, int64_t s1, int64_t s2,
                                                   TokMap map, int na, int H, int D, int unit0, int64_t total) {
@@ -384,7 +409,7 @@ Layout make_layout(const MonarchArgs& p, int n, size_t e) {
     l.Vk = take(n * MK * D * e);
     l.S1f = take(n * p.b1 * AJ * NL * 4);
     l.dRb = take(n * p.b1 * AJ * NL * 4);
-    l.Rb = take(n * p.b1 * AJ * NL * e);
+    l.Rb = take(n * p.b1 * AJ * p.nf * (size_t)(p.b2 > 64 ? p.b2 : 64) * e);      // row pitch 64 when step 1 of the forward writes it
     l.dS1 = take(n * p.b1 * AJ * NL * e);
     l.Kbar = take(n * AJ * RR * D * e);
     l.Y = take(n * AJ * RR * D * e);
@@ -433,6 +458,11 @@ void gemm(Ctx& cx, bool ta, bool tb, int M, int N, int K, float alpha, float bet
     }
 }
 
+// dtype code of the fused left-factor kernel for operand type E, or -1 (fp32 operands stay on the GEMMs)
+template <typename E> constexpr int left_dtype() { return -1; }
+template <> constexpr int left_dtype<BF16>() { return SFM_BF16; }
+template <> constexpr int left_dtype<F16>() { return SFM_F16; }
+
 template <typename E>
 int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     typedef typename El<E>::type T;
@@ -477,50 +507,86 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     // operands per t = (u, k, f): [b2 x D] blocks of K, V, dK, dV; [AJ x b2] blocks of R, dR; [AJ x D] blocks of Kbar, Y, dKbar, dY
     const Op Kk_t{lay.Kk, D, (int64_t)b2 * D}, Vk_t{lay.Vk, D, (int64_t)b2 * D};
     const Op dKk_t{lay.dKk, D, (int64_t)b2 * D}, dVk_t{lay.dVk, D, (int64_t)b2 * D};
-    const Op Rb_t{lay.Rb, b2, (int64_t)AJ * b2}, dRb_t{lay.dRb, b2, (int64_t)AJ * b2};
+    const Op dRb_t{lay.dRb, b2, (int64_t)AJ * b2};
     const Op Kbar_t{lay.Kbar, D, (int64_t)AJ * D}, Y_t{lay.Y, D, (int64_t)AJ * D};
     const Op dKbar_t{lay.dKbar, D, (int64_t)AJ * D}, dY_t{lay.dY, D, (int64_t)AJ * D};
 
     const int64_t nseg = (int64_t)n * b1 * AJ * nf;
-    // 1. S1 = Qk Kk^T per (u, k)
-    gemm(cx, false, true, AJ, NL, D, 1.f, 0.f, Qk_uk, Kk_uk, S1_uk, tE, tF, nuk);
-    hipLaunchKernelGGL((softmax_right<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const float*)(ws + lay.S1f),
-                       (T*)(ws + lay.Rb), (float*)(ws + lay.c), b1, AJ, nf, b2, s, nseg);
-    // 2, 3. Kbar, Y blocks = R block . K / V block per t
-    gemm(cx, false, false, AJ, D, b2, 1.f, 0.f, Rb_t, Kk_t, Kbar_t, tE, tE, nt);
-    gemm(cx, false, false, AJ, D, b2, 1.f, 0.f, Rb_t, Vk_t, Y_t, tE, tE, nt);
-    // 4, 5. per unit and (a, j): S2 = q_i . Kbar_r, dLm = dO_i . Y_r; the [RR x D] matrix of column aj is every AJ-th row
-    for (int u = 0; u < n && !cx.status; ++u) {
-        const Op Qa_u{lay.Qa + (size_t)u * MQ * D * e, D, (int64_t)b1 * D}, dOa_u{lay.dOa + (size_t)u * MQ * D * e, D, (int64_t)b1 * D};
-        const Op Kbar_u{lay.Kbar + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D}, Y_u{lay.Y + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D};
-        const Op S2_u{lay.S2f + (size_t)u * AJ * b1 * RR * 4, RR, (int64_t)b1 * RR}, dLm_u{lay.dLmf + (size_t)u * AJ * b1 * RR * 4, RR, (int64_t)b1 * RR};
-        gemm(cx, false, true, b1, RR, D, 1.f, 0.f, Qa_u, Kbar_u, S2_u, tE, tF, AJ);
-        gemm(cx, false, true, b1, RR, D, 1.f, 0.f, dOa_u, Y_u, dLm_u, tE, tF, AJ);
+    const bool fused_left = left_dtype<E>() >= 0 && monarch_bwd_left_supported(left_dtype<E>(), D, b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
+    // the forward's MFMA step 1 recomputes Kbar, Y, c and R straight into this scratch ([t][aj] rows)
+    const bool fused_fwd = fused_left && monarch_mfma_supported(left_dtype<E>(), D, b2) && getenv("SFM_BWD_FWD_GEMM") == nullptr;
+    const int rb_ld = fused_fwd ? 64 : b2;
+    const Op Rb_t{lay.Rb, rb_ld, (int64_t)AJ * rb_ld};
+    if (fused_fwd) {
+        MonarchArgs f1 = p;
+        f1.kbar = ws + lay.Kbar;
+        f1.y = ws + lay.Y;
+        f1.cl = (float*)(ws + lay.c);
+        f1.rb = ws + lay.Rb;
+        f1.ws_unit = (uint32_t)((int64_t)RR * AJ);
+        f1.ws_aj = 1;
+        f1.ws_row = (uint32_t)(nf * AJ);
+        f1.ws_f = (uint32_t)AJ;
+        if (!cx.status) cx.status = launch_monarch_step1(f1, left_dtype<E>(), n, stream);
+    } else {
+        // 1. S1 = Qk Kk^T per (u, k)
+        gemm(cx, false, true, AJ, NL, D, 1.f, 0.f, Qk_uk, Kk_uk, S1_uk, tE, tF, nuk);
+        hipLaunchKernelGGL((softmax_right<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const float*)(ws + lay.S1f),
+                           (T*)(ws + lay.Rb), (float*)(ws + lay.c), b1, AJ, nf, b2, s, nseg);
+        // 2, 3. Kbar, Y blocks = R block . K / V block per t
+        gemm(cx, false, false, AJ, D, b2, 1.f, 0.f, Rb_t, Kk_t, Kbar_t, tE, tE, nt);
+        gemm(cx, false, false, AJ, D, b2, 1.f, 0.f, Rb_t, Vk_t, Y_t, tE, tE, nt);
     }
-    hipLaunchKernelGGL((softmax_left<E>), dim3((unsigned)((int64_t)n * AJ * b1)), dim3(256), 0, stream, (const float*)(ws + lay.S2f),
-                       (const float*)(ws + lay.dLmf), (const float*)(ws + lay.c), (T*)(ws + lay.L), (T*)(ws + lay.dS2), b1, b2, AJ, nf,
-                       p.causal, s);
-    {
-        const int64_t tot = (int64_t)n * AJ * RR;
-        hipLaunchKernelGGL((reduce_dc<E>), dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, stream, (const T*)(ws + lay.dS2),
-                           (float*)(ws + lay.dc), b1, AJ, RR, tot);
+    if (fused_left) {
+        // 4-7 in one kernel: statistics and gradients of the left factor without the [i x r] matrices in memory
+        if (!cx.status)
+            cx.status = launch_monarch_bwd_left(left_dtype<E>(), D, n, b1, b2, AJ, nf, p.causal, s, ws + lay.Qa, ws + lay.dOa, ws + lay.Kbar,
+                                                ws + lay.Y, (const float*)(ws + lay.c), fused_fwd ? 1 : 0, ws + lay.dKbar, ws + lay.dY,
+                                                (float*)(ws + lay.dc), ws + lay.dS2, stream);
+    } else {
+        // 4, 5. per unit and (a, j): S2 = q_i . Kbar_r, dLm = dO_i . Y_r; the [RR x D] matrix of column aj is every AJ-th row
+        for (int u = 0; u < n && !cx.status; ++u) {
+            const Op Qa_u{lay.Qa + (size_t)u * MQ * D * e, D, (int64_t)b1 * D}, dOa_u{lay.dOa + (size_t)u * MQ * D * e, D, (int64_t)b1 * D};
+            const Op Kbar_u{lay.Kbar + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D}, Y_u{lay.Y + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D};
+            const Op S2_u{lay.S2f + (size_t)u * AJ * b1 * RR * 4, RR, (int64_t)b1 * RR}, dLm_u{lay.dLmf + (size_t)u * AJ * b1 * RR * 4, RR, (int64_t)b1 * RR};
+            gemm(cx, false, true, b1, RR, D, 1.f, 0.f, Qa_u, Kbar_u, S2_u, tE, tF, AJ);
+            gemm(cx, false, true, b1, RR, D, 1.f, 0.f, dOa_u, Y_u, dLm_u, tE, tF, AJ);
+        }
+        hipLaunchKernelGGL((softmax_left<E>), dim3((unsigned)((int64_t)n * AJ * b1)), dim3(256), 0, stream, (const float*)(ws + lay.S2f),
+                           (const float*)(ws + lay.dLmf), (const float*)(ws + lay.c), (T*)(ws + lay.L), (T*)(ws + lay.dS2), b1, b2, AJ, nf,
+                           p.causal, s);
+        {
+            const int64_t tot = (int64_t)n * AJ * RR;
+            hipLaunchKernelGGL((reduce_dc<E>), dim3((unsigned)((tot + 255) / 256)), dim3(256), 0, stream, (const T*)(ws + lay.dS2),
+                               (float*)(ws + lay.dc), b1, AJ, RR, tot);
+        }
+        // 6, 7, 8. per unit and (a, j): dY = L^T dO, dKbar = s dS2^T q, dQ (left factor) = s dS2 Kbar
+        for (int u = 0; u < n && !cx.status; ++u) {
+            const Op Qa_u{lay.Qa + (size_t)u * MQ * D * e, D, (int64_t)b1 * D}, dOa_u{lay.dOa + (size_t)u * MQ * D * e, D, (int64_t)b1 * D};
+            const Op Kbar_u{lay.Kbar + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D};
+            const Op dKbar_u{lay.dKbar + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D}, dY_u{lay.dY + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D};
+            const Op L_u{lay.L + (size_t)u * AJ * b1 * RR * e, RR, (int64_t)b1 * RR}, dS2_u{lay.dS2 + (size_t)u * AJ * b1 * RR * e, RR, (int64_t)b1 * RR};
+            const Op dQa_u{lay.dQa + (size_t)u * MQ * D * 4, D, (int64_t)b1 * D};
+            gemm(cx, true, false, RR, D, b1, 1.f, 0.f, L_u, dOa_u, dY_u, tE, tE, AJ);
+            gemm(cx, true, false, RR, D, b1, s, 0.f, dS2_u, Qa_u, dKbar_u, tE, tE, AJ);
+        }
     }
-    // 6, 7, 8. per unit and (a, j): dY = L^T dO, dKbar = s dS2^T q, dQ (left factor) = s dS2 Kbar
+    // 8. per unit and (a, j): dQ (left factor) = s dS2 Kbar
     for (int u = 0; u < n && !cx.status; ++u) {
-        const Op Qa_u{lay.Qa + (size_t)u * MQ * D * e, D, (int64_t)b1 * D}, dOa_u{lay.dOa + (size_t)u * MQ * D * e, D, (int64_t)b1 * D};
         const Op Kbar_u{lay.Kbar + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D};
-        const Op dKbar_u{lay.dKbar + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D}, dY_u{lay.dY + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D};
-        const Op L_u{lay.L + (size_t)u * AJ * b1 * RR * e, RR, (int64_t)b1 * RR}, dS2_u{lay.dS2 + (size_t)u * AJ * b1 * RR * e, RR, (int64_t)b1 * RR};
+        const Op dS2_u{lay.dS2 + (size_t)u * AJ * b1 * RR * e, RR, (int64_t)b1 * RR};
         const Op dQa_u{lay.dQa + (size_t)u * MQ * D * 4, D, (int64_t)b1 * D};
-        gemm(cx, true, false, RR, D, b1, 1.f, 0.f, L_u, dOa_u, dY_u, tE, tE, AJ);
-        gemm(cx, true, false, RR, D, b1, s, 0.f, dS2_u, Qa_u, dKbar_u, tE, tE, AJ);
         gemm(cx, false, false, b1, D, RR, s, 0.f, dS2_u, Kbar_u, dQa_u, tE, tF, AJ);
     }
     // 9. dR block = dKbar block . K block^T + dY block . V block^T per t
     gemm(cx, false, true, AJ, b2, D, 1.f, 0.f, dKbar_t, Kk_t, dRb_t, tE, tF, nt);
     gemm(cx, false, true, AJ, b2, D, 1.f, 1.f, dY_t, Vk_t, dRb_t, tE, tF, nt);
-    hipLaunchKernelGGL((softmax_right_bwd<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const float*)(ws + lay.S1f),
-                       (const float*)(ws + lay.dRb), (const float*)(ws + lay.dc), (T*)(ws + lay.dS1), b1, AJ, nf, b2, s, nseg);
+    if (fused_fwd)
+        hipLaunchKernelGGL((softmax_right_bwd_r<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const T*)(ws + lay.Rb),
+                           (const float*)(ws + lay.dRb), (const float*)(ws + lay.dc), (T*)(ws + lay.dS1), b1, AJ, nf, b2, nseg);
+    else
+        hipLaunchKernelGGL((softmax_right_bwd<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const float*)(ws + lay.S1f),
+                           (const float*)(ws + lay.dRb), (const float*)(ws + lay.dc), (T*)(ws + lay.dS1), b1, AJ, nf, b2, s, nseg);
     // 10. dQ (right factor) = s dS1 K per (u, k);  11. dK = s dS1^T q per (u, k)
     gemm(cx, false, false, AJ, D, NL, s, 0.f, dS1_uk, Kk_uk, dQk_uk, tE, tF, nuk);
     gemm(cx, true, false, NL, D, AJ, s, 0.f, dS1_uk, Qk_uk, dKk_uk, tE, tF, nuk);

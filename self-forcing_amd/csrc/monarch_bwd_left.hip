@@ -1,0 +1,296 @@
+// Left-factor part of the Monarch backward on gfx950 MFMA (bf16 / fp16, head_dim 64 or 128, block rows b1 <= 32).
+//
+// Replaces, inside the backward of the two-step attention, the per-(a, j) products and row kernels
+//     S2 = q_i . Kbar_r,  dLm = dO_i . Y_r,  L = softmax_r(s S2 - c),  dS2 = L (dLm - sum_r L dLm),
+//     dc_r = - sum_i dS2,  dY_r = sum_i L dO_i,  dKbar_r = s sum_i dS2 q_i
+// (wan/modules/monarch_attn.py:852-886 `_z_bwd_preprocess`, :1034-1222 `_z_bwd`) with one kernel that never writes
+// the [i x r] matrices S2, dLm, L.  dS2 is still written (16 bit) because the product dQ = s dS2 Kbar contracts over
+// r and stays a batched library GEMM.
+//
+// One wave per (unit, a, j); its b1 query rows and their dO rows sit in LDS, the r = (k, f) rows of Kbar and Y stream
+// from global memory 32 at a time, twice: pass 1 for the softmax statistics (row maximum, sum, and sum of L dLm, kept
+// per lane and merged across lanes once at the end), pass 2 for the gradients.  Logits are computed as
+// S2[i, r] (A = query rows, B = Kbar rows), so that a lane owns one r and holds 16 of the i: the accumulator layout
+// is then directly the B operand [n = r, k = i] of dY^T = dO^T L and dKbar^T = s Q^T dS2, whose A operands are
+// transposing LDS reads of the dO / Q rows, and dc is an in-lane sum.
+
+#include <hip/hip_runtime.h>
+
+#include "sfm_attn.h"
+#include "sfm_common.hpp"
+
+namespace sfm {
+namespace {
+
+struct LeftArgs {
+    const uint16_t* qa;      // [u][aj][b1][D]
+    const uint16_t* doa;     // [u][aj][b1][D]
+    const uint16_t* kbar;    // row r of (u, aj) at ((u * RR + r) * AJ + aj) * D
+    const uint16_t* y;
+    const float* c;          // c_rows == 0: [u][aj][RR], natural log units; c_rows == 1: [(u * RR + r) * AJ + aj], log2 units
+    int c_rows;
+    uint16_t* dkbar;         // like kbar
+    uint16_t* dy;
+    float* dc;               // [u][aj][RR]
+    uint16_t* ds2;           // [u][aj][b1][RR]
+    int b1, b2, AJ, nf, RR, causal;
+    float scale;
+};
+
+typedef short bl_s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2 bl_read_tr(const char* lds, uint32_t off) {
+    bl_s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((bl_s16x4 __attribute__((address_space(3)))*)(lds + off));
+    return __builtin_bit_cast(u32x2, v);
+}
+
+template <class E, int D>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void monarch_bwd_left_kernel(LeftArgs p) {
+    constexpr int DS = D / 16, DT = D / 32;
+    constexpr int kPitch = (D + 8) * 2;                   // bytes per staged row
+    constexpr int kPerWave = 2 * 32 * kPitch;             // q rows, then dO rows
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, m = lane & 31, hf = lane >> 5;
+    const int ajraw = blockIdx.x * 4 + wave;
+    const bool aj_ok = ajraw < p.AJ;
+    const int aj = aj_ok ? ajraw : p.AJ - 1;              // a wave past the end repeats the last column and stores nothing
+    const int u = blockIdx.y;
+    const int RR = p.RR, b1 = p.b1;
+    const int64_t uaj = (int64_t)u * p.AJ + aj;
+
+    char* qs = lds + wave * kPerWave;
+    char* dos = qs + 32 * kPitch;
+    {
+        const uint16_t* qg = p.qa + uaj * b1 * D;
+        const uint16_t* dg = p.doa + uaj * b1 * D;
+        constexpr int CH = D / 8;
+        for (int cidx = lane; cidx < 32 * CH; cidx += 64) {
+            const int r = cidx / CH, ch = cidx % CH;
+            u32x4 a = {0u, 0u, 0u, 0u}, b = a;
+            if (r < b1) {
+                a = *(const u32x4*)(qg + r * D + ch * 8);
+                b = *(const u32x4*)(dg + r * D + ch * 8);
+            }
+            *(u32x4*)(qs + r * kPitch + ch * 16) = a;
+            *(u32x4*)(dos + r * kPitch + ch * 16) = b;
+        }
+    }
+    __syncthreads();
+
+    const int a_blk = aj / p.b2;
+    const int flim = p.causal ? min(p.nf, (a_blk / p.causal + 1) * p.causal) : p.nf;      // visible kv block-frames
+    const int64_t rstride = (int64_t)p.AJ * D;                                           // elements between rows r, r + 1
+    const uint16_t* kb = p.kbar + ((int64_t)u * RR * p.AJ + aj) * D;
+    const uint16_t* yb = p.y + ((int64_t)u * RR * p.AJ + aj) * D;
+    const float* cp = p.c_rows ? p.c + (int64_t)u * RR * p.AJ + aj : p.c + uaj * RR;
+    const int64_t cstep = p.c_rows ? p.AJ : 1;
+    const float cmul = p.c_rows ? 1.f : kLog2e;
+    const float sc2 = p.scale * kLog2e;
+    const int nch = (RR + 31) / 32;
+
+    u32x4 kcur[DS], ycur[DS];
+    float ccur = 0.f;
+    auto load_tile = [&](int n) {
+        const int r = min(32 * n + m, RR - 1);
+        const uint16_t* kr = kb + (int64_t)r * rstride + 8 * hf;
+        const uint16_t* yr = yb + (int64_t)r * rstride + 8 * hf;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            kcur[ds] = *(const u32x4*)(kr + 16 * ds);
+            ycur[ds] = *(const u32x4*)(yr + 16 * ds);
+        }
+        ccur = cp[(int64_t)r * cstep] * cmul;
+    };
+    // logits S2[i, r] and dLm[i, r]: lane -> r = 32 n + m, register v -> i = 8 (v >> 2) + 4 hf + (v & 3)
+    auto products = [&](f32x16& s, f32x16& d) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = d[v] = 0.f;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            const u32x4 qb = *(const u32x4*)(qs + m * kPitch + (16 * ds + 8 * hf) * 2);
+            const u32x4 db = *(const u32x4*)(dos + m * kPitch + (16 * ds + 8 * hf) * 2);
+            s = E::mfma32(qb, kcur[ds], s);
+            d = E::mfma32(db, ycur[ds], d);
+        }
+    };
+    auto row_ok = [&](int n) {
+        const int r = 32 * n + m;
+        return r < RR && (r % p.nf) < flim;
+    };
+
+    // ---- pass 1: per lane, for its 16 rows i, the running maximum, sum and sum of L dLm over the lane's own r
+    float mloc[16], lloc[16], dloc[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        mloc[v] = -INFINITY;
+        lloc[v] = dloc[v] = 0.f;
+    }
+    load_tile(0);
+    for (int n = 0; n < nch; ++n) {
+        f32x16 s, d;
+        products(s, d);
+        const float cl2 = ccur;
+        const bool ok = row_ok(n);
+        load_tile(min(n + 1, nch - 1));
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float z = ok ? s[v] * sc2 - cl2 : -INFINITY;
+            const float mnew = fmaxf(mloc[v], z);
+            const float mref = mnew == -INFINITY ? 0.f : mnew;
+            const float alpha = fast_exp2(mloc[v] - mref), e = fast_exp2(z - mref);
+            lloc[v] = lloc[v] * alpha + e;
+            dloc[v] = dloc[v] * alpha + e * d[v];
+            mloc[v] = mnew;
+        }
+    }
+    // merge over the 32 lanes of a half (they hold the same rows i); every row has at least one visible r
+    float lse[16], delta[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        float mm = mloc[v], ll = lloc[v], dd = dloc[v];
+#pragma unroll
+        for (int o = 1; o < 32; o <<= 1) {
+            const float m2 = __shfl_xor(mm, o), l2 = __shfl_xor(ll, o), d2 = __shfl_xor(dd, o);
+            const float mnew = fmaxf(mm, m2);
+            const float mref = mnew == -INFINITY ? 0.f : mnew;
+            const float a1 = fast_exp2(mm - mref), a2 = fast_exp2(m2 - mref);
+            ll = ll * a1 + l2 * a2;
+            dd = dd * a1 + d2 * a2;
+            mm = mnew;
+        }
+        lse[v] = mm + log2f(ll);
+        delta[v] = dd / ll;
+    }
+
+    // ---- pass 2: gradients
+    // transposing reads of the staged rows: lane (m, hf) gets, for head-dim column 32 dt + m, rows i = 16 ks + 4 hf +
+    // {0..3} and + 8 + {0..3}, the order in which the packed accumulators hold i (two reads, see perm_row)
+    uint32_t tr0, tr1;
+    {
+        const int s16 = lane & 15, g16 = lane >> 4;
+        const int rl = 4 * hf + (s16 >> 2);
+        const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
+        tr0 = (uint32_t)(rl * kPitch + cl * 16 + (s16 & 1) * 8);
+        tr1 = tr0 + 8 * kPitch;
+    }
+    uint16_t* const dkb = p.dkbar + ((int64_t)u * RR * p.AJ + aj) * D;
+    uint16_t* const dyb = p.dy + ((int64_t)u * RR * p.AJ + aj) * D;
+    float* const dcp = p.dc + uaj * RR;
+    uint16_t* const ds2p = p.ds2 + uaj * b1 * RR;
+
+    load_tile(0);
+    for (int n = 0; n < nch; ++n) {
+        f32x16 s, d;
+        products(s, d);
+        const float cl2 = ccur;
+        const bool ok = row_ok(n);
+        const int r = 32 * n + m;
+        const bool r_in = r < RR;
+        load_tile(min(n + 1, nch - 1));
+        float dsum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float pv = ok ? fast_exp2(s[v] * sc2 - cl2 - lse[v]) : 0.f;
+            const float gv = pv * (d[v] - delta[v]);
+            s[v] = pv;                                   // L[i, r]
+            d[v] = gv;                                   // dS2[i, r]
+            dsum += gv;
+        }
+        dsum = xhalf_sum(dsum);
+        if (aj_ok && r_in && hf == 0) dcp[r] = -dsum;
+        if (aj_ok && r_in) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
+                if (i < b1) ds2p[(int64_t)i * RR + r] = E::from_float(d[v]);
+            }
+        }
+        u32x4 pl[2], pg[2];                              // B operands [n = r, k = i] for the two steps of 16 rows i
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            pl[ks].x = pack2<E>(s[8 * ks + 0], s[8 * ks + 1]); pl[ks].y = pack2<E>(s[8 * ks + 2], s[8 * ks + 3]);
+            pl[ks].z = pack2<E>(s[8 * ks + 4], s[8 * ks + 5]); pl[ks].w = pack2<E>(s[8 * ks + 6], s[8 * ks + 7]);
+            pg[ks].x = pack2<E>(d[8 * ks + 0], d[8 * ks + 1]); pg[ks].y = pack2<E>(d[8 * ks + 2], d[8 * ks + 3]);
+            pg[ks].z = pack2<E>(d[8 * ks + 4], d[8 * ks + 5]); pg[ks].w = pack2<E>(d[8 * ks + 6], d[8 * ks + 7]);
+        }
+        // dY^T[d, r] = sum_i dO^T[d, i] L[i, r],  dKbar^T[d, r] = s sum_i Q^T[d, i] dS2[i, r], 32 head-dim rows at a time
+#pragma unroll
+        for (int which = 0; which < 2; ++which) {
+            const char* src = which == 0 ? dos : qs;
+            uint16_t* const orow = (which == 0 ? dyb : dkb) + (int64_t)min(r, RR - 1) * rstride;
+            const float osc = which == 0 ? 1.f : p.scale;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                f32x16 o;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o[v] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    const u32x2 lo = bl_read_tr(src, tr0 + ks * 16 * kPitch + dt * 64);
+                    const u32x2 hi = bl_read_tr(src, tr1 + ks * 16 * kPitch + dt * 64);
+                    const u32x4 aop = {lo.x, lo.y, hi.x, hi.y};
+                    o = E::mfma32(aop, which == 0 ? pl[ks] : pg[ks], o);
+                }
+                // lane (r, hf) holds head-dim 32 dt + 8 g + 4 hf + 0..3; the half-swap leaves 8 consecutive ones per lane
+#pragma unroll
+                for (int gp = 0; gp < 2; ++gp) {
+                    const int g0 = 2 * gp, g1 = 2 * gp + 1;
+                    auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(o[4 * g0 + 0] * osc, o[4 * g0 + 1] * osc),
+                                                               pack2<E>(o[4 * g1 + 0] * osc, o[4 * g1 + 1] * osc), false, false);
+                    auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(o[4 * g0 + 2] * osc, o[4 * g0 + 3] * osc),
+                                                               pack2<E>(o[4 * g1 + 2] * osc, o[4 * g1 + 3] * osc), false, false);
+                    const u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+                    if (aj_ok && r_in) *(u32x4*)(orow + 32 * dt + 16 * gp + 8 * hf) = w;
+                }
+            }
+        }
+    }
+}
+
+}  // namespace
+
+bool monarch_bwd_left_supported(int dtype, int D, int b1) {
+    return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b1 >= 1 && b1 <= 32;
+}
+
+int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* qa,
+                            const void* doa, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy,
+                            float* dc, void* ds2, hipStream_t stream) {
+    LeftArgs a;
+    a.c_rows = c_rows;
+    a.qa = (const uint16_t*)qa; a.doa = (const uint16_t*)doa;
+    a.kbar = (const uint16_t*)kbar; a.y = (const uint16_t*)y;
+    a.c = c;
+    a.dkbar = (uint16_t*)dkbar; a.dy = (uint16_t*)dy;
+    a.dc = dc;
+    a.ds2 = (uint16_t*)ds2;
+    a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.nf = nf; a.RR = nf * b1; a.causal = causal;
+    a.scale = scale;
+    const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n);
+    const size_t ldsb = (size_t)4 * 2 * 32 * (D + 8) * 2;
+    const void* fn = nullptr;
+    if (dtype == SFM_BF16) fn = D == 128 ? (const void*)monarch_bwd_left_kernel<BF16, 128> : (const void*)monarch_bwd_left_kernel<BF16, 64>;
+    else fn = D == 128 ? (const void*)monarch_bwd_left_kernel<F16, 128> : (const void*)monarch_bwd_left_kernel<F16, 64>;
+    if (ldsb > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsb);
+        if (e != hipSuccess) {
+            set_error("monarch backward (left factor): cannot reserve %zu bytes of LDS: %s", ldsb, hipGetErrorString(e));
+            return SFM_ERR_HIP;
+        }
+    }
+    if (dtype == SFM_BF16) {
+        if (D == 128) hipLaunchKernelGGL((monarch_bwd_left_kernel<BF16, 128>), grid, dim3(256), ldsb, stream, a);
+        else hipLaunchKernelGGL((monarch_bwd_left_kernel<BF16, 64>), grid, dim3(256), ldsb, stream, a);
+    } else {
+        if (D == 128) hipLaunchKernelGGL((monarch_bwd_left_kernel<F16, 128>), grid, dim3(256), ldsb, stream, a);
+        else hipLaunchKernelGGL((monarch_bwd_left_kernel<F16, 64>), grid, dim3(256), ldsb, stream, a);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("monarch backward (left factor): launch failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+}  // namespace sfm

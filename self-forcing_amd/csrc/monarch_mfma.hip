@@ -38,7 +38,8 @@ struct S1Lds {
     static __host__ __device__ constexpr size_t bytes() { return 2 * (size_t)kElems; }
 };
 
-template <class E, int D>
+// WR: also write the right factor R (16 bit, 64 values per scratch row) to p.rb; the backward uses it.
+template <class E, int D, bool WR = false>
 __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) void monarch_step1_kernel(MonarchArgs p) {
     using L = S1Lds<D>;
     constexpr int DS = D / 16;   // contraction steps of the logits
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int b2 = p.b2;
     const int NT = b2 > 32 ? 2 : 1;                       // 32-row tiles of the key axis l
     const uint32_t qs1 = (uint32_t)p.qs[1], ks1 = (uint32_t)p.ks[1];
-    const uint32_t fstep = (uint32_t)p.b1 * p.ws_row;     // scratch rows between consecutive f
+    const uint32_t fstep = p.ws_f ? p.ws_f : (uint32_t)p.b1 * p.ws_row;     // scratch rows between consecutive f
 
     struct Tile {
         int f, k, ul, a0, ncols;
@@ -288,6 +289,20 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             }
             // sum_l R log2 R (both halves of a column hold, and store, the same value)
             *(float*)((char*)p.cl + (size_t)srow * 4 + cloff) = ent * inv_l - (mx + log2f(sum));
+            if (WR) {
+                // R[l] for l = 16 st + 0..15: the lower half of the wave holds 0..3 and 8..11, the upper half 4..7 and
+                // 12..15; exchanging the lower half's second pair with the upper half's first leaves 8 consecutive values
+                char* rrow = (char*)p.rb + ((size_t)srow + cloff / 4) * 128 + 16 * hf;
+#pragma unroll
+                for (int st = 0; st < 4; ++st) {
+                    if (st < 2 * NT) {
+                        auto rx = __builtin_amdgcn_permlane32_swap(pb[st].x, pb[st].z, false, false);
+                        auto ry = __builtin_amdgcn_permlane32_swap(pb[st].y, pb[st].w, false, false);
+                        const u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+                        *(u32x4*)(rrow + 32 * st) = w;
+                    }
+                }
+            }
         }
         // contractions with K^T then V^T, 32 head-dim columns at a time.  A 32 x 32 accumulator tile holds,
         // per lane (column c, half hf), head-dim 8g + 4hf + 0..3 for g = 0..3; swapping the g-odd dwords of the
@@ -612,6 +627,46 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const 
         return SFM_ERR_HIP;
     }
     return SFM_OK;
+}
+
+template <class E, int D>
+static int launch_step1_t(const MonarchArgs& a, int nunits, hipStream_t stream) {
+    const int ncols = a.a_chunk * a.b2;
+    const int ntiles = (ncols + 31) / 32;
+    const int nwaves = ntiles < 4 ? 4 : ntiles;
+    if (ntiles < 1 || nwaves > 8 || (8 * (D / 2) + nwaves * 64 - 1) / (nwaves * 64) > 2) {
+        set_error("internal: step-1 launch shape (a_chunk=%d, b2=%d)", a.a_chunk, a.b2);
+        return SFM_ERR_UNSUPPORTED;
+    }
+    const int groups = nwaves <= 5 ? 2 : 1;
+    const size_t lds1 = S1Lds<D>::bytes() * groups;
+    const void* fn = a.rb ? (const void*)monarch_step1_kernel<E, D, true> : (const void*)monarch_step1_kernel<E, D, false>;
+    if (lds1 > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1);
+        if (e != hipSuccess) {
+            set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+            return SFM_ERR_HIP;
+        }
+    }
+    MonarchArgs a1 = a;
+    a1.s1_total = a.nf * a.b1 * nunits * a.n_achunks;
+    a1.s1_groups = groups;
+    int wgs = a.s1_wgs > 0 ? a.s1_wgs : cu_count();
+    if (wgs > (a1.s1_total + groups - 1) / groups) wgs = (a1.s1_total + groups - 1) / groups;
+    if (a.rb) hipLaunchKernelGGL((monarch_step1_kernel<E, D, true>), dim3(wgs), dim3(nwaves * 64 * groups), lds1, stream, a1);
+    else hipLaunchKernelGGL((monarch_step1_kernel<E, D, false>), dim3(wgs), dim3(nwaves * 64 * groups), lds1, stream, a1);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        set_error("hip launch failed: %s", hipGetErrorString(err));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream) {
+    if (dtype == SFM_BF16)
+        return a.D == 128 ? launch_step1_t<BF16, 128>(a, nunits, stream) : launch_step1_t<BF16, 64>(a, nunits, stream);
+    return a.D == 128 ? launch_step1_t<F16, 128>(a, nunits, stream) : launch_step1_t<F16, 64>(a, nunits, stream);
 }
 
 int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev) {

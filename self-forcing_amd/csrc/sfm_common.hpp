@@ -136,6 +136,8 @@ struct MonarchArgs {
     int r_pad;       // rows per (a, j) block of the workspace: round_up(nf*b1, 32)
     // scratch row index of (unit ul, a, j, r) = ul*ws_unit + (a*b2 + j)*ws_aj + r*ws_row
     uint32_t ws_unit, ws_aj, ws_row;
+    uint32_t ws_f;   // MFMA step 1 only: rows between consecutive kv block-frames f of one (unit, a, j, k); 0 = b1 * ws_row
+    void* rb;        // MFMA step 1 only, optional: the right factor R, 16 bit, 64 values per scratch row (same row index)
     int unit0;       // first (b*H + h) unit of this pass
     int causal;      // block-causal size in block-frames, 0 = none
     float scale;
@@ -178,6 +180,13 @@ int launch_monarch_bwd(const MonarchBwdArgs& g, int dtype, int nunits, hipStream
 bool monarch_bwd_gemm_available();
 size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits);
 int launch_monarch_bwd_gemm(const MonarchBwdArgs& g, int dtype, int nunits, void* workspace, hipStream_t stream);
+// step 1 of the MFMA forward alone, with the scratch strides of `a` and, if a.rb is set, the right factor written out
+int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream);
+// fused left-factor part of the backward (monarch_bwd_left.hip); operands in the GEMM path's scratch layouts
+bool monarch_bwd_left_supported(int dtype, int D, int b1);
+int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* qa,
+                            const void* doa, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy,
+                            float* dc, void* ds2, hipStream_t stream);
 
 void set_error(const char* fmt, ...);
 int cu_count();                                  // compute units of the current device (cached per thread)
