@@ -160,7 +160,7 @@ def op_level(torch, sfa, args):
                                      "(4680 q x 32760 kv), new chunk written at tokens 28080..32760",
                          "ms_per_call": ms_call, "tflops": tfl, "mfma_frac": tfl / MFMA_BF16_PEAK_TFLOPS,
                          "kernel_ms": {"monarch_step1": s1_ms, "monarch_step2": s2_ms}},
-        "monarch_bwd": {"workload": "gradients of q and of all 21 cached K/V frames at the same shape (fp32 kernels)",
+        "monarch_bwd": {"workload": "gradients of q and of all 21 cached K/V frames at the same shape",
                         "ms_per_call": bwd_ms},
         "dense_fallback": {"ms_per_call": dense_ms, "tflops": dense_tfl, "mfma_frac": dense_tfl / MFMA_BF16_PEAK_TFLOPS,
                            "mfma_probe_tflops": probe.value, "frac_of_probe": dense_tfl / probe.value},
