@@ -13,7 +13,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsfm_attn.so")
 SOURCES = ["sfm_api.hip", "monarch_mfma.hip", "monarch_generic.hip", "dense_attn.hip", "qk_prologue.hip", "block_fused.hip",
-           "monarch_bwd_gemm.hip", "monarch_bwd_left.hip", "probe.hip", "conv3d_cl.hip"]
+           "monarch_bwd_gemm.hip", "monarch_bwd_left.hip", "monarch_bwd_right.hip", "probe.hip", "conv3d_cl.hip"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -392,7 +392,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // Scratch of a pass over n units, in bytes (all sub-buffers 256-byte aligned).
 struct Layout {
-    size_t Qk, dOk, Qa, dOa, Kk, Vk, S1f, dRb, Rb, dS1, Kbar, Y, dKbar, dY, c, dc, S2f, dLmf, L, dS2, dQa, dQk, dKk, dVk, total;
+    size_t Qk, Qa, dOa, Kk, Vk, S1f, dRb, Rb, dS1, Kbar, Y, dKbar, dY, c, dc, S2f, dLmf, L, dS2, dQa, dQk, dKk, dVk, total;
 };
 
 Layout make_layout(const MonarchArgs& p, int n, size_t e) {
@@ -402,7 +402,6 @@ Layout make_layout(const MonarchArgs& p, int n, size_t e) {
     size_t o = 0;
     auto take = [&](size_t bytes) { size_t at = o; o += align256(bytes); return at; };
     l.Qk = take(n * MQ * D * e);
-    l.dOk = take(n * MQ * D * e);
     l.Qa = take(n * MQ * D * e);
     l.dOa = take(n * MQ * D * e);
     l.Kk = take(n * MK * D * e);
@@ -490,8 +489,6 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
                            na, H, D, p.unit0, 0, tq);
         hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.Qa), p.q, p.qs[0], p.qs[1], p.qs[2], p.qmap,
                            na, H, D, p.unit0, 1, tq);
-        hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.dOk), g.dout, g.dos[0], g.dos[1], g.dos[2],
-                           p.qmap, na, H, D, p.unit0, 0, tq);
         hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.dOa), g.dout, g.dos[0], g.dos[1], g.dos[2],
                            p.qmap, na, H, D, p.unit0, 1, tq);
         hipLaunchKernelGGL((gather_rows<E>), dim3(gk), dim3(256), 0, stream, (T*)(ws + lay.Kk), p.k, p.ks[0], p.ks[1], p.ks[2], p.kmap,
@@ -578,21 +575,34 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
         const Op dQa_u{lay.dQa + (size_t)u * MQ * D * 4, D, (int64_t)b1 * D};
         gemm(cx, false, false, b1, D, RR, s, 0.f, dS2_u, Kbar_u, dQa_u, tE, tF, AJ);
     }
-    // 9. dR block = dKbar block . K block^T + dY block . V block^T per t
-    gemm(cx, false, true, AJ, b2, D, 1.f, 0.f, dKbar_t, Kk_t, dRb_t, tE, tF, nt);
-    gemm(cx, false, true, AJ, b2, D, 1.f, 1.f, dY_t, Vk_t, dRb_t, tE, tF, nt);
-    if (fused_fwd)
+    // 9, the right factor's softmax backward, 12 and 13 in one kernel per tile t
+    const bool fused_right = fused_fwd && monarch_bwd_right_supported(left_dtype<E>(), D, b2, AJ) && getenv("SFM_BWD_RIGHT_GEMM") == nullptr;
+    if (fused_right) {
+        if (!cx.status)
+            cx.status = launch_monarch_bwd_right(left_dtype<E>(), D, nt, b1, b2, AJ, nf, ws + lay.Kk, ws + lay.Vk, ws + lay.Rb, ws + lay.dKbar,
+                                                 ws + lay.dY, (const float*)(ws + lay.dc), ws + lay.dS1, (float*)(ws + lay.dKk),
+                                                 (float*)(ws + lay.dVk), stream);
+    } else {
+        // 9. dR block = dKbar block . K block^T + dY block . V block^T per t
+        gemm(cx, false, true, AJ, b2, D, 1.f, 0.f, dKbar_t, Kk_t, dRb_t, tE, tF, nt);
+        gemm(cx, false, true, AJ, b2, D, 1.f, 1.f, dY_t, Vk_t, dRb_t, tE, tF, nt);
+    }
+    if (fused_right) {
+        // dS1 is already written
+    } else if (fused_fwd)
         hipLaunchKernelGGL((softmax_right_bwd_r<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const T*)(ws + lay.Rb),
                            (const float*)(ws + lay.dRb), (const float*)(ws + lay.dc), (T*)(ws + lay.dS1), b1, AJ, nf, b2, nseg);
     else
         hipLaunchKernelGGL((softmax_right_bwd<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const float*)(ws + lay.S1f),
                            (const float*)(ws + lay.dRb), (const float*)(ws + lay.dc), (T*)(ws + lay.dS1), b1, AJ, nf, b2, s, nseg);
-    // 10. dQ (right factor) = s dS1 K per (u, k);  11. dK = s dS1^T q per (u, k)
+    // 10. dQ (right factor) = s dS1 K per (u, k);  11. dK (+)= s dS1^T q per (u, k)
     gemm(cx, false, false, AJ, D, NL, s, 0.f, dS1_uk, Kk_uk, dQk_uk, tE, tF, nuk);
-    gemm(cx, true, false, NL, D, AJ, s, 0.f, dS1_uk, Qk_uk, dKk_uk, tE, tF, nuk);
-    // 12. dK block += R block^T dKbar block;  13. dV block = R block^T dY block per t
-    gemm(cx, true, false, b2, D, AJ, 1.f, 1.f, Rb_t, dKbar_t, dKk_t, tE, tF, nt);
-    gemm(cx, true, false, b2, D, AJ, 1.f, 0.f, Rb_t, dY_t, dVk_t, tE, tF, nt);
+    gemm(cx, true, false, NL, D, AJ, s, fused_right ? 1.f : 0.f, dS1_uk, Qk_uk, dKk_uk, tE, tF, nuk);
+    if (!fused_right) {
+        // 12. dK block += R block^T dKbar block;  13. dV block = R block^T dY block per t
+        gemm(cx, true, false, b2, D, AJ, 1.f, 1.f, Rb_t, dKbar_t, dKk_t, tE, tF, nt);
+        gemm(cx, true, false, b2, D, AJ, 1.f, 0.f, Rb_t, dY_t, dVk_t, tE, tF, nt);
+    }
     if (cx.status) return cx.status;
     // scatter the gradients back to the callers' layouts
     {

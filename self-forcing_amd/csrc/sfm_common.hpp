@@ -187,6 +187,11 @@ bool monarch_bwd_left_supported(int dtype, int D, int b1);
 int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* qa,
                             const void* doa, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy,
                             float* dc, void* ds2, hipStream_t stream);
+// fused right-factor part of the backward (monarch_bwd_right.hip): dS1, dK and dV blocks of every tile t = (unit, k, f)
+bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ);
+int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, const void* kk, const void* vk,
+                             const void* rb, const void* dkbar, const void* dy, const float* dc, void* ds1, float* dkk, float* dvk,
+                             hipStream_t stream);
 
 void set_error(const char* fmt, ...);
 int cu_count();                                  // compute units of the current device (cached per thread)

@@ -127,6 +127,26 @@ def test_480p_block_shape_bf16_one_head(bwd_path):
     _close(vd.grad, vr.grad, torch.bfloat16)
 
 
+@pytest.mark.parametrize("h,w,Fq,Fk,D,causal,dtype", [
+    (4, 52, 3, 3, 128, True, torch.bfloat16),      # 156 (a, j) columns: every fused kernel, last column block partial
+    (4, 52, 3, 5, 64, False, torch.float16),
+    (4, 52, 4, 4, 64, True, torch.bfloat16),       # 208 columns: the right factor's blocks stay on the library products
+    (5, 6, 2, 3, 64, False, torch.bfloat16),       # b2 = 6, not a multiple of 4: likewise
+])
+def test_16bit_gradients_across_the_fused_kernels_limits(h, w, Fq, Fk, D, causal, dtype):
+    H = 2
+    q0, do = (randn((1, Fq * h * w, H, D), 150 + i, dtype) for i in range(2))
+    k0, v0 = (randn((1, Fk * h * w, H, D), 152 + i, dtype) for i in range(2))
+    kw = {"block_causal_size": h * w} if causal else {}
+    qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
+    monarch.monarch_attn(qr, kr, vr, 1, 1, 1, h, w, **kw).backward(do.double())
+    qd, kd, vd = _leaf(q0, DEV), _leaf(k0, DEV), _leaf(v0, DEV)
+    mattn.monarch_attn(qd, kd, vd, 1, 1, 1, h, w, **kw).backward(do.to(DEV))
+    _close(qd.grad, qr.grad, dtype)
+    _close(kd.grad, kr.grad, dtype)
+    _close(vd.grad, vr.grad, dtype)
+
+
 def test_descriptor_errors():
     q = randn((1, 64, 1, 32), 140, torch.float32).to(DEV).requires_grad_(True)
     with pytest.raises(NotImplementedError):
