@@ -419,7 +419,7 @@ Layout make_layout(const MonarchArgs& p, int n, size_t e) {
     l.S2f = take(n * AJ * p.b1 * RR * 4);
     l.dLmf = take(n * AJ * p.b1 * RR * 4);
     l.L = take(n * AJ * p.b1 * RR * e);
-    l.dS2 = take(n * AJ * p.b1 * RR * e);
+    l.dS2 = take(n * AJ * p.b1 * ((RR + 7) / 8 * 8) * e);                          // rows padded to 8 for the fused kernels
     l.dQa = take(n * MQ * D * 4);
     l.dQk = take(n * MQ * D * 4);
     l.dKk = take(n * MK * D * 4);
@@ -512,6 +512,9 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     const bool fused_left = left_dtype<E>() >= 0 && monarch_bwd_left_supported(left_dtype<E>(), D, b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
     // the forward's MFMA step 1 recomputes Kbar, Y, c and R straight into this scratch ([t][aj] rows)
     const bool fused_fwd = fused_left && monarch_mfma_supported(left_dtype<E>(), D, b2) && getenv("SFM_BWD_FWD_GEMM") == nullptr;
+    // dQ of the left factor in its own kernel, which also adds the right factor's part and writes the caller's dq
+    const bool fused_dqa = fused_left && getenv("SFM_BWD_DQA_GEMM") == nullptr;
+    const int ds2_ld = fused_left ? (RR + 7) / 8 * 8 : RR;
     const int rb_ld = fused_fwd ? 64 : b2;
     const Op Rb_t{lay.Rb, rb_ld, (int64_t)AJ * rb_ld};
     if (fused_fwd) {
@@ -539,7 +542,7 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
         if (!cx.status)
             cx.status = launch_monarch_bwd_left(left_dtype<E>(), D, n, b1, b2, AJ, nf, p.causal, s, ws + lay.Qa, ws + lay.dOa, ws + lay.Kbar,
                                                 ws + lay.Y, (const float*)(ws + lay.c), fused_fwd ? 1 : 0, ws + lay.dKbar, ws + lay.dY,
-                                                (float*)(ws + lay.dc), ws + lay.dS2, stream);
+                                                (float*)(ws + lay.dc), ws + lay.dS2, ds2_ld, stream);
     } else {
         // 4, 5. per unit and (a, j): S2 = q_i . Kbar_r, dLm = dO_i . Y_r; the [RR x D] matrix of column aj is every AJ-th row
         for (int u = 0; u < n && !cx.status; ++u) {
@@ -569,9 +572,9 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
         }
     }
     // 8. per unit and (a, j): dQ (left factor) = s dS2 Kbar
-    for (int u = 0; u < n && !cx.status; ++u) {
+    for (int u = 0; u < n && !cx.status && !fused_dqa; ++u) {
         const Op Kbar_u{lay.Kbar + (size_t)u * AJ * RR * D * e, (int64_t)AJ * D, D};
-        const Op dS2_u{lay.dS2 + (size_t)u * AJ * b1 * RR * e, RR, (int64_t)b1 * RR};
+        const Op dS2_u{lay.dS2 + (size_t)u * AJ * b1 * ds2_ld * e, ds2_ld, (int64_t)b1 * ds2_ld};
         const Op dQa_u{lay.dQa + (size_t)u * MQ * D * 4, D, (int64_t)b1 * D};
         gemm(cx, false, false, b1, D, RR, s, 0.f, dS2_u, Kbar_u, dQa_u, tE, tF, AJ);
     }
@@ -607,12 +610,17 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     // scatter the gradients back to the callers' layouts
     {
         const int64_t tq = (int64_t)n * MQ * (D / 4);
-        hipLaunchKernelGGL(scatter_dq, dim3((unsigned)((tq + 255) / 256)), dim3(256), 0, stream, (const float*)(ws + lay.dQa),
-                           (const float*)(ws + lay.dQk), g.dq, g.dqs[0], g.dqs[1], g.dqs[2], p.qmap, na, H, D, p.unit0, tq);
+        if (fused_dqa)
+            cx.status = launch_monarch_bwd_dqa(left_dtype<E>(), D, n, b1, b2, AJ, nf, s, ws + lay.Kbar, ws + lay.dS2, ds2_ld,
+                                               (const float*)(ws + lay.dQk), g.dq, g.dqs, p.qmap, H, p.unit0, stream);
+        else
+            hipLaunchKernelGGL(scatter_dq, dim3((unsigned)((tq + 255) / 256)), dim3(256), 0, stream, (const float*)(ws + lay.dQa),
+                               (const float*)(ws + lay.dQk), g.dq, g.dqs[0], g.dqs[1], g.dqs[2], p.qmap, na, H, D, p.unit0, tq);
         const int64_t tk = (int64_t)n * b1 * (g.kv_f1 - g.kv_f0) * b2 * (D / 4);
         hipLaunchKernelGGL((scatter_dkv<E>), dim3((unsigned)((tk + 255) / 256)), dim3(256), 0, stream, (const float*)(ws + lay.dKk),
                            (const float*)(ws + lay.dVk), (T*)g.dk, (T*)g.dv, g.dks[0], g.dks[1], g.dks[2], p.kmap, nf, g.kv_f0, g.kv_f1,
                            g.dk_row0, H, D, p.unit0, tk);
+        if (cx.status) return cx.status;
     }
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) {

@@ -32,7 +32,8 @@ struct LeftArgs {
     uint16_t* dkbar;         // like kbar
     uint16_t* dy;
     float* dc;               // [u][aj][RR]
-    uint16_t* ds2;           // [u][aj][b1][RR]
+    uint16_t* ds2;           // [u][aj][b1][ds2_ld], ds2_ld >= RR
+    int ds2_ld;
     int b1, b2, AJ, nf, RR, causal;
     float scale;
 };
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     uint16_t* const dkb = p.dkbar + ((int64_t)u * RR * p.AJ + aj) * D;
     uint16_t* const dyb = p.dy + ((int64_t)u * RR * p.AJ + aj) * D;
     float* const dcp = p.dc + uaj * RR;
-    uint16_t* const ds2p = p.ds2 + uaj * b1 * RR;
+    uint16_t* const ds2p = p.ds2 + uaj * b1 * p.ds2_ld;
 
     load_tile(0);
     for (int n = 0; n < nch; ++n) {
@@ -202,7 +203,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
-                if (i < b1) ds2p[(int64_t)i * RR + r] = E::from_float(d[v]);
+                if (i < b1) ds2p[(int64_t)i * p.ds2_ld + r] = E::from_float(d[v]);
             }
         }
         u32x4 pl[2], pg[2];                              // B operands [n = r, k = i] for the two steps of 16 rows i
@@ -247,6 +248,151 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// dQ of the left factor, dQ[i, :] = s sum_r dS2[i, r] Kbar[r, :] per (unit, a, j), plus the right factor's part
+// (already reduced per (unit, k) by a library GEMM), written straight to the caller's dq rows.
+// One wave per (unit, a, j): its Kbar rows go through LDS 32 at a time (global_load_lds_dwordx4, double buffered,
+// 16-byte chunks XOR-swizzled per row) and come back as the B operand [n = d, k = r] through transposing reads; the
+// A operand [m = i, k = r] is dS2 straight from memory, two 8-byte pieces per step in the order in which the
+// transposing reads deliver r.
+struct DqaArgs {
+    const char* kbar;        // row r of (u, aj) at ((u * RR + r) * AJ + aj) * D elements
+    const uint16_t* ds2;     // [u][aj][b1][ds2_ld], ds2_ld a multiple of 4
+    const float* dqk;        // [u][i][aj][D]
+    float* dq;               // caller's tensor, strides s0 (batch), s1 (token), s2 (head)
+    int64_t s0, s1, s2;
+    TokMap map;
+    int ds2_ld, b1, b2, AJ, RR, H, unit0;
+    float scale;
+};
+
+template <int CPR>
+__device__ __forceinline__ int bl_swz(int r) {
+    return CPR >= 16 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
+}
+__device__ __forceinline__ void bl_load_lds16(const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
+}
+
+template <class E, int D>
+__global__ __launch_bounds__(256) void monarch_bwd_dqa_kernel(DqaArgs p) {
+    constexpr int DT = D / 32, CPR = D / 8;
+    constexpr int kPitch = 2 * D;
+    constexpr int kTile = 32 * kPitch;
+    constexpr int kInstr = 32 * CPR / 64;                 // 64-lane loads per tile
+    extern __shared__ __attribute__((aligned(256))) char lds[];
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
+
+    const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ajraw = blockIdx.x * 4 + wave;
+    const bool aj_ok = ajraw < p.AJ;
+    const int aj = aj_ok ? ajraw : p.AJ - 1;              // a wave past the end repeats the last column and stores nothing
+    const int u = blockIdx.y;
+    const int RR = p.RR, b1 = p.b1;
+    const int64_t uaj = (int64_t)u * p.AJ + aj;
+    const int nch = (RR + 31) / 32;
+    const uint32_t rstride = (uint32_t)p.AJ * kPitch;     // bytes between rows r, r + 1
+    const char* kb = p.kbar + ((int64_t)u * RR * p.AJ + aj) * kPitch;
+    const uint32_t buf0 = lds0 + (uint32_t)wave * 2 * kTile;
+    const char* mine = lds + wave * 2 * kTile;
+
+    // LDS position P (16-byte units) of a tile holds chunk (P % CPR) ^ swz(row) of row P / CPR
+    auto stage = [&](int n) {
+#pragma unroll
+        for (int q = 0; q < kInstr; ++q) {
+            const int P = 64 * q + lane;
+            const int row = P / CPR, c = (P % CPR) ^ bl_swz<CPR>(row);
+            const int r = min(32 * n + row, RR - 1);
+            bl_load_lds16(kb, (uint32_t)r * rstride + (uint32_t)c * 16, buf0 + (uint32_t)(n & 1) * kTile + (uint32_t)q * 1024);
+        }
+    };
+    // dS2 pieces of row i = m: r = 32 n + 16 ks + 4 hf + {0..3} and + 8 + {0..3}
+    const uint16_t* arow = p.ds2 + (uaj * b1 + min(m, b1 - 1)) * p.ds2_ld + 4 * hf;
+    u32x4 acur[2], anext[2];
+    auto load_a = [&](int n, u32x4 (&a)[2]) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int r0 = 32 * n + 16 * ks + 4 * hf;
+            u32x2 lo = {0u, 0u}, hi = {0u, 0u};
+            if (r0 + 4 <= RR) lo = *(const u32x2*)(arow + 32 * n + 16 * ks);
+            else
+                for (int e2 = 0; e2 < 4; ++e2)
+                    if (r0 + e2 < RR) {
+                        const uint32_t x = arow[32 * n + 16 * ks + e2];
+                        if (e2 < 2) lo.x |= x << (16 * e2); else lo.y |= x << (16 * (e2 - 2));
+                    }
+            if (r0 + 12 <= RR) hi = *(const u32x2*)(arow + 32 * n + 16 * ks + 8);
+            else
+                for (int e2 = 0; e2 < 4; ++e2)
+                    if (r0 + 8 + e2 < RR) {
+                        const uint32_t x = arow[32 * n + 16 * ks + 8 + e2];
+                        if (e2 < 2) hi.x |= x << (16 * e2); else hi.y |= x << (16 * (e2 - 2));
+                    }
+            a[ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
+    };
+
+    uint32_t tr[DT][2];
+    {
+        const int s16 = lane & 15, g16 = lane >> 4;
+        const int rl = 4 * hf + (s16 >> 2);
+        const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int r = rl + 8 * half;             // swz depends on r mod 16 only
+                tr[dt][half] = (uint32_t)(r * kPitch + (((4 * dt + cl) ^ bl_swz<CPR>(r)) << 4) + (s16 & 1) * 8);
+            }
+    }
+
+    f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
+
+    stage(0);
+    load_a(0, acur);
+    for (int n = 0; n < nch; ++n) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");          // tile n and its dS2 pieces have landed
+        if (n + 1 < nch) {
+            stage(n + 1);
+            load_a(n + 1, anext);
+        }
+        const char* tile = mine + (n & 1) * kTile;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const u32x2 lo = bl_read_tr(tile, tr[dt][0] + ks * 16 * kPitch);
+                const u32x2 hi = bl_read_tr(tile, tr[dt][1] + ks * 16 * kPitch);
+                const u32x4 bop = {lo.x, lo.y, hi.x, hi.y};
+                acc[dt] = E::mfma32(acur[ks], bop, acc[dt]);
+            }
+        acur[0] = anext[0];
+        acur[1] = anext[1];
+    }
+    if (!aj_ok) return;
+    // lane (d = 32 dt + m) holds rows i = 8 g + 4 hf + e
+    const int a_blk = aj / p.b2, j = aj % p.b2;
+    const int unit = p.unit0 + u;
+    const int b = unit / p.H, h = unit % p.H;
+    float* const out = p.dq + b * p.s0 + h * p.s2;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
+        if (i < b1) {
+            const int64_t tok = p.map.row(a_blk, i) + j;
+            const float* add = p.dqk + (((int64_t)u * b1 + i) * p.AJ + aj) * D;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) out[tok * p.s1 + 32 * dt + m] = acc[dt][v] * p.scale + add[32 * dt + m];
+        }
+    }
+}
+
 }  // namespace
 
 bool monarch_bwd_left_supported(int dtype, int D, int b1) {
@@ -255,8 +401,9 @@ bool monarch_bwd_left_supported(int dtype, int D, int b1) {
 
 int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* qa,
                             const void* doa, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy,
-                            float* dc, void* ds2, hipStream_t stream) {
+                            float* dc, void* ds2, int ds2_ld, hipStream_t stream) {
     LeftArgs a;
+    a.ds2_ld = ds2_ld;
     a.c_rows = c_rows;
     a.qa = (const uint16_t*)qa; a.doa = (const uint16_t*)doa;
     a.kbar = (const uint16_t*)kbar; a.y = (const uint16_t*)y;
@@ -288,6 +435,39 @@ int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("monarch backward (left factor): launch failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+int launch_monarch_bwd_dqa(int dtype, int D, int n, int b1, int b2, int AJ, int nf, float scale, const void* kbar, const void* ds2,
+                           int ds2_ld, const float* dqk, float* dq, const int64_t* dqs, const TokMap& map, int H, int unit0,
+                           hipStream_t stream) {
+    if (ds2_ld % 4 || ds2_ld < nf * b1) {
+        set_error("monarch backward (dQ of the left factor): row pitch %d of dS2 must be a multiple of 4 and >= %d", ds2_ld, nf * b1);
+        return SFM_ERR_SHAPE;
+    }
+    DqaArgs a;
+    a.kbar = (const char*)kbar;
+    a.ds2 = (const uint16_t*)ds2;
+    a.dqk = dqk;
+    a.dq = dq;
+    a.s0 = dqs[0]; a.s1 = dqs[1]; a.s2 = dqs[2];
+    a.map = map;
+    a.ds2_ld = ds2_ld; a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.RR = nf * b1; a.H = H; a.unit0 = unit0;
+    a.scale = scale;
+    const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n);
+    const size_t ldsb = (size_t)4 * 2 * 32 * 2 * D;
+    if (dtype == SFM_BF16) {
+        if (D == 128) hipLaunchKernelGGL((monarch_bwd_dqa_kernel<BF16, 128>), grid, dim3(256), ldsb, stream, a);
+        else hipLaunchKernelGGL((monarch_bwd_dqa_kernel<BF16, 64>), grid, dim3(256), ldsb, stream, a);
+    } else {
+        if (D == 128) hipLaunchKernelGGL((monarch_bwd_dqa_kernel<F16, 128>), grid, dim3(256), ldsb, stream, a);
+        else hipLaunchKernelGGL((monarch_bwd_dqa_kernel<F16, 64>), grid, dim3(256), ldsb, stream, a);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("monarch backward (dQ of the left factor): launch failed: %s", hipGetErrorString(e));
         return SFM_ERR_HIP;
     }
     return SFM_OK;

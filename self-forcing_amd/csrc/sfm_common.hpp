@@ -186,7 +186,11 @@ int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_
 bool monarch_bwd_left_supported(int dtype, int D, int b1);
 int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* qa,
                             const void* doa, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy,
-                            float* dc, void* ds2, hipStream_t stream);
+                            float* dc, void* ds2, int ds2_ld, hipStream_t stream);
+// dq rows (caller's layout) = s dS2 Kbar per (unit, a, j) + the right factor's dQk; same limits as the left kernel
+int launch_monarch_bwd_dqa(int dtype, int D, int n, int b1, int b2, int AJ, int nf, float scale, const void* kbar, const void* ds2,
+                           int ds2_ld, const float* dqk, float* dq, const int64_t* dqs, const TokMap& map, int H, int unit0,
+                           hipStream_t stream);
 // fused right-factor part of the backward (monarch_bwd_right.hip): dS1, dK and dV blocks of every tile t = (unit, k, f)
 bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ);
 int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, const void* kk, const void* vk,
