@@ -480,6 +480,19 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     const float s = p.scale;
     const rocblas_datatype tE = El<E>::kBlas, tF = rocblas_datatype_f32_r;
 
+    const int64_t nseg = (int64_t)n * b1 * AJ * nf;
+    const bool fused_left = left_dtype<E>() >= 0 && monarch_bwd_left_supported(left_dtype<E>(), D, b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
+    // the forward's MFMA step 1 recomputes Kbar, Y, c and R straight into this scratch ([t][aj] rows)
+    const bool fused_fwd = fused_left && monarch_mfma_supported(left_dtype<E>(), D, b2) && getenv("SFM_BWD_FWD_GEMM") == nullptr;
+    // dQ of the left factor in its own kernel, which also adds the right factor's part and writes the caller's dq
+    const bool fused_dqa = fused_left && getenv("SFM_BWD_DQA_GEMM") == nullptr;
+    const int ds2_ld = fused_left ? (RR + 7) / 8 * 8 : RR;
+    const int rb_ld = fused_fwd ? 64 : b2;
+    // 9, the right factor's softmax backward, 11, 12, 13 and the scatter of dk / dv in one kernel per tile t
+    const bool direct_ok = (g.dks[0] | g.dks[1] | g.dks[2] | p.vs[0] | p.vs[1] | p.vs[2]) % 8 == 0 &&
+                           ((uintptr_t)g.dk | (uintptr_t)g.dv | (uintptr_t)p.v) % 16 == 0;
+    const bool fused_right = fused_fwd && direct_ok && monarch_bwd_right_supported(left_dtype<E>(), D, b2, AJ) &&
+                             getenv("SFM_BWD_RIGHT_GEMM") == nullptr;
     // gather q, dout (query map; both row orders) and k, v (key map)
     {
         constexpr int kPer = 8 / sizeof(T);
@@ -493,7 +506,8 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
                            p.qmap, na, H, D, p.unit0, 1, tq);
         hipLaunchKernelGGL((gather_rows<E>), dim3(gk), dim3(256), 0, stream, (T*)(ws + lay.Kk), p.k, p.ks[0], p.ks[1], p.ks[2], p.kmap,
                            nf, H, D, p.unit0, 0, tk);
-        hipLaunchKernelGGL((gather_rows<E>), dim3(gk), dim3(256), 0, stream, (T*)(ws + lay.Vk), p.v, p.vs[0], p.vs[1], p.vs[2], p.kmap,
+        if (!fused_right)                               // the fused right-factor kernel reads v where it is
+            hipLaunchKernelGGL((gather_rows<E>), dim3(gk), dim3(256), 0, stream, (T*)(ws + lay.Vk), p.v, p.vs[0], p.vs[1], p.vs[2], p.kmap,
                            nf, H, D, p.unit0, 0, tk);
     }
     const int nuk = n * b1, nt = n * b1 * nf;
@@ -508,14 +522,6 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     const Op Kbar_t{lay.Kbar, D, (int64_t)AJ * D}, Y_t{lay.Y, D, (int64_t)AJ * D};
     const Op dKbar_t{lay.dKbar, D, (int64_t)AJ * D}, dY_t{lay.dY, D, (int64_t)AJ * D};
 
-    const int64_t nseg = (int64_t)n * b1 * AJ * nf;
-    const bool fused_left = left_dtype<E>() >= 0 && monarch_bwd_left_supported(left_dtype<E>(), D, b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
-    // the forward's MFMA step 1 recomputes Kbar, Y, c and R straight into this scratch ([t][aj] rows)
-    const bool fused_fwd = fused_left && monarch_mfma_supported(left_dtype<E>(), D, b2) && getenv("SFM_BWD_FWD_GEMM") == nullptr;
-    // dQ of the left factor in its own kernel, which also adds the right factor's part and writes the caller's dq
-    const bool fused_dqa = fused_left && getenv("SFM_BWD_DQA_GEMM") == nullptr;
-    const int ds2_ld = fused_left ? (RR + 7) / 8 * 8 : RR;
-    const int rb_ld = fused_fwd ? 64 : b2;
     const Op Rb_t{lay.Rb, rb_ld, (int64_t)AJ * rb_ld};
     if (fused_fwd) {
         MonarchArgs f1 = p;
@@ -578,13 +584,11 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
         const Op dQa_u{lay.dQa + (size_t)u * MQ * D * 4, D, (int64_t)b1 * D};
         gemm(cx, false, false, b1, D, RR, s, 0.f, dS2_u, Kbar_u, dQa_u, tE, tF, AJ);
     }
-    // 9, the right factor's softmax backward, 12 and 13 in one kernel per tile t
-    const bool fused_right = fused_fwd && monarch_bwd_right_supported(left_dtype<E>(), D, b2, AJ) && getenv("SFM_BWD_RIGHT_GEMM") == nullptr;
     if (fused_right) {
         if (!cx.status)
-            cx.status = launch_monarch_bwd_right(left_dtype<E>(), D, nt, b1, b2, AJ, nf, ws + lay.Kk, ws + lay.Vk, ws + lay.Rb, ws + lay.dKbar,
-                                                 ws + lay.dY, (const float*)(ws + lay.dc), ws + lay.dS1, (float*)(ws + lay.dKk),
-                                                 (float*)(ws + lay.dVk), stream);
+            cx.status = launch_monarch_bwd_right(left_dtype<E>(), D, nt, b1, b2, AJ, nf, s, ws + lay.Kk, p.v, p.vs, ws + lay.Rb,
+                                                 ws + lay.dKbar, ws + lay.dY, (const float*)(ws + lay.dc), ws + lay.Qk, ws + lay.dS1, g.dk,
+                                                 g.dv, g.dks, g.dk_row0, p.kmap, H, p.unit0, g.kv_f0, g.kv_f1, stream);
     } else {
         // 9. dR block = dKbar block . K block^T + dY block . V block^T per t
         gemm(cx, false, true, AJ, b2, D, 1.f, 0.f, dKbar_t, Kk_t, dRb_t, tE, tF, nt);
@@ -598,10 +602,11 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     else
         hipLaunchKernelGGL((softmax_right_bwd<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const float*)(ws + lay.S1f),
                            (const float*)(ws + lay.dRb), (const float*)(ws + lay.dc), (T*)(ws + lay.dS1), b1, AJ, nf, b2, s, nseg);
-    // 10. dQ (right factor) = s dS1 K per (u, k);  11. dK (+)= s dS1^T q per (u, k)
+    // 10. dQ (right factor) = s dS1 K per (u, k)
     gemm(cx, false, false, AJ, D, NL, s, 0.f, dS1_uk, Kk_uk, dQk_uk, tE, tF, nuk);
-    gemm(cx, true, false, NL, D, AJ, s, fused_right ? 1.f : 0.f, dS1_uk, Qk_uk, dKk_uk, tE, tF, nuk);
     if (!fused_right) {
+        // 11. dK = s dS1^T q per (u, k)
+        gemm(cx, true, false, NL, D, AJ, s, 0.f, dS1_uk, Qk_uk, dKk_uk, tE, tF, nuk);
         // 12. dK block += R block^T dKbar block;  13. dV block = R block^T dY block per t
         gemm(cx, true, false, b2, D, AJ, 1.f, 1.f, Rb_t, dKbar_t, dKk_t, tE, tF, nt);
         gemm(cx, true, false, b2, D, AJ, 1.f, 0.f, Rb_t, dY_t, dVk_t, tE, tF, nt);
@@ -617,9 +622,10 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
             hipLaunchKernelGGL(scatter_dq, dim3((unsigned)((tq + 255) / 256)), dim3(256), 0, stream, (const float*)(ws + lay.dQa),
                                (const float*)(ws + lay.dQk), g.dq, g.dqs[0], g.dqs[1], g.dqs[2], p.qmap, na, H, D, p.unit0, tq);
         const int64_t tk = (int64_t)n * b1 * (g.kv_f1 - g.kv_f0) * b2 * (D / 4);
-        hipLaunchKernelGGL((scatter_dkv<E>), dim3((unsigned)((tk + 255) / 256)), dim3(256), 0, stream, (const float*)(ws + lay.dKk),
-                           (const float*)(ws + lay.dVk), (T*)g.dk, (T*)g.dv, g.dks[0], g.dks[1], g.dks[2], p.kmap, nf, g.kv_f0, g.kv_f1,
-                           g.dk_row0, H, D, p.unit0, tk);
+        if (!fused_right && tk > 0)
+            hipLaunchKernelGGL((scatter_dkv<E>), dim3((unsigned)((tk + 255) / 256)), dim3(256), 0, stream, (const float*)(ws + lay.dKk),
+                               (const float*)(ws + lay.dVk), (T*)g.dk, (T*)g.dv, g.dks[0], g.dks[1], g.dks[2], p.kmap, nf, g.kv_f0,
+                               g.kv_f1, g.dk_row0, H, D, p.unit0, tk);
         if (cx.status) return cx.status;
     }
     hipError_t err = hipGetLastError();

@@ -4,15 +4,21 @@
 // Replaces, per tile t = (unit, k, f), the small batched products and the row kernel of the GEMM chain
 //     dR[aj, l]  = dKbar[aj,:] . K[l,:] + dY[aj,:] . V[l,:]
 //     dS1[aj, l] = R (dR + dc ln R - sum_l R (dR + dc ln R))
-//     dK[l, :]   = sum_aj R[aj, l] dKbar[aj,:]          (the s dS1^T q term is added by the library GEMM that follows)
+//     dK[l, :]   = sum_aj R[aj, l] dKbar[aj,:] + s sum_aj dS1[aj, l] q[aj,:]
 //     dV[l, :]   = sum_aj R[aj, l] dY[aj,:]
 // (wan/modules/monarch_attn.py:403-596 `_al_cl_y_bwd`).  One workgroup per tile: the K and V blocks, the tile's rows of
 // R, dKbar and dY (all contiguous in the backward's scratch) go straight into LDS (global_load_lds_dwordx4, 16-byte
 // chunks XOR-swizzled per row as in the dense attention kernel), rows past the end are zeroed.
-//   phase 1: wave = 32 columns aj.  dR^T[l, aj] with A = K / V rows, B = dKbar / dY rows, so that a lane owns one
-//            column and the softmax backward is in-lane plus one cross-half add; dS1 leaves as 8-byte pieces.
-//   phase 2: wave = (dK or dV, 32 head-dim rows).  C^T[d, l] with both operands from transposing LDS reads
-//            (ds_read_tr16_b64): A = dKbar^T / dY^T, B = R^T, contraction over the columns aj.
+// Sixteen waves per workgroup (one workgroup fills the LDS of a compute unit, so the waves have to come from it).
+//   phase 1: wave = 32 columns aj x 32 key rows l (ten waves busy).  dR^T[l, aj] with A = K / V rows, B = dKbar / dY
+//            rows, so that a lane owns one column and the softmax backward is in-lane plus one cross-half add and one
+//            exchange between the two waves of a column through LDS.
+//   phase 2: wave = 32 head-dim rows x 32 key rows of dV or of dK.  C^T[d, l] with both operands from transposing LDS
+//            reads (ds_read_tr16_b64): A = dY^T / dKbar^T / q^T, B = R or dS1 (kept in LDS, 16 bit, over the K / V tiles once
+//            phase 1 is done with them), contraction over the columns aj.  The products with R run right after the
+//            logits of phase 1; the query rows of (unit, k) then load over the dY tile while the softmax backward runs.  dK and dV leave in the tensor dtype, straight to the caller's rows; tiles whose
+//            kv block-frame is outside the wanted range skip phase 2.
+// dS1 is also written to memory (16 bit) for dQ = s dS1 K, which contracts over f across tiles and stays a library GEMM.
 
 #include <hip/hip_runtime.h>
 
@@ -28,15 +34,20 @@ constexpr int kMaxAJ = 160;
 
 struct RightArgs {
     const char* kk;          // [t][b2][D]
-    const char* vk;
+    const char* v;           // caller's tensor: row kmap.row(f, k) + l, strides vs0 (batch), vs1 (row), vs2 (head), in elements
+    int64_t vs0, vs1, vs2;
     const char* rb;          // [t][AJ][64]
     const char* dkbar;       // [t][AJ][D]
     const char* dy;
     const float* dc;         // [u][AJ][RR]
+    const char* qk;          // [(u, k)][AJ][D]
     uint16_t* ds1;           // [(u, k)][AJ][nf * b2]
-    float* dkk;              // [t][b2][D]
-    float* dvk;
-    int b1, b2, AJ, nf;
+    uint16_t* dk;            // caller's tensors: row kmap.row(f, k) + l - row0, strides s0 (batch), s1 (row), s2 (head)
+    uint16_t* dv;
+    int64_t s0, s1, s2, row0;
+    TokMap kmap;
+    int b1, b2, AJ, nf, H, unit0, f0, f1;
+    float scale;
 };
 
 typedef short br_s16x4 __attribute__((ext_vector_type(4)));
@@ -54,8 +65,10 @@ __device__ __forceinline__ int br_swz(int r) {
     return CPR >= 16 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
 }
 
+constexpr int kWaves = 16, kThreads = 64 * kWaves;
+
 template <class E, int D>
-__global__ __launch_bounds__(320) void monarch_bwd_right_kernel(RightArgs p) {
+__global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p) {
     constexpr int DS = D / 16, DT = D / 32;
     constexpr int CPR = D / 8;                            // chunks per row of the D-wide tiles
     constexpr int kPitch = 2 * D;
@@ -63,6 +76,9 @@ __global__ __launch_bounds__(320) void monarch_bwd_right_kernel(RightArgs p) {
     constexpr int kG = kMaxAJ * kPitch;                   // dKbar or dY tile, 160 rows
     constexpr int kR = kMaxAJ * 128;                      // R tile, 160 rows of 64
     constexpr int oK = 0, oV = kKV, oG = 2 * kKV, oH = 2 * kKV + kG, oR = 2 * kKV + 2 * kG;
+    // dS1 tile (like R): over the K / V tiles after phase 1 where it fits there (head_dim 128), else behind the R tile
+    constexpr int oS = kR <= 2 * kKV ? 0 : oR + kR;
+    constexpr int oDot = oR + kR + (kR <= 2 * kKV ? 0 : kR);              // float [2][160]: per-column partial sums of the two l halves
     extern __shared__ __attribute__((aligned(256))) char lds[];
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
 
@@ -76,144 +92,179 @@ __global__ __launch_bounds__(320) void monarch_bwd_right_kernel(RightArgs p) {
     const int64_t u = uk / p.b1;
 
     // ---- stage the five tiles: LDS position P (16-byte units) of a tile holds chunk (P % CPR) ^ swz(row) of row P / CPR
-    auto stage = [&](const char* src, int nchunks, uint32_t dst, auto cpr_c) {
+    auto stage = [&](const char* src, uint32_t row_bytes, int nchunks, uint32_t dst, auto cpr_c) {
         constexpr int C = decltype(cpr_c)::value;
-        for (int g = wave; g * 64 < nchunks; g += 5) {
+        for (int g = wave; g * 64 < nchunks; g += kWaves) {
             const int P = min(g * 64 + lane, nchunks - 1);             // lanes past the end repeat the last chunk (into a pad row, zeroed below)
             const int r = P / C, c = (P % C) ^ br_swz<C>(r);
-            br_load_lds16(src, (uint32_t)((r * C + c) * 16), lds0 + dst + (uint32_t)g * 1024);
+            br_load_lds16(src, (uint32_t)r * row_bytes + (uint32_t)(c * 16), lds0 + dst + (uint32_t)g * 1024);
         }
     };
     using c_d = std::integral_constant<int, CPR>;
     using c_r = std::integral_constant<int, 8>;
-    stage(p.kk + t * b2 * kPitch, b2 * CPR, oK, c_d{});
-    stage(p.vk + t * b2 * kPitch, b2 * CPR, oV, c_d{});
-    stage(p.dkbar + t * AJ * kPitch, AJ * CPR, oG, c_d{});
-    stage(p.dy + t * AJ * kPitch, AJ * CPR, oH, c_d{});
-    stage(p.rb + t * AJ * 128, AJ * 8, oR, c_r{});
+    const int unit = p.unit0 + (int)u;
+    stage(p.kk + t * b2 * kPitch, kPitch, b2 * CPR, oK, c_d{});
+    stage(p.v + ((int64_t)(unit / p.H) * p.vs0 + (int64_t)(unit % p.H) * p.vs2 + p.kmap.row(f, k) * p.vs1) * 2, (uint32_t)(p.vs1 * 2),
+          b2 * CPR, oV, c_d{});
+    stage(p.dkbar + t * AJ * kPitch, kPitch, AJ * CPR, oG, c_d{});
+    stage(p.dy + t * AJ * kPitch, kPitch, AJ * CPR, oH, c_d{});
+    stage(p.rb + t * AJ * 128, 128, AJ * 8, oR, c_r{});
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     // rows past the end of a tile are zero, so that they add nothing to any contraction
     {
         const u32x4 z = {0u, 0u, 0u, 0u};
-        for (int i = tid; i < (64 - b2) * CPR; i += 320) {
+        for (int i = tid; i < (64 - b2) * CPR; i += kThreads) {
             *(u32x4*)(lds + oK + b2 * kPitch + i * 16) = z;
             *(u32x4*)(lds + oV + b2 * kPitch + i * 16) = z;
         }
-        for (int i = tid; i < (kMaxAJ - AJ) * CPR; i += 320) {
+        for (int i = tid; i < (kMaxAJ - AJ) * CPR; i += kThreads) {
             *(u32x4*)(lds + oG + AJ * kPitch + i * 16) = z;
             *(u32x4*)(lds + oH + AJ * kPitch + i * 16) = z;
         }
-        for (int i = tid; i < (kMaxAJ - AJ) * 8; i += 320) *(u32x4*)(lds + oR + AJ * 128 + i * 16) = z;
+        for (int i = tid; i < (kMaxAJ - AJ) * 8; i += kThreads) *(u32x4*)(lds + oR + AJ * 128 + i * 16) = z;
     }
     __syncthreads();
 
-    // ---- phase 1: dS1 for the wave's 32 columns
-    {
-        const int col = 32 * wave + m;                                   // < 160
-        const bool col_ok = col < AJ;
-        const uint32_t a_off = (uint32_t)m * kPitch + (uint32_t)((hf ^ br_swz<CPR>(m)) << 4);          // rows l = 32 tl + m (swz depends on r mod 16)
+    const bool want = f >= p.f0 && f < p.f1;                             // uniform: dK / dV of this kv block-frame are asked for
+
+    // phase 2 operands: C^T[d, l] = sum_aj A^T[d, aj] B[aj, l]; a wave owns 32 head-dim rows x 32 key rows of dV (waves
+    // 0 .. 2 DT - 1) or of dK (the next 2 DT waves)
+    const int s16 = lane & 15, g16 = lane >> 4;
+    const int rl = 4 * hf + (s16 >> 2);
+    const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
+    const uint32_t sub = (uint32_t)(s16 & 1) * 8;
+    const int dt = wave % DT, lb = (wave / DT) & 1, which = wave / (2 * DT);      // which: 0 dV, 1 dK, else idle
+    auto product = [&](uint32_t oA, uint32_t oB, f32x16& acc) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+        const int ca = 4 * dt + cl, cb = 4 * lb + cl;
+#pragma unroll
+        for (int ks = 0; ks < kMaxAJ / 16; ++ks) {
+            const int r0 = 16 * ks + rl, r1 = r0 + 8;                     // rows aj of the two halves of the operands
+            const u32x2 alo = br_read_tr(lds, oA + (uint32_t)r0 * kPitch + (uint32_t)((ca ^ br_swz<CPR>(r0)) << 4) + sub);
+            const u32x2 ahi = br_read_tr(lds, oA + (uint32_t)r1 * kPitch + (uint32_t)((ca ^ br_swz<CPR>(r1)) << 4) + sub);
+            const u32x2 blo = br_read_tr(lds, oB + (uint32_t)r0 * 128 + (uint32_t)((cb ^ br_swz<8>(r0)) << 4) + sub);
+            const u32x2 bhi = br_read_tr(lds, oB + (uint32_t)r1 * 128 + (uint32_t)((cb ^ br_swz<8>(r1)) << 4) + sub);
+            const u32x4 aop = {alo.x, alo.y, ahi.x, ahi.y};
+            const u32x4 bop = {blo.x, blo.y, bhi.x, bhi.y};
+            acc = E::mfma32(aop, bop, acc);
+        }
+    };
+    // lane (l, hf) holds head-dim 32 dt + 8 g + 4 hf + 0..3 of key row l; the half swap leaves 8 consecutive ones per lane
+    const int64_t obase = (int64_t)(unit / p.H) * p.s0 + (int64_t)(unit % p.H) * p.s2 + (p.kmap.row(f, k) - p.row0) * p.s1;
+    auto store = [&](uint16_t* dst, const f32x16& acc) {
+        const int l = 32 * lb + m;
+        uint16_t* row = dst + obase + min(l, b2 - 1) * p.s1 + 32 * dt + 8 * hf;
+#pragma unroll
+        for (int gp = 0; gp < 2; ++gp) {
+            const int g0 = 8 * gp, g1 = 8 * gp + 4;
+            auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[g0 + 0], acc[g0 + 1]), pack2<E>(acc[g1 + 0], acc[g1 + 1]), false, false);
+            auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[g0 + 2], acc[g0 + 3]), pack2<E>(acc[g1 + 2], acc[g1 + 3]), false, false);
+            const u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+            if (l < b2) *(u32x4*)(row + 16 * gp) = w;
+        }
+    };
+
+    // ---- phase 1 (waves 0..9 = (32 columns aj, 32 rows l) blocks of dS1), products: dR^T
+    const bool active = wave < 10;
+    const int cblk = wave % 5, tl = (wave / 5) & 1;
+    const int col = 32 * cblk + m;                                       // < 160
+    f32x16 dr;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dr[v] = 0.f;
+    if (active) {
+        const uint32_t a_off = (uint32_t)(32 * tl + m) * kPitch + (uint32_t)((hf ^ br_swz<CPR>(m)) << 4);   // swz depends on r mod 16
         const uint32_t b_off = (uint32_t)col * kPitch + (uint32_t)((hf ^ br_swz<CPR>(col)) << 4);
-        f32x16 dr[2];
-#pragma unroll
-        for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) dr[tl][v] = 0.f;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
             const u32x4 bg = *(const u32x4*)(lds + oG + (b_off ^ (uint32_t)(ds << 5)));
             const u32x4 bh = *(const u32x4*)(lds + oH + (b_off ^ (uint32_t)(ds << 5)));
-#pragma unroll
-            for (int tl = 0; tl < 2; ++tl) {
-                const u32x4 ak = *(const u32x4*)(lds + oK + tl * 32 * kPitch + (a_off ^ (uint32_t)(ds << 5)));
-                const u32x4 av = *(const u32x4*)(lds + oV + tl * 32 * kPitch + (a_off ^ (uint32_t)(ds << 5)));
-                dr[tl] = E::mfma32(ak, bg, dr[tl]);
-                dr[tl] = E::mfma32(av, bh, dr[tl]);
-            }
+            const u32x4 ak = *(const u32x4*)(lds + oK + (a_off ^ (uint32_t)(ds << 5)));
+            const u32x4 av = *(const u32x4*)(lds + oV + (a_off ^ (uint32_t)(ds << 5)));
+            dr = E::mfma32(ak, bg, dr);
+            dr = E::mfma32(av, bh, dr);
         }
-        // R[col][l] for the l this lane holds: l = 32 tl + 8 g + 4 hf + 0..3, i.e. 8 bytes of chunk 4 tl + g
-        const float dcv = col_ok ? p.dc[(u * AJ + col) * ((int64_t)nf * p.b1) + (int64_t)k * nf + f] : 0.f;
-        float rv[2][16];
-        float dot = 0.f;
-#pragma unroll
-        for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int c = 4 * tl + g;
-                const u32x2 w = *(const u32x2*)(lds + oR + col * 128 + ((c ^ br_swz<8>(col)) << 4) + 8 * hf);
-                const float r0 = E::to_float((uint16_t)(w.x & 0xffffu)), r1 = E::to_float((uint16_t)(w.x >> 16));
-                const float r2 = E::to_float((uint16_t)(w.y & 0xffffu)), r3 = E::to_float((uint16_t)(w.y >> 16));
-                const bool live = 32 * tl + 8 * g + 4 * hf < b2;        // b2 is a multiple of 4: whole pieces
-                const float rr[4] = {live ? r0 : 0.f, live ? r1 : 0.f, live ? r2 : 0.f, live ? r3 : 0.f};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int v = 4 * g + e;
-                    float gv = dr[tl][v];
-                    if (rr[e] > 0.f) gv += dcv * __logf(rr[e]);          // dR + dc ln R
-                    else gv = 0.f;
-                    rv[tl][v] = rr[e];
-                    dr[tl][v] = gv;
-                    dot += rr[e] * gv;
-                }
-            }
-        dot = xhalf_sum(dot);
-        uint16_t* out = p.ds1 + (uk * AJ + col) * ((int64_t)nf * b2) + (int64_t)f * b2;
-#pragma unroll
-        for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int l0 = 32 * tl + 8 * g + 4 * hf;
-                u32x2 w;
-                w.x = pack2<E>(rv[tl][4 * g + 0] * (dr[tl][4 * g + 0] - dot), rv[tl][4 * g + 1] * (dr[tl][4 * g + 1] - dot));
-                w.y = pack2<E>(rv[tl][4 * g + 2] * (dr[tl][4 * g + 2] - dot), rv[tl][4 * g + 3] * (dr[tl][4 * g + 3] - dot));
-                if (col_ok && l0 < b2) *(u32x2*)(out + l0) = w;
-            }
     }
+    // ---- phase 2, the products that only need the loaded tiles: dV = R^T dY (finished), R^T dKbar
+    f32x16 acc;
+    if (want) {
+        if (which == 0) {
+            product(oH, oR, acc);                                        // stored at the end: a store in flight would hold up the wait for the query rows
+        } else if (which == 1) {
+            product(oG, oR, acc);
+        }
+    }
+    __syncthreads();                                                     // K, V, dKbar, dY tiles are free
+    // the query rows of (unit, k) take the place of the dY tile while the softmax backward runs
+    if (want) stage(p.qk + uk * AJ * kPitch, kPitch, AJ * CPR, oH, c_d{});
 
-    // ---- phase 2: dK^T[d, l] = sum_aj dKbar^T[d, aj] R[aj, l] and the same with dY for dV; work items (product, 32 head-dim rows)
-    {
-        const int s16 = lane & 15, g16 = lane >> 4;
-        const int rl = 4 * hf + (s16 >> 2);
-        const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
-        const uint32_t sub = (uint32_t)(s16 & 1) * 8;
-        for (int item = wave; item < 2 * DT; item += 5) {
-            const int which = item / DT, dt = item % DT;
-            const uint32_t oA = which == 0 ? oG : oH;
-            f32x16 acc[2];
+    // ---- phase 1, softmax backward.  R[col][l] for the l this lane holds: l = 32 tl + 8 g + 4 hf + 0..3, 8 bytes of chunk 4 tl + g
+    float rv[16];
+    float dot = 0.f;
+    if (active) {
+        const float dcv = col < AJ ? p.dc[(u * AJ + col) * ((int64_t)nf * p.b1) + (int64_t)k * nf + f] : 0.f;
 #pragma unroll
-            for (int lb = 0; lb < 2; ++lb)
+        for (int g = 0; g < 4; ++g) {
+            const int c = 4 * tl + g;
+            const u32x2 w = *(const u32x2*)(lds + oR + col * 128 + ((c ^ br_swz<8>(col)) << 4) + 8 * hf);
+            const float r0 = E::to_float((uint16_t)(w.x & 0xffffu)), r1 = E::to_float((uint16_t)(w.x >> 16));
+            const float r2 = E::to_float((uint16_t)(w.y & 0xffffu)), r3 = E::to_float((uint16_t)(w.y >> 16));
+            const bool live = 32 * tl + 8 * g + 4 * hf < b2;            // b2 is a multiple of 4: whole pieces
+            const float rr[4] = {live ? r0 : 0.f, live ? r1 : 0.f, live ? r2 : 0.f, live ? r3 : 0.f};
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[lb][v] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < kMaxAJ / 16; ++ks) {
-                const int r0 = 16 * ks + rl, r1 = r0 + 8;                 // rows aj of the two halves of the operand
-                const int ca = 4 * dt + cl;
-                const u32x2 alo = br_read_tr(lds, oA + (uint32_t)r0 * kPitch + (uint32_t)((ca ^ br_swz<CPR>(r0)) << 4) + sub);
-                const u32x2 ahi = br_read_tr(lds, oA + (uint32_t)r1 * kPitch + (uint32_t)((ca ^ br_swz<CPR>(r1)) << 4) + sub);
-                const u32x4 aop = {alo.x, alo.y, ahi.x, ahi.y};
-#pragma unroll
-                for (int lb = 0; lb < 2; ++lb) {
-                    const int cb = 4 * lb + cl;
-                    const u32x2 blo = br_read_tr(lds, oR + (uint32_t)r0 * 128 + (uint32_t)((cb ^ br_swz<8>(r0)) << 4) + sub);
-                    const u32x2 bhi = br_read_tr(lds, oR + (uint32_t)r1 * 128 + (uint32_t)((cb ^ br_swz<8>(r1)) << 4) + sub);
-                    const u32x4 bop = {blo.x, blo.y, bhi.x, bhi.y};
-                    acc[lb] = E::mfma32(aop, bop, acc[lb]);
-                }
-            }
-            float* dst = which == 0 ? p.dkk : p.dvk;
-#pragma unroll
-            for (int lb = 0; lb < 2; ++lb) {
-                const int l = 32 * lb + m;
-                if (l < b2) {
-                    float* row = dst + (t * b2 + l) * D + 32 * dt + 4 * hf;
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const f32x4 w = {acc[lb][4 * g + 0], acc[lb][4 * g + 1], acc[lb][4 * g + 2], acc[lb][4 * g + 3]};
-                        *(f32x4*)(row + 8 * g) = w;
-                    }
-                }
+            for (int e = 0; e < 4; ++e) {
+                const int v = 4 * g + e;
+                float gv = dr[v];
+                if (rr[e] > 0.f) gv += dcv * __logf(rr[e]);              // dR + dc ln R
+                else gv = 0.f;
+                rv[v] = rr[e];
+                dr[v] = gv;
+                dot += rr[e] * gv;
             }
         }
+        dot = xhalf_sum(dot);
+        if (hf == 0) *(float*)(lds + oDot + (tl * kMaxAJ + col) * 4) = dot;
+    }
+    lds_barrier();                                                       // (the query rows stay in flight)
+    if (active) {
+        dot = *(const float*)(lds + oDot + col * 4) + *(const float*)(lds + oDot + (kMaxAJ + col) * 4);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u32x2 w;
+            w.x = pack2<E>(rv[4 * g + 0] * (dr[4 * g + 0] - dot), rv[4 * g + 1] * (dr[4 * g + 1] - dot));
+            w.y = pack2<E>(rv[4 * g + 2] * (dr[4 * g + 2] - dot), rv[4 * g + 3] * (dr[4 * g + 3] - dot));
+            // into the dS1 tile, laid out like R's (columns past the end and l >= b2 come out as zeros)
+            *(u32x2*)(lds + oS + col * 128 + (((4 * tl + g) ^ br_swz<8>(col)) << 4) + 8 * hf) = w;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                     // the query rows have landed
+    __syncthreads();                                                     // the dS1 tile is complete
+    // dS1 to memory for dQ = s dS1 K: row aj is b2 consecutive elements, 8-byte pieces, consecutive lanes along a row
+    {
+        const int ppr = b2 / 4;                                          // pieces per row
+        uint16_t* out = p.ds1 + uk * AJ * ((int64_t)nf * b2) + (int64_t)f * b2;
+        for (int i = tid; i < AJ * ppr; i += kThreads) {
+            const int row = i / ppr, pc = i % ppr;
+            const u32x2 w = *(const u32x2*)(lds + oS + row * 128 + (((pc >> 1) ^ br_swz<8>(row)) << 4) + 8 * (pc & 1));
+            *(u32x2*)(out + (int64_t)row * nf * b2 + 4 * pc) = w;
+        }
+    }
+    if (!want) return;
+    if ((AJ * CPR) % 64) {                                               // the last load spilled copies of a chunk into the zero rows
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        for (int i = tid; i < (kMaxAJ - AJ) * CPR; i += kThreads) *(u32x4*)(lds + oH + AJ * kPitch + i * 16) = z;
+        __syncthreads();
+    }
+    // ---- phase 2, the product that needs dS1: dK = R^T dKbar + s dS1^T q
+    if (which == 1) {
+        f32x16 accq;
+        product(oH, oS, accq);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] += p.scale * accq[v];
+        store(p.dk, acc);
+    } else if (which == 0) {
+        store(p.dv, acc);
     }
 }
 
@@ -223,17 +274,29 @@ bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ) {
     return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 >= 4 && b2 <= 64 && b2 % 4 == 0 && AJ <= kMaxAJ;
 }
 
-int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, const void* kk, const void* vk,
-                             const void* rb, const void* dkbar, const void* dy, const float* dc, void* ds1, float* dkk, float* dvk,
+int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, float scale, const void* kk, const void* v,
+                             const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* qk, void* ds1, void* dk,
+                             void* dv, const int64_t* dks, int64_t row0, const TokMap& kmap, int H, int unit0, int f0, int f1,
                              hipStream_t stream) {
+    if ((dks[0] | dks[1] | dks[2] | vs[0] | vs[1] | vs[2]) % 8 || ((uintptr_t)dk | (uintptr_t)dv | (uintptr_t)v) % 16 ||
+        (int64_t)(b2 - 1) * vs[1] * 2 + 2 * D > 0xffffffffll) {
+        set_error("monarch backward (right factor): v / dk / dv strides must be multiples of 8 elements and the pointers 16-byte aligned");
+        return SFM_ERR_STRIDE;
+    }
     RightArgs a;
-    a.kk = (const char*)kk; a.vk = (const char*)vk; a.rb = (const char*)rb;
+    a.kk = (const char*)kk; a.rb = (const char*)rb;
+    a.v = (const char*)v; a.vs0 = vs[0]; a.vs1 = vs[1]; a.vs2 = vs[2];
     a.dkbar = (const char*)dkbar; a.dy = (const char*)dy;
     a.dc = dc;
+    a.qk = (const char*)qk;
     a.ds1 = (uint16_t*)ds1;
-    a.dkk = dkk; a.dvk = dvk;
-    a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.nf = nf;
-    const size_t ldsb = (size_t)2 * 64 * 2 * D + (size_t)2 * kMaxAJ * 2 * D + (size_t)kMaxAJ * 128;
+    a.dk = (uint16_t*)dk; a.dv = (uint16_t*)dv;
+    a.s0 = dks[0]; a.s1 = dks[1]; a.s2 = dks[2]; a.row0 = row0;
+    a.kmap = kmap;
+    a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.nf = nf; a.H = H; a.unit0 = unit0; a.f0 = f0; a.f1 = f1;
+    a.scale = scale;
+    const size_t kv = (size_t)2 * 64 * 2 * D, rt = (size_t)kMaxAJ * 128;
+    const size_t ldsb = kv + (size_t)2 * kMaxAJ * 2 * D + rt + (rt <= kv ? 0 : rt) + 2 * kMaxAJ * 4;
     const void* fn = nullptr;
     if (dtype == SFM_BF16) fn = D == 128 ? (const void*)monarch_bwd_right_kernel<BF16, 128> : (const void*)monarch_bwd_right_kernel<BF16, 64>;
     else fn = D == 128 ? (const void*)monarch_bwd_right_kernel<F16, 128> : (const void*)monarch_bwd_right_kernel<F16, 64>;
@@ -246,11 +309,11 @@ int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, i
     }
     const dim3 grid((unsigned)ntiles);
     if (dtype == SFM_BF16) {
-        if (D == 128) hipLaunchKernelGGL((monarch_bwd_right_kernel<BF16, 128>), grid, dim3(320), ldsb, stream, a);
-        else hipLaunchKernelGGL((monarch_bwd_right_kernel<BF16, 64>), grid, dim3(320), ldsb, stream, a);
+        if (D == 128) hipLaunchKernelGGL((monarch_bwd_right_kernel<BF16, 128>), grid, dim3(kThreads), ldsb, stream, a);
+        else hipLaunchKernelGGL((monarch_bwd_right_kernel<BF16, 64>), grid, dim3(kThreads), ldsb, stream, a);
     } else {
-        if (D == 128) hipLaunchKernelGGL((monarch_bwd_right_kernel<F16, 128>), grid, dim3(320), ldsb, stream, a);
-        else hipLaunchKernelGGL((monarch_bwd_right_kernel<F16, 64>), grid, dim3(320), ldsb, stream, a);
+        if (D == 128) hipLaunchKernelGGL((monarch_bwd_right_kernel<F16, 128>), grid, dim3(kThreads), ldsb, stream, a);
+        else hipLaunchKernelGGL((monarch_bwd_right_kernel<F16, 64>), grid, dim3(kThreads), ldsb, stream, a);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

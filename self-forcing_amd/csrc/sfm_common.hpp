@@ -191,10 +191,12 @@ int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int
 int launch_monarch_bwd_dqa(int dtype, int D, int n, int b1, int b2, int AJ, int nf, float scale, const void* kbar, const void* ds2,
                            int ds2_ld, const float* dqk, float* dq, const int64_t* dqs, const TokMap& map, int H, int unit0,
                            hipStream_t stream);
-// fused right-factor part of the backward (monarch_bwd_right.hip): dS1, dK and dV blocks of every tile t = (unit, k, f)
+// fused right-factor part of the backward (monarch_bwd_right.hip): per tile t = (unit, k, f) the dS1 block (scratch, for
+// dQ = s dS1 K) and the finished dK / dV rows of kv block-frames [f0, f1) in the caller's tensors; v is the caller's tensor too
 bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ);
-int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, const void* kk, const void* vk,
-                             const void* rb, const void* dkbar, const void* dy, const float* dc, void* ds1, float* dkk, float* dvk,
+int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, float scale, const void* kk, const void* v,
+                             const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* qk, void* ds1, void* dk,
+                             void* dv, const int64_t* dks, int64_t row0, const TokMap& kmap, int H, int unit0, int f0, int f1,
                              hipStream_t stream);
 
 void set_error(const char* fmt, ...);
