@@ -74,6 +74,16 @@ int sfm_monarch_workspace_bytes(const sfm_monarch_desc* desc, int32_t heads_per_
 int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
                     void* workspace, size_t workspace_bytes, void* stream);
 
+/* Forward that also keeps what the backward can reuse, as the reference's forward does under autograd
+ * (OUTPUT_FULL_LSE and ctx.save_for_backward(q, k, v, z, z_lse), monarch_attn.py:1309, 1317, 1559): `stats` receives
+ * one float per (batch, head, query token), the base-2 log-sum-exp of the row's left-factor logits, in the library's
+ * own order (row pitch round_up(b1, 32) per (batch, head, a, j)); treat it as opaque and hand it to
+ * sfm_monarch_bwd_saved together with `out`.  sfm_monarch_stats_bytes gives its size, 0 when the forward that would
+ * run for this descriptor produces no statistics (then use sfm_monarch_fwd and sfm_monarch_bwd). */
+int sfm_monarch_stats_bytes(const sfm_monarch_desc* desc, size_t* bytes);
+int sfm_monarch_fwd_stats(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out, float* stats,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
 /* Measurement variant of sfm_monarch_fwd: brackets the two kernels of every pass with hipEvents recorded on
  * `stream`, WAITS for them, and returns the summed kernel durations in milliseconds.  No counterpart in the
  * reference (its pipeline times whole chunks with torch.cuda.Event, pipeline/causal_inference.py:105-115). */
@@ -89,7 +99,7 @@ int sfm_monarch_fwd_timed(const sfm_monarch_desc* desc, const void* q, const voi
  *                       order of k: token order, or block order when fwd.kv_block_order = 1
  *   kv_grad_frame_*     kv block-frames whose gradients are produced; a proper sub-range is the reference's
  *                       grad_only_new_kv (:1364-1374) and needs block order
- * Everything is recomputed from q, k, v (the forward saves nothing but its inputs).  The workspace size depends
+ * Everything is recomputed from q, k, v (see sfm_monarch_bwd_saved for the variant that reuses the forward's output).  The workspace size depends
  * on the implementation in use (sfm_monarch_bwd_uses_gemm); query it in the same process state. */
 typedef struct sfm_monarch_bwd_desc {
     sfm_monarch_desc fwd;
@@ -106,6 +116,14 @@ int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t he
 int sfm_monarch_bwd_uses_gemm(void);
 int sfm_monarch_bwd(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* dout,
                     float* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream);
+
+/* sfm_monarch_bwd with the forward's output and row statistics (sfm_monarch_fwd_stats on the same descriptor and
+ * inputs) at hand, as the reference's backward has z and z_lse (monarch_attn.py:1327, 1567): the left factor's
+ * statistics pass is skipped.  `out` has the layout of `dout` (fwd.o_stride).  Same results as sfm_monarch_bwd up to
+ * rounding; implementations that cannot use the saved tensors ignore them. */
+int sfm_monarch_bwd_saved(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* out,
+                          const float* stats, const void* dout, float* dq, void* dk, void* dv, void* workspace,
+                          size_t workspace_bytes, void* stream);
 
 /* Writes new_k/new_v [B, n_new, H, D] (token order) into k_cache/v_cache[:, start_idx:end_idx]
  * in Monarch block order.  Replaces monarch_attn.py:1784-1785 + 1230-1231.

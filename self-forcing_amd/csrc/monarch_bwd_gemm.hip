@@ -392,7 +392,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // Scratch of a pass over n units, in bytes (all sub-buffers 256-byte aligned).
 struct Layout {
-    size_t Qk, Qa, dOa, Kk, Vk, S1f, dRb, Rb, dS1, Kbar, Y, dKbar, dY, c, dc, S2f, dLmf, L, dS2, dQa, dQk, dKk, dVk, total;
+    size_t Qk, Qa, dOa, Oa, Kk, Vk, S1f, dRb, Rb, dS1, Kbar, Y, dKbar, dY, c, dc, S2f, dLmf, L, dS2, dQa, dQk, dKk, dVk, total;
 };
 
 Layout make_layout(const MonarchArgs& p, int n, size_t e) {
@@ -404,6 +404,7 @@ Layout make_layout(const MonarchArgs& p, int n, size_t e) {
     l.Qk = take(n * MQ * D * e);
     l.Qa = take(n * MQ * D * e);
     l.dOa = take(n * MQ * D * e);
+    l.Oa = take(n * MQ * D * e);
     l.Kk = take(n * MK * D * e);
     l.Vk = take(n * MK * D * e);
     l.S1f = take(n * p.b1 * AJ * NL * 4);
@@ -493,6 +494,8 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
                            ((uintptr_t)g.dk | (uintptr_t)g.dv | (uintptr_t)p.v) % 16 == 0;
     const bool fused_right = fused_fwd && direct_ok && monarch_bwd_right_supported(left_dtype<E>(), D, b2, AJ) &&
                              getenv("SFM_BWD_RIGHT_GEMM") == nullptr;
+    // the forward's output and row statistics, when the caller kept them, save the left factor's first pass
+    const bool saved = fused_left && g.fout != nullptr && g.fstats != nullptr;
     // gather q, dout (query map; both row orders) and k, v (key map)
     {
         constexpr int kPer = 8 / sizeof(T);
@@ -504,6 +507,9 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
                            na, H, D, p.unit0, 1, tq);
         hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.dOa), g.dout, g.dos[0], g.dos[1], g.dos[2],
                            p.qmap, na, H, D, p.unit0, 1, tq);
+        if (saved)
+            hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.Oa), g.fout, g.dos[0], g.dos[1], g.dos[2],
+                               p.qmap, na, H, D, p.unit0, 1, tq);
         hipLaunchKernelGGL((gather_rows<E>), dim3(gk), dim3(256), 0, stream, (T*)(ws + lay.Kk), p.k, p.ks[0], p.ks[1], p.ks[2], p.kmap,
                            nf, H, D, p.unit0, 0, tk);
         if (!fused_right)                               // the fused right-factor kernel reads v where it is
@@ -548,7 +554,8 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
         if (!cx.status)
             cx.status = launch_monarch_bwd_left(left_dtype<E>(), D, n, b1, b2, AJ, nf, p.causal, s, ws + lay.Qa, ws + lay.dOa, ws + lay.Kbar,
                                                 ws + lay.Y, (const float*)(ws + lay.c), fused_fwd ? 1 : 0, ws + lay.dKbar, ws + lay.dY,
-                                                (float*)(ws + lay.dc), ws + lay.dS2, ds2_ld, stream);
+                                                (float*)(ws + lay.dc), ws + lay.dS2, ds2_ld, saved ? ws + lay.Oa : nullptr,
+                                                saved ? g.fstats : nullptr, (b1 + 31) / 32 * 32, p.unit0, stream);
     } else {
         // 4, 5. per unit and (a, j): S2 = q_i . Kbar_r, dLm = dO_i . Y_r; the [RR x D] matrix of column aj is every AJ-th row
         for (int u = 0; u < n && !cx.status; ++u) {

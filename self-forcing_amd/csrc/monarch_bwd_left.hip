@@ -34,6 +34,9 @@ struct LeftArgs {
     float* dc;               // [u][aj][RR]
     uint16_t* ds2;           // [u][aj][b1][ds2_ld], ds2_ld >= RR
     int ds2_ld;
+    const uint16_t* oa;      // optional, with stats: the forward's output rows [u][aj][b1][D]
+    const float* stats;      // log2-sum-exp of the logits of row (unit, aj, i) at ((unit0 + u) * AJ + aj) * stats_ld + i
+    int stats_ld, unit0;
     int b1, b2, AJ, nf, RR, causal;
     float scale;
 };
@@ -48,7 +51,7 @@ template <class E, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void monarch_bwd_left_kernel(LeftArgs p) {
     constexpr int DS = D / 16, DT = D / 32;
     constexpr int kPitch = (D + 8) * 2;                   // bytes per staged row
-    constexpr int kPerWave = 2 * 32 * kPitch;             // q rows, then dO rows
+    constexpr int kPerWave = 2 * 32 * kPitch + 128;       // q rows, then dO rows, then 32 floats
     extern __shared__ __attribute__((aligned(16))) char lds[];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, m = lane & 31, hf = lane >> 5;
@@ -61,19 +64,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     char* qs = lds + wave * kPerWave;
     char* dos = qs + 32 * kPitch;
+    float* dls = (float*)(dos + 32 * kPitch);
+    const bool saved = p.stats != nullptr;                // uniform: the forward's output and row statistics are at hand
     {
         const uint16_t* qg = p.qa + uaj * b1 * D;
         const uint16_t* dg = p.doa + uaj * b1 * D;
+        const uint16_t* og = saved ? p.oa + uaj * b1 * D : dg;
         constexpr int CH = D / 8;
         for (int cidx = lane; cidx < 32 * CH; cidx += 64) {
             const int r = cidx / CH, ch = cidx % CH;
             u32x4 a = {0u, 0u, 0u, 0u}, b = a;
+            float dot = 0.f;
             if (r < b1) {
                 a = *(const u32x4*)(qg + r * D + ch * 8);
                 b = *(const u32x4*)(dg + r * D + ch * 8);
+                if (saved) {                              // sum_r L dLm of row i is dO_i . O_i
+                    const u32x4 o = *(const u32x4*)(og + r * D + ch * 8);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        dot += E::to_float((uint16_t)(b[e] & 0xffffu)) * E::to_float((uint16_t)(o[e] & 0xffffu)) +
+                               E::to_float((uint16_t)(b[e] >> 16)) * E::to_float((uint16_t)(o[e] >> 16));
+                }
             }
             *(u32x4*)(qs + r * kPitch + ch * 16) = a;
             *(u32x4*)(dos + r * kPitch + ch * 16) = b;
+            if (saved) {
+#pragma unroll
+                for (int o = 1; o < CH; o <<= 1) dot += __shfl_xor(dot, o);
+                if (ch == 0) dls[r] = dot;
+            }
         }
     }
     __syncthreads();
@@ -119,48 +138,58 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         return r < RR && (r % p.nf) < flim;
     };
 
-    // ---- pass 1: per lane, for its 16 rows i, the running maximum, sum and sum of L dLm over the lane's own r
-    float mloc[16], lloc[16], dloc[16];
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        mloc[v] = -INFINITY;
-        lloc[v] = dloc[v] = 0.f;
-    }
-    load_tile(0);
-    for (int n = 0; n < nch; ++n) {
-        f32x16 s, d;
-        products(s, d);
-        const float cl2 = ccur;
-        const bool ok = row_ok(n);
-        load_tile(min(n + 1, nch - 1));
+    float lse[16], delta[16];
+    if (saved) {
+        const float* st = p.stats + ((int64_t)(p.unit0 + u) * p.AJ + aj) * p.stats_ld;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const float z = ok ? s[v] * sc2 - cl2 : -INFINITY;
-            const float mnew = fmaxf(mloc[v], z);
-            const float mref = mnew == -INFINITY ? 0.f : mnew;
-            const float alpha = fast_exp2(mloc[v] - mref), e = fast_exp2(z - mref);
-            lloc[v] = lloc[v] * alpha + e;
-            dloc[v] = dloc[v] * alpha + e * d[v];
-            mloc[v] = mnew;
+            const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
+            lse[v] = st[min(i, b1 - 1)];
+            delta[v] = dls[i];
         }
-    }
-    // merge over the 32 lanes of a half (they hold the same rows i); every row has at least one visible r
-    float lse[16], delta[16];
+    } else {
+        // ---- pass 1: per lane, for its 16 rows i, the running maximum, sum and sum of L dLm over the lane's own r
+        float mloc[16], lloc[16], dloc[16];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        float mm = mloc[v], ll = lloc[v], dd = dloc[v];
-#pragma unroll
-        for (int o = 1; o < 32; o <<= 1) {
-            const float m2 = __shfl_xor(mm, o), l2 = __shfl_xor(ll, o), d2 = __shfl_xor(dd, o);
-            const float mnew = fmaxf(mm, m2);
-            const float mref = mnew == -INFINITY ? 0.f : mnew;
-            const float a1 = fast_exp2(mm - mref), a2 = fast_exp2(m2 - mref);
-            ll = ll * a1 + l2 * a2;
-            dd = dd * a1 + d2 * a2;
-            mm = mnew;
+        for (int v = 0; v < 16; ++v) {
+            mloc[v] = -INFINITY;
+            lloc[v] = dloc[v] = 0.f;
         }
-        lse[v] = mm + log2f(ll);
-        delta[v] = dd / ll;
+        load_tile(0);
+        for (int n = 0; n < nch; ++n) {
+            f32x16 s, d;
+            products(s, d);
+            const float cl2 = ccur;
+            const bool ok = row_ok(n);
+            load_tile(min(n + 1, nch - 1));
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float z = ok ? s[v] * sc2 - cl2 : -INFINITY;
+                const float mnew = fmaxf(mloc[v], z);
+                const float mref = mnew == -INFINITY ? 0.f : mnew;
+                const float alpha = fast_exp2(mloc[v] - mref), e = fast_exp2(z - mref);
+                lloc[v] = lloc[v] * alpha + e;
+                dloc[v] = dloc[v] * alpha + e * d[v];
+                mloc[v] = mnew;
+            }
+        }
+        // merge over the 32 lanes of a half (they hold the same rows i); every row has at least one visible r
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            float mm = mloc[v], ll = lloc[v], dd = dloc[v];
+#pragma unroll
+            for (int o = 1; o < 32; o <<= 1) {
+                const float m2 = __shfl_xor(mm, o), l2 = __shfl_xor(ll, o), d2 = __shfl_xor(dd, o);
+                const float mnew = fmaxf(mm, m2);
+                const float mref = mnew == -INFINITY ? 0.f : mnew;
+                const float a1 = fast_exp2(mm - mref), a2 = fast_exp2(m2 - mref);
+                ll = ll * a1 + l2 * a2;
+                dd = dd * a1 + d2 * a2;
+                mm = mnew;
+            }
+            lse[v] = mm + log2f(ll);
+            delta[v] = dd / ll;
+        }
     }
 
     // ---- pass 2: gradients
@@ -401,9 +430,11 @@ bool monarch_bwd_left_supported(int dtype, int D, int b1) {
 
 int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* qa,
                             const void* doa, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy,
-                            float* dc, void* ds2, int ds2_ld, hipStream_t stream) {
+                            float* dc, void* ds2, int ds2_ld, const void* oa, const float* stats, int stats_ld, int unit0,
+                            hipStream_t stream) {
     LeftArgs a;
     a.ds2_ld = ds2_ld;
+    a.oa = (const uint16_t*)oa; a.stats = oa ? stats : nullptr; a.stats_ld = stats_ld; a.unit0 = unit0;
     a.c_rows = c_rows;
     a.qa = (const uint16_t*)qa; a.doa = (const uint16_t*)doa;
     a.kbar = (const uint16_t*)kbar; a.y = (const uint16_t*)y;
@@ -414,7 +445,7 @@ int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int
     a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.nf = nf; a.RR = nf * b1; a.causal = causal;
     a.scale = scale;
     const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n);
-    const size_t ldsb = (size_t)4 * 2 * 32 * (D + 8) * 2;
+    const size_t ldsb = (size_t)4 * (2 * 32 * (D + 8) * 2 + 128);
     const void* fn = nullptr;
     if (dtype == SFM_BF16) fn = D == 128 ? (const void*)monarch_bwd_left_kernel<BF16, 128> : (const void*)monarch_bwd_left_kernel<BF16, 64>;
     else fn = D == 128 ? (const void*)monarch_bwd_left_kernel<F16, 128> : (const void*)monarch_bwd_left_kernel<F16, 64>;

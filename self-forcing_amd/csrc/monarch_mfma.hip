@@ -539,7 +539,10 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
     }
 
     // epilogue: O[i, d] = O^T / l, through the wave's LDS region (the query rows are dead now)
-    const float inv = 1.f / xhalf_sum(lrun);
+    const float ltot = xhalf_sum(lrun);
+    const float inv = 1.f / ltot;
+    if (p.stats != nullptr && hf == 0 && j_ok && i0 + m < p.b1)
+        p.stats[((int64_t)unit * (p.na * b2) + a * b2 + j) * p.stats_ld + i0 + m] = mrun + log2f(ltot);
     __syncthreads();
 #pragma unroll
     for (int dp = 0; dp < DPn; ++dp)

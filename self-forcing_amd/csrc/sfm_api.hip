@@ -199,7 +199,7 @@ using namespace sfm;
 
 extern "C" {
 
-int sfm_version(void) { return 4; }
+int sfm_version(void) { return 5; }
 
 const char* sfm_last_error(void) { return g_err; }
 
@@ -255,10 +255,14 @@ static void init_args(const sfm_monarch_desc* desc, const MonarchPlan& pl, Monar
 }
 
 static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
-                            void* workspace, size_t workspace_bytes, void* stream, float* step_ms) {
+                            void* workspace, size_t workspace_bytes, void* stream, float* step_ms, float* stats = nullptr) {
     MonarchPlan pl;
     int rc = plan_monarch(desc, &pl);
     if (rc) return rc;
+    if (stats && (!pl.mfma || pl.iter)) {
+        set_error("row statistics come from the MFMA forward only (16-bit tensors, head_dim 64 or 128, b2 <= 64, num_iters 1)");
+        return SFM_ERR_UNSUPPORTED;
+    }
     if (!q || !k || !v || !out) {
         set_error("q, k, v and out must be non-NULL");
         return SFM_ERR_NULL;
@@ -282,6 +286,8 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
     MonarchArgs a;
     init_args(desc, pl, &a);
     a.q = q; a.k = k; a.v = v; a.out = out;
+    a.stats = stats;
+    a.stats_ld = (uint32_t)((pl.b1 + 31) / 32 * 32);
     const size_t rows = (size_t)pl.na * pl.b2 * pl.r_pad;
     const size_t mat_bytes = rows * desc->D * (pl.mfma ? 2 : 4);
     for (int u0 = 0; u0 < pl.units; u0 += upp) {
@@ -333,6 +339,27 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
 int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
                     void* workspace, size_t workspace_bytes, void* stream) {
     return monarch_fwd_impl(desc, q, k, v, out, workspace, workspace_bytes, stream, nullptr);
+}
+
+int sfm_monarch_stats_bytes(const sfm_monarch_desc* desc, size_t* bytes) {
+    if (!bytes) {
+        set_error("bytes is NULL");
+        return SFM_ERR_NULL;
+    }
+    MonarchPlan pl;
+    int rc = plan_monarch(desc, &pl);
+    if (rc) return rc;
+    *bytes = pl.mfma && !pl.iter ? (size_t)pl.units * pl.na * pl.b2 * ((pl.b1 + 31) / 32 * 32) * sizeof(float) : 0;
+    return SFM_OK;
+}
+
+int sfm_monarch_fwd_stats(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out, float* stats,
+                          void* workspace, size_t workspace_bytes, void* stream) {
+    if (!stats) {
+        set_error("stats is NULL");
+        return SFM_ERR_NULL;
+    }
+    return monarch_fwd_impl(desc, q, k, v, out, workspace, workspace_bytes, stream, nullptr, stats);
 }
 
 int sfm_monarch_fwd_timed(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
@@ -414,8 +441,32 @@ int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t he
     return SFM_OK;
 }
 
+static int monarch_bwd_impl(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* out,
+                            const float* stats, const void* dout, float* dq, void* dk, void* dv, void* workspace,
+                            size_t workspace_bytes, void* stream);
+
 int sfm_monarch_bwd(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* dout,
                     float* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream) {
+    return monarch_bwd_impl(desc, q, k, v, nullptr, nullptr, dout, dq, dk, dv, workspace, workspace_bytes, stream);
+}
+
+int sfm_monarch_bwd_saved(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* out,
+                          const float* stats, const void* dout, float* dq, void* dk, void* dv, void* workspace,
+                          size_t workspace_bytes, void* stream) {
+    if (!out || !stats) {
+        set_error("out and stats must be non-NULL (sfm_monarch_bwd recomputes them)");
+        return SFM_ERR_NULL;
+    }
+    if (!aligned16(out) || (((uintptr_t)stats) & 3)) {
+        set_error("out must be 16-byte aligned, stats 4-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    return monarch_bwd_impl(desc, q, k, v, out, stats, dout, dq, dk, dv, workspace, workspace_bytes, stream);
+}
+
+static int monarch_bwd_impl(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* out,
+                            const float* stats, const void* dout, float* dq, void* dk, void* dv, void* workspace,
+                            size_t workspace_bytes, void* stream) {
     MonarchPlan pl;
     size_t per_unit = 0;
     int rc = plan_bwd(desc, &pl, &per_unit);
@@ -445,6 +496,7 @@ int sfm_monarch_bwd(const sfm_monarch_bwd_desc* desc, const void* q, const void*
         }
         g.p.q = q; g.p.k = k; g.p.v = v;
         g.dout = dout; g.dq = dq; g.dk = dk; g.dv = dv;
+        g.fout = out; g.fstats = stats;
         for (int i = 0; i < 3; ++i) {
             g.dos[i] = desc->fwd.o_stride[i];
             g.dqs[i] = desc->dq_stride[i];

@@ -138,6 +138,8 @@ struct MonarchArgs {
     uint32_t ws_unit, ws_aj, ws_row;
     uint32_t ws_f;   // MFMA step 1 only: rows between consecutive kv block-frames f of one (unit, a, j, k); 0 = b1 * ws_row
     void* rb;        // MFMA step 1 only, optional: the right factor R, 16 bit, 64 values per scratch row (same row index)
+    float* stats;    // MFMA step 2 only, optional: log2-sum-exp of each query row's left-factor logits,
+    uint32_t stats_ld;   // at ((b*H + h) * na*b2 + a*b2 + j) * stats_ld + i
     int unit0;       // first (b*H + h) unit of this pass
     int causal;      // block-causal size in block-frames, 0 = none
     float scale;
@@ -165,6 +167,8 @@ struct MonarchBwdArgs {
     float* dy;               // same layout as p.y
     float* dcl;              // same layout as p.cl: gradient of sum_l R ln R
     int kv_f0, kv_f1;        // kv block-frames whose dK / dV are wanted
+    const void* fout;        // optional, with fstats: the forward's output (layout of dout) and its row statistics
+    const float* fstats;     // (MonarchArgs::stats of that forward, row pitch round_up(b1, 32))
 };
 
 // Optional timing hooks: ev[0] is recorded before step 1, ev[1] between the steps, ev[2] after step 2.
@@ -186,7 +190,8 @@ int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_
 bool monarch_bwd_left_supported(int dtype, int D, int b1);
 int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* qa,
                             const void* doa, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy,
-                            float* dc, void* ds2, int ds2_ld, hipStream_t stream);
+                            float* dc, void* ds2, int ds2_ld, const void* oa, const float* stats, int stats_ld, int unit0,
+                            hipStream_t stream);
 // dq rows (caller's layout) = s dS2 Kbar per (unit, a, j) + the right factor's dQk; same limits as the left kernel
 int launch_monarch_bwd_dqa(int dtype, int D, int n, int b1, int b2, int AJ, int nf, float scale, const void* kbar, const void* ds2,
                            int ds2_ld, const float* dqk, float* dq, const int64_t* dqs, const TokMap& map, int H, int unit0,

@@ -20,7 +20,8 @@ ERR_NAMES = {
 SYMBOLS = [
     "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
-    "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm", "sfm_probe_mfma_bf16", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_last_error", "sfm_version",
+    "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm",
+    "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_probe_mfma_bf16", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_last_error", "sfm_version",
 ]
 
 
@@ -89,6 +90,9 @@ def load():
                                           C.POINTER(C.c_float), C.POINTER(C.c_float)]
     lib.sfm_monarch_bwd_workspace_bytes.argtypes = [C.POINTER(MonarchBwdDesc), C.c_int32, C.POINTER(C.c_size_t)]
     lib.sfm_monarch_bwd.argtypes = [C.POINTER(MonarchBwdDesc), P, P, P, P, P, P, P, P, C.c_size_t, P]
+    lib.sfm_monarch_stats_bytes.argtypes = [C.POINTER(MonarchDesc), C.POINTER(C.c_size_t)]
+    lib.sfm_monarch_fwd_stats.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, P, C.c_size_t, P]
+    lib.sfm_monarch_bwd_saved.argtypes = [C.POINTER(MonarchBwdDesc), P, P, P, P, P, P, P, P, P, P, C.c_size_t, P]
     lib.sfm_kv_cache_write.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(Tiling), P, P, S3, P, P,
                                        S3, I64, I64, I64, P]
     lib.sfm_monarch_attn_with_kv_cache.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, S3, I64, I64, P, P,

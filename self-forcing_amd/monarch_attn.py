@@ -69,16 +69,72 @@ def _from_block_order(x, f_tied, h_reduce, w_reduce, h, w):
     return x.permute(0, 1, 4, 2, 5, 3, 6, 7, 8).reshape(B, n, H, D)
 
 
-def _monarch_bwd(q, k, v, dout, tiling, sm_scale, kv_block_order, cbf, kv_f0=0, kv_f1=None, heads_per_pass=0):
-    """Raw call of sfm_monarch_bwd: returns (dq float32, dk, dv); dk, dv cover kv block-frames [kv_f0, kv_f1) in
-    the row order of k."""
+def _causal_block_frames(q, k, tiling, block_causal_size, num_iters=1):
+    """Block-causal size in tokens -> block-frames, with the reference's checks (monarch_attn.py:1485-1491)."""
+    if block_causal_size is None:
+        return 0
+    f_tied, h_reduce, w_reduce, h, w = tiling
+    per_block = f_tied * (h // h_reduce) * (w // w_reduce)
+    if q.shape[1] % block_causal_size:
+        raise ValueError(f"block_causal_size ({block_causal_size}) must divide sequence length ({q.shape[1]})")
+    if k.shape[1] != q.shape[1]:
+        raise ValueError("causal attention needs kv length equal to q length")
+    if block_causal_size % per_block:
+        raise ValueError("block_causal_size must align with Monarch block sizes")
+    if num_iters != 1:
+        raise ValueError("causal currently only supported for num_iters=1")
+    return block_causal_size // per_block
+
+
+def kv_cache_write(new_k, new_v, k_cache, v_cache, start_idx, end_idx, f_tied, h_reduce, w_reduce, h, w):
+    """new_k / new_v (token order) into k_cache / v_cache[:, start_idx:end_idx] in Monarch block order
+    (monarch_attn.py:1784-1785, 1230-1231)."""
+    if new_k.stride() != new_v.stride():
+        new_k, new_v = new_k.contiguous(), new_v.contiguous()
+    if k_cache.stride() != v_cache.stride():
+        raise ValueError("k_cache and v_cache must share their strides")
+    B, _, H, D = new_k.shape
+    with torch.cuda.device(new_k.device):
+        _l.check(_l.load().sfm_kv_cache_write(_DT[new_k.dtype], B, H, D, C.byref(_l.Tiling(f_tied, h_reduce, w_reduce, h, w)),
+                                              new_k.data_ptr(), new_v.data_ptr(), _l.strides3(new_k), k_cache.data_ptr(),
+                                              v_cache.data_ptr(), _l.strides3(k_cache), k_cache.shape[1], start_idx, end_idx,
+                                              _stream(new_k)))
+
+
+def _monarch_fwd_stats(q, k, v, tiling, sm_scale, kv_block_order, cbf, heads_per_pass=0):
+    """Forward for autograd: returns (out, stats) where stats is the opaque row-statistics tensor that
+    sfm_monarch_bwd_saved takes, or None when the forward that runs for these tensors produces none (the
+    reference's forward keeps z and z_lse the same way, monarch_attn.py:1309-1317)."""
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    d = _desc(q, k, v, out, *tiling, sm_scale, kv_block_order, cbf, 1)
+    n = C.c_size_t(0)
+    _l.check(_l.load().sfm_monarch_stats_bytes(C.byref(d), C.byref(n)))
+    nbytes = monarch_workspace_bytes(d, heads_per_pass)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    stats = torch.empty(n.value // 4, dtype=torch.float32, device=q.device) if n.value else None
+    with torch.cuda.device(q.device):
+        if stats is None:
+            _l.check(_l.load().sfm_monarch_fwd(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                               ws.data_ptr(), nbytes, _stream(q)))
+        else:
+            _l.check(_l.load().sfm_monarch_fwd_stats(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                                     stats.data_ptr(), ws.data_ptr(), nbytes, _stream(q)))
+    return out, stats
+
+
+def _monarch_bwd(q, k, v, dout, tiling, sm_scale, kv_block_order, cbf, kv_f0=0, kv_f1=None, heads_per_pass=0, out=None,
+                 stats=None):
+    """Raw call of sfm_monarch_bwd (or sfm_monarch_bwd_saved when the forward's `out` and `stats` are given): returns
+    (dq float32, dk, dv); dk, dv cover kv block-frames [kv_f0, kv_f1) in the row order of k."""
     f_tied, h_reduce, w_reduce, h, w = tiling
     per_frame = f_tied * (h // h_reduce) * (w // w_reduce)
     nf = k.shape[1] // per_frame
     if kv_f1 is None:
         kv_f1 = nf
-    if dout.stride(3) != 1:
+    if dout.stride(3) != 1 or (out is not None and dout.stride() != out.stride()):
         dout = dout.contiguous()
+    if out is not None and out.stride() != dout.stride():
+        out = out.contiguous()
     dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
     dk = torch.empty((k.shape[0], (kv_f1 - kv_f0) * per_frame, k.shape[2], k.shape[3]), dtype=k.dtype, device=k.device)
     dv = torch.empty_like(dk)
@@ -91,9 +147,14 @@ def _monarch_bwd(q, k, v, dout, tiling, sm_scale, kv_block_order, cbf, kv_f0=0, 
     _l.check(_l.load().sfm_monarch_bwd_workspace_bytes(C.byref(bd), heads_per_pass, C.byref(n)))
     ws = torch.empty(n.value, dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):
-        _l.check(_l.load().sfm_monarch_bwd(C.byref(bd), q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(),
-                                           dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), n.value,
-                                           _stream(q)))
+        if out is None or stats is None:
+            _l.check(_l.load().sfm_monarch_bwd(C.byref(bd), q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(),
+                                               dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), n.value,
+                                               _stream(q)))
+        else:
+            _l.check(_l.load().sfm_monarch_bwd_saved(C.byref(bd), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                                     stats.data_ptr(), dout.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                                     dv.data_ptr(), ws.data_ptr(), n.value, _stream(q)))
     return dq, dk, dv
 
 
@@ -102,20 +163,27 @@ class _MonarchFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, tiling, sm_scale, block_causal_size, heads_per_pass, kv_block_order):
-        out = monarch_attn(q, k, v, *tiling, sm_scale=sm_scale, block_causal_size=block_causal_size,
-                           heads_per_pass=heads_per_pass, kv_block_order=kv_block_order)
-        ctx.save_for_backward(q, k, v)
-        ctx.cfg = (tiling, sm_scale, block_causal_size, kv_block_order)
+        cbf = _causal_block_frames(q, k, tiling, block_causal_size)
+        _check4("q", q)
+        _check4("k", k, q.dtype, q.device)
+        _check4("v", v, q.dtype, q.device)
+        if k.stride() != v.stride():
+            k, v = k.contiguous(), v.contiguous()
+        out, stats = _monarch_fwd_stats(q, k, v, tiling, sm_scale, 1 if kv_block_order else 0, cbf, heads_per_pass)
+        ctx.has_stats = stats is not None
+        if stats is not None:
+            ctx.save_for_backward(q, k, v, out, stats)
+        else:
+            ctx.save_for_backward(q, k, v)
+        ctx.cfg = (tiling, sm_scale, cbf, kv_block_order)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v = ctx.saved_tensors
-        tiling, sm_scale, block_causal_size, kv_block_order = ctx.cfg
-        cbf = 0
-        if block_causal_size is not None:
-            cbf = block_causal_size // (tiling[0] * (tiling[3] // tiling[1]) * (tiling[4] // tiling[2]))
-        dq, dk, dv = _monarch_bwd(q, k, v, dout, tiling, sm_scale, 1 if kv_block_order else 0, cbf)
+        q, k, v, *kept = ctx.saved_tensors
+        out, stats = kept if ctx.has_stats else (None, None)
+        tiling, sm_scale, cbf, kv_block_order = ctx.cfg
+        dq, dk, dv = _monarch_bwd(q, k, v, dout, tiling, sm_scale, 1 if kv_block_order else 0, cbf, out=out, stats=stats)
         return dq.to(q.dtype), dk, dv, None, None, None, None, None
 
 
@@ -127,25 +195,37 @@ class _MonarchCacheFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, tiling, sm_scale, grad_only_new_kv,
                 heads_per_pass):
-        out = monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, *tiling,
-                                         sm_scale=sm_scale, heads_per_pass=heads_per_pass)
-        ctx.save_for_backward(q, k_cache, v_cache)
+        _check4("q", q)
+        for name, t in (("k_cache", k_cache), ("v_cache", v_cache), ("new_k", new_k), ("new_v", new_v)):
+            _check4(name, t, q.dtype, q.device)
+        if k_cache.shape != v_cache.shape or new_k.shape != new_v.shape:
+            raise ValueError("k/v shapes differ")
+        if new_k.shape[1] != end_idx - start_idx:
+            raise ValueError(f"new_k holds {new_k.shape[1]} tokens but end_idx - start_idx = {end_idx - start_idx}")
+        kv_cache_write(new_k, new_v, k_cache, v_cache, start_idx, end_idx, *tiling)
+        out, stats = _monarch_fwd_stats(q, k_cache, v_cache, tiling, sm_scale, 1, 0, heads_per_pass)
+        ctx.has_stats = stats is not None
+        if stats is not None:
+            ctx.save_for_backward(q, k_cache, v_cache, out, stats)
+        else:
+            ctx.save_for_backward(q, k_cache, v_cache)
         ctx.cfg = (start_idx, end_idx, tiling, sm_scale, grad_only_new_kv)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k_cache, v_cache = ctx.saved_tensors
+        q, k_cache, v_cache, *kept = ctx.saved_tensors
+        out, stats = kept if ctx.has_stats else (None, None)
         start_idx, end_idx, tiling, sm_scale, grad_only_new_kv = ctx.cfg
         f_tied, h_reduce, w_reduce, h, w = tiling
         per_frame = f_tied * (h // h_reduce) * (w // w_reduce)
         if grad_only_new_kv:
             dq, dk, dv = _monarch_bwd(q, k_cache, v_cache, dout, tiling, sm_scale, 1, 0, start_idx // per_frame,
-                                      end_idx // per_frame)
+                                      end_idx // per_frame, out=out, stats=stats)
             dk_cache = dv_cache = None
             dk_new, dv_new = dk, dv
         else:
-            dq, dk_cache, dv_cache = _monarch_bwd(q, k_cache, v_cache, dout, tiling, sm_scale, 1, 0)
+            dq, dk_cache, dv_cache = _monarch_bwd(q, k_cache, v_cache, dout, tiling, sm_scale, 1, 0, out=out, stats=stats)
             dk_new, dv_new = dk_cache[:, start_idx:end_idx], dv_cache[:, start_idx:end_idx]
         dk_new = _from_block_order(dk_new, *tiling)
         dv_new = _from_block_order(dv_new, *tiling)
@@ -210,18 +290,7 @@ def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block
         k, v = k.contiguous(), v.contiguous()
     if sm_scale is None:
         sm_scale = q.shape[-1] ** -0.5
-    cbf = 0
-    if block_causal_size is not None:
-        per_block = f_tied * (h // h_reduce) * (w // w_reduce)
-        if q.shape[1] % block_causal_size:
-            raise ValueError(f"block_causal_size ({block_causal_size}) must divide sequence length ({q.shape[1]})")
-        if k.shape[1] != q.shape[1]:
-            raise ValueError("causal attention needs kv length equal to q length")
-        if block_causal_size % per_block:
-            raise ValueError("block_causal_size must align with Monarch block sizes")
-        cbf = block_causal_size // per_block
-        if num_iters != 1:
-            raise ValueError("causal currently only supported for num_iters=1")
+    cbf = _causal_block_frames(q, k, (f_tied, h_reduce, w_reduce, h, w), block_causal_size, num_iters)
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     d = _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1 if kv_block_order else 0, cbf, num_iters)
     nbytes = monarch_workspace_bytes(d, heads_per_pass)

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 9 and set(names) == set(L.SYMBOLS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sfm_version() == 4
+    assert lib.sfm_version() == 5
 
 
 def test_struct_sizes_match_header_layout():

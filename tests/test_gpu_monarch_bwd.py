@@ -147,6 +147,32 @@ def test_16bit_gradients_across_the_fused_kernels_limits(h, w, Fq, Fk, D, causal
     _close(vd.grad, vr.grad, dtype)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_backward_with_and_without_the_forwards_saved_tensors(causal):
+    """sfm_monarch_bwd recomputes the left factor's row statistics; sfm_monarch_bwd_saved takes them (and the output)
+    from sfm_monarch_fwd_stats.  Both against the float64 oracle, and the forward with statistics against the plain one."""
+    h, w, F, H, D = 4, 52, 3, 2, 128
+    dtype = torch.bfloat16
+    q0, do = (randn((1, F * h * w, H, D), 160 + i, dtype) for i in range(2))
+    k0, v0 = (randn((1, F * h * w, H, D), 162 + i, dtype) for i in range(2))
+    kw = {"block_causal_size": h * w} if causal else {}
+    qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
+    monarch.monarch_attn(qr, kr, vr, 1, 1, 1, h, w, **kw).backward(do.double())
+    qd, kd, vd, dod = q0.to(DEV), k0.to(DEV), v0.to(DEV), do.to(DEV)
+    tiling, cbf = (1, 1, 1, h, w), 1 if causal else 0
+    out, stats = mattn._monarch_fwd_stats(qd, kd, vd, tiling, D ** -0.5, 0, cbf)
+    assert stats is not None and stats.dtype == torch.float32
+    assert torch.equal(out, mattn.monarch_attn(qd, kd, vd, *tiling, **kw))
+    for kept in ({}, {"out": out, "stats": stats}):
+        dq, dk, dv = mattn._monarch_bwd(qd, kd, vd, dod, tiling, D ** -0.5, 0, cbf, **kept)
+        _close(dq, qr.grad, dtype)
+        _close(dk, kr.grad, dtype)
+        _close(dv, vr.grad, dtype)
+    # fp32 tensors run the forward without statistics: the autograd path falls back to recomputing
+    out32, stats32 = mattn._monarch_fwd_stats(qd.float(), kd.float(), vd.float(), tiling, D ** -0.5, 0, cbf)
+    assert stats32 is None
+
+
 def test_descriptor_errors():
     q = randn((1, 64, 1, 32), 140, torch.float32).to(DEV).requires_grad_(True)
     with pytest.raises(NotImplementedError):
