@@ -66,14 +66,14 @@ extern "C" int sfm_probe_mfma_bf16(int32_t iters, void* stream, float* tflops) {
         return SFM_ERR_HIP;
     }
     hipLaunchKernelGGL(mfma_probe_kernel, dim3(wgs), dim3(256), 0, st, iters);          // warm-up
-    hipEventRecord(e0, st);
+    (void)hipEventRecord(e0, st);
     hipLaunchKernelGGL(mfma_probe_kernel, dim3(wgs), dim3(256), 0, st, iters);
-    hipEventRecord(e1, st);
+    (void)hipEventRecord(e1, st);
     hipError_t e = hipEventSynchronize(e1);
     float ms = 0.f;
     if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     if (e != hipSuccess || ms <= 0.f) {
         set_error("sfm_probe_mfma_bf16: %s", hipGetErrorString(e));
         return SFM_ERR_HIP;

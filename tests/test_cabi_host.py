@@ -106,6 +106,33 @@ def test_monarch_fwd_pointer_and_workspace_checks():
     assert lib.sfm_monarch_fwd(None, fake, fake, fake, fake, fake, need, None) == -1
 
 
+def test_row_statistics_size_and_argument_checks():
+    """sfm_monarch_stats_bytes: one float per (unit, a, j) and block row, rows padded to 32; 0 where the forward that
+    would run keeps none.  The entry points that write / read them refuse NULL and misaligned pointers first."""
+    lib = L.load()
+    n = C.c_size_t(1)
+    assert lib.sfm_monarch_stats_bytes(C.byref(_desc()), C.byref(n)) == 0 and n.value == 2 * 3 * 52 * 32 * 4
+    assert lib.sfm_monarch_stats_bytes(C.byref(_desc(dtype=L.SFM_F32)), C.byref(n)) == 0 and n.value == 0
+    assert lib.sfm_monarch_stats_bytes(C.byref(_desc(num_iters=2)), C.byref(n)) == 0 and n.value == 0
+    assert lib.sfm_monarch_stats_bytes(C.byref(_desc()), None) == -1
+    d = _desc()
+    _, need = _ws(d, 1)
+    fake = 0x10000
+    assert lib.sfm_monarch_fwd_stats(C.byref(d), fake, fake, fake, fake, None, fake, need, None) == -1
+    assert lib.sfm_monarch_fwd_stats(C.byref(_desc(dtype=L.SFM_F32)), fake, fake, fake, fake, fake, fake, 1 << 40, None) == -9
+    bd = L.MonarchBwdDesc()
+    bd.fwd = d
+    bd.dq_stride = (C.c_int64 * 3)(d.q_tokens * 256, 256, 128)
+    bd.dkv_stride = (C.c_int64 * 3)(d.kv_tokens * 256, 256, 128)
+    bd.kv_grad_frame_start, bd.kv_grad_frame_end = 0, 21
+    args = [fake] * 4
+    assert lib.sfm_monarch_bwd_saved(C.byref(bd), fake, fake, fake, None, fake, *args, fake, 1 << 40, None) == -1
+    assert lib.sfm_monarch_bwd_saved(C.byref(bd), fake, fake, fake, fake, None, *args, fake, 1 << 40, None) == -1
+    assert lib.sfm_monarch_bwd_saved(C.byref(bd), fake, fake, fake, fake + 2, fake, *args, fake, 1 << 40, None) == -7
+    assert lib.sfm_monarch_bwd_saved(C.byref(bd), fake, fake, fake, fake, fake + 2, *args, fake, 1 << 40, None) == -7
+    assert lib.sfm_monarch_bwd_saved(C.byref(bd), fake, fake, fake, fake, fake, None, fake, fake, fake, fake, 1 << 40, None) == -1
+
+
 def test_kv_cache_op_range_checks_happen_before_any_write():
     lib = L.load()
     d = _desc()
