@@ -395,36 +395,62 @@ struct Layout {
     size_t Qk, Qa, dOa, Oa, Kk, Vk, S1f, dRb, Rb, dS1, Kbar, Y, dKbar, dY, c, dc, S2f, dLmf, L, dS2, dQa, dQk, dKk, dVk, total;
 };
 
-Layout make_layout(const MonarchArgs& p, int n, size_t e) {
+// dtype code of the fused kernels for operand type E, or -1 (fp32 operands stay on the GEMMs)
+template <typename E> constexpr int left_dtype() { return -1; }
+template <> constexpr int left_dtype<BF16>() { return SFM_BF16; }
+template <> constexpr int left_dtype<F16>() { return SFM_F16; }
+
+// Which parts of the chain run as fused kernels: decided by shapes, strides and (for measurements) the environment,
+// so that the workspace query and the run agree.
+struct Parts {
+    bool left;     // 4-7: statistics and gradients of the left factor without the [i x r] matrices in memory
+    bool fwd;      // 1-3: the forward's MFMA step 1 recomputes Kbar, Y, c and R straight into the scratch ([t][aj] rows)
+    bool dqa;      // 8 and the scatter of dq: dQ of the left factor in its own kernel, which also adds the right factor's part
+    bool right;    // 9, the right factor's softmax backward, 11-13 and the scatter of dk / dv in one kernel per tile t
+};
+
+Parts make_parts(const MonarchArgs& p, int dtype, const int64_t* dks) {
+    Parts f;
+    const bool h16 = dtype == SFM_BF16 || dtype == SFM_F16;
+    f.left = h16 && monarch_bwd_left_supported(dtype, p.D, p.b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
+    f.fwd = f.left && monarch_mfma_supported(dtype, p.D, p.b2) && getenv("SFM_BWD_FWD_GEMM") == nullptr;
+    f.dqa = f.left && getenv("SFM_BWD_DQA_GEMM") == nullptr;
+    const bool direct_ok = (dks[0] | dks[1] | dks[2] | p.vs[0] | p.vs[1] | p.vs[2]) % 8 == 0;      // 16-byte rows of v, dk, dv
+    f.right = f.fwd && direct_ok && monarch_bwd_right_supported(dtype, p.D, p.b2, p.na * p.b2) &&
+              getenv("SFM_BWD_RIGHT_GEMM") == nullptr;
+    return f;
+}
+
+Layout make_layout(const MonarchArgs& p, int n, size_t e, const Parts& f) {
     const size_t AJ = (size_t)p.na * p.b2, RR = (size_t)p.nf * p.b1, D = p.D;
     const size_t MQ = (size_t)p.b1 * AJ, MK = (size_t)p.b1 * p.nf * p.b2, NL = (size_t)p.nf * p.b2;
     Layout l;
     size_t o = 0;
-    auto take = [&](size_t bytes) { size_t at = o; o += align256(bytes); return at; };
-    l.Qk = take(n * MQ * D * e);
-    l.Qa = take(n * MQ * D * e);
-    l.dOa = take(n * MQ * D * e);
-    l.Oa = take(n * MQ * D * e);
-    l.Kk = take(n * MK * D * e);
-    l.Vk = take(n * MK * D * e);
-    l.S1f = take(n * p.b1 * AJ * NL * 4);
-    l.dRb = take(n * p.b1 * AJ * NL * 4);
-    l.Rb = take(n * p.b1 * AJ * p.nf * (size_t)(p.b2 > 64 ? p.b2 : 64) * e);      // row pitch 64 when step 1 of the forward writes it
-    l.dS1 = take(n * p.b1 * AJ * NL * e);
-    l.Kbar = take(n * AJ * RR * D * e);
-    l.Y = take(n * AJ * RR * D * e);
-    l.dKbar = take(n * AJ * RR * D * e);
-    l.dY = take(n * AJ * RR * D * e);
-    l.c = take(n * AJ * RR * 4);
-    l.dc = take(n * AJ * RR * 4);
-    l.S2f = take(n * AJ * p.b1 * RR * 4);
-    l.dLmf = take(n * AJ * p.b1 * RR * 4);
-    l.L = take(n * AJ * p.b1 * RR * e);
-    l.dS2 = take(n * AJ * p.b1 * ((RR + 7) / 8 * 8) * e);                          // rows padded to 8 for the fused kernels
-    l.dQa = take(n * MQ * D * 4);
-    l.dQk = take(n * MQ * D * 4);
-    l.dKk = take(n * MK * D * 4);
-    l.dVk = take(n * MK * D * 4);
+    auto take = [&](bool used, size_t bytes) { size_t at = o; o += used ? align256(bytes) : 0; return at; };
+    l.Qk = take(true, n * MQ * D * e);
+    l.Qa = take(true, n * MQ * D * e);
+    l.dOa = take(true, n * MQ * D * e);
+    l.Oa = take(f.left, n * MQ * D * e);
+    l.Kk = take(true, n * MK * D * e);
+    l.Vk = take(!f.right, n * MK * D * e);
+    l.S1f = take(!f.fwd, n * p.b1 * AJ * NL * 4);
+    l.dRb = take(!f.right, n * p.b1 * AJ * NL * 4);
+    l.Rb = take(true, n * p.b1 * AJ * p.nf * (size_t)(p.b2 > 64 ? p.b2 : 64) * e);      // row pitch 64 when step 1 of the forward writes it
+    l.dS1 = take(true, n * p.b1 * AJ * NL * e);
+    l.Kbar = take(true, n * AJ * RR * D * e);
+    l.Y = take(true, n * AJ * RR * D * e);
+    l.dKbar = take(true, n * AJ * RR * D * e);
+    l.dY = take(true, n * AJ * RR * D * e);
+    l.c = take(true, n * AJ * RR * 4);
+    l.dc = take(true, n * AJ * RR * 4);
+    l.S2f = take(!f.left, n * AJ * p.b1 * RR * 4);
+    l.dLmf = take(!f.left, n * AJ * p.b1 * RR * 4);
+    l.L = take(!f.left, n * AJ * p.b1 * RR * e);
+    l.dS2 = take(true, n * AJ * p.b1 * ((RR + 7) / 8 * 8) * e);                         // rows padded to 8 for the fused kernels
+    l.dQa = take(!f.dqa, n * MQ * D * 4);
+    l.dQk = take(true, n * MQ * D * 4);
+    l.dKk = take(!f.right, n * MK * D * 4);
+    l.dVk = take(!f.right, n * MK * D * 4);
     l.total = o;
     return l;
 }
@@ -458,17 +484,13 @@ void gemm(Ctx& cx, bool ta, bool tb, int M, int N, int K, float alpha, float bet
     }
 }
 
-// dtype code of the fused left-factor kernel for operand type E, or -1 (fp32 operands stay on the GEMMs)
-template <typename E> constexpr int left_dtype() { return -1; }
-template <> constexpr int left_dtype<BF16>() { return SFM_BF16; }
-template <> constexpr int left_dtype<F16>() { return SFM_F16; }
-
 template <typename E>
 int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     typedef typename El<E>::type T;
     const MonarchArgs& p = g.p;
     const size_t e = sizeof(T);
-    const Layout lay = make_layout(p, n, e);
+    const Parts parts = make_parts(p, left_dtype<E>() >= 0 ? left_dtype<E>() : SFM_F32, g.dks);
+    const Layout lay = make_layout(p, n, e, parts);
     char* ws = (char*)workspace;
     Ctx cx{blas_handle(stream), ws, 0};
     if (!cx.h) {
@@ -482,18 +504,13 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     const rocblas_datatype tE = El<E>::kBlas, tF = rocblas_datatype_f32_r;
 
     const int64_t nseg = (int64_t)n * b1 * AJ * nf;
-    const bool fused_left = left_dtype<E>() >= 0 && monarch_bwd_left_supported(left_dtype<E>(), D, b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
-    // the forward's MFMA step 1 recomputes Kbar, Y, c and R straight into this scratch ([t][aj] rows)
-    const bool fused_fwd = fused_left && monarch_mfma_supported(left_dtype<E>(), D, b2) && getenv("SFM_BWD_FWD_GEMM") == nullptr;
-    // dQ of the left factor in its own kernel, which also adds the right factor's part and writes the caller's dq
-    const bool fused_dqa = fused_left && getenv("SFM_BWD_DQA_GEMM") == nullptr;
+    const bool fused_left = parts.left, fused_fwd = parts.fwd, fused_dqa = parts.dqa, fused_right = parts.right;
     const int ds2_ld = fused_left ? (RR + 7) / 8 * 8 : RR;
     const int rb_ld = fused_fwd ? 64 : b2;
-    // 9, the right factor's softmax backward, 11, 12, 13 and the scatter of dk / dv in one kernel per tile t
-    const bool direct_ok = (g.dks[0] | g.dks[1] | g.dks[2] | p.vs[0] | p.vs[1] | p.vs[2]) % 8 == 0 &&
-                           ((uintptr_t)g.dk | (uintptr_t)g.dv | (uintptr_t)p.v) % 16 == 0;
-    const bool fused_right = fused_fwd && direct_ok && monarch_bwd_right_supported(left_dtype<E>(), D, b2, AJ) &&
-                             getenv("SFM_BWD_RIGHT_GEMM") == nullptr;
+    if (fused_right && ((uintptr_t)g.dk | (uintptr_t)g.dv | (uintptr_t)p.v) % 16) {
+        set_error("Monarch backward: v, dk and dv must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
     // the forward's output and row statistics, when the caller kept them, save the left factor's first pass
     const bool saved = fused_left && g.fout != nullptr && g.fstats != nullptr;
     // gather q, dout (query map; both row orders) and k, v (key map)
@@ -647,8 +664,8 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
 
 bool monarch_bwd_gemm_available() { return blas_load(); }
 
-size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits) {
-    return make_layout(p, nunits, dtype == SFM_F32 ? 4 : 2).total;
+size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits, const int64_t* dkv_stride) {
+    return make_layout(p, nunits, dtype == SFM_F32 ? 4 : 2, make_parts(p, dtype, dkv_stride)).total;
 }
 
 int launch_monarch_bwd_gemm(const MonarchBwdArgs& g, int dtype, int nunits, void* workspace, hipStream_t stream) {

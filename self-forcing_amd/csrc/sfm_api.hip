@@ -430,8 +430,8 @@ int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t he
         init_args(&desc->fwd, pl, &a);
         int n = heads_per_pass > 0 ? (heads_per_pass > pl.units ? pl.units : heads_per_pass) : pl.units;
         if (heads_per_pass == 0)
-            while (n > 1 && monarch_bwd_gemm_bytes(a, desc->fwd.dtype, n) > ((size_t)7 << 29)) --n;     // 3.5 GiB
-        *bytes = monarch_bwd_gemm_bytes(a, desc->fwd.dtype, n);
+            while (n > 1 && monarch_bwd_gemm_bytes(a, desc->fwd.dtype, n, desc->dkv_stride) > ((size_t)7 << 29)) --n;     // 3.5 GiB
+        *bytes = monarch_bwd_gemm_bytes(a, desc->fwd.dtype, n, desc->dkv_stride);
         return SFM_OK;
     }
     size_t n = heads_per_pass > 0 ? (size_t)heads_per_pass : ((size_t)3 << 30) / per_unit;
@@ -488,10 +488,10 @@ static int monarch_bwd_impl(const sfm_monarch_bwd_desc* desc, const void* q, con
         memset(&g, 0, sizeof(g));
         init_args(&desc->fwd, pl, &g.p);
         int n = pl.units;
-        while (n > 1 && monarch_bwd_gemm_bytes(g.p, desc->fwd.dtype, n) > workspace_bytes) --n;
-        if (monarch_bwd_gemm_bytes(g.p, desc->fwd.dtype, n) > workspace_bytes) {
+        while (n > 1 && monarch_bwd_gemm_bytes(g.p, desc->fwd.dtype, n, desc->dkv_stride) > workspace_bytes) --n;
+        if (monarch_bwd_gemm_bytes(g.p, desc->fwd.dtype, n, desc->dkv_stride) > workspace_bytes) {
             set_error("workspace holds %zu bytes, one (batch, head) unit needs %zu", workspace_bytes,
-                      monarch_bwd_gemm_bytes(g.p, desc->fwd.dtype, 1));
+                      monarch_bwd_gemm_bytes(g.p, desc->fwd.dtype, 1, desc->dkv_stride));
             return SFM_ERR_WORKSPACE;
         }
         g.p.q = q; g.p.k = k; g.p.v = v;

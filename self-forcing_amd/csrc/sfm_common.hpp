@@ -182,7 +182,7 @@ bool monarch_mfma_supported(int dtype, int D, int b2);
 int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
 int launch_monarch_bwd(const MonarchBwdArgs& g, int dtype, int nunits, hipStream_t stream);
 bool monarch_bwd_gemm_available();
-size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits);
+size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits, const int64_t* dkv_stride);
 int launch_monarch_bwd_gemm(const MonarchBwdArgs& g, int dtype, int nunits, void* workspace, hipStream_t stream);
 // step 1 of the MFMA forward alone, with the scratch strides of `a` and, if a.rb is set, the right factor written out
 int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream);

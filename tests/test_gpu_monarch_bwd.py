@@ -173,6 +173,24 @@ def test_backward_with_and_without_the_forwards_saved_tensors(causal):
     assert stats32 is None
 
 
+@pytest.mark.parametrize("switch", ["SFM_BWD_LEFT_GEMM", "SFM_BWD_FWD_GEMM", "SFM_BWD_DQA_GEMM", "SFM_BWD_RIGHT_GEMM"])
+def test_each_fused_part_can_fall_back_to_the_library_chain(switch, monkeypatch):
+    """The measurement switches that put one fused part back on the batched GEMMs + row kernels (what also runs for
+    shapes a fused kernel does not take): same gradients, and the workspace query follows the switch."""
+    monkeypatch.setenv(switch, "1")
+    h, w, F, H, D = 4, 20, 2, 2, 64
+    dtype = torch.bfloat16
+    q0, do = (randn((1, F * h * w, H, D), 170 + i, dtype) for i in range(2))
+    k0, v0 = (randn((1, 3 * h * w, H, D), 172 + i, dtype) for i in range(2))
+    qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
+    monarch.monarch_attn(qr, kr, vr, 1, 1, 1, h, w).backward(do.double())
+    qd, kd, vd = _leaf(q0, DEV), _leaf(k0, DEV), _leaf(v0, DEV)
+    mattn.monarch_attn(qd, kd, vd, 1, 1, 1, h, w).backward(do.to(DEV))
+    _close(qd.grad, qr.grad, dtype)
+    _close(kd.grad, kr.grad, dtype)
+    _close(vd.grad, vr.grad, dtype)
+
+
 def test_descriptor_errors():
     q = randn((1, 64, 1, 32), 140, torch.float32).to(DEV).requires_grad_(True)
     with pytest.raises(NotImplementedError):
