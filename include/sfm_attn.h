@@ -164,6 +164,27 @@ int sfm_full_attention_with_kv_cache(const sfm_dense_desc* desc, const void* q, 
                                      const void* new_k, const void* new_v, const int64_t new_stride[3],
                                      int64_t start_idx, int64_t end_idx, void* out, float* lse, void* stream);
 
+/* Backward of sfm_dense_fwd / sfm_full_attention_with_kv_cache.  Replaces _attn_bwd_preprocess, _attn_bwd and
+ * _attention.backward (attn_patch.py:121-166, 169-302, 354-413): bf16 / fp16, head_dim 64 or 128.
+ *   fwd                 the forward descriptor; o_stride describes both `out` and `dout`
+ *   out, lse            what the forward returned (lse: float32 [B, H, q_tokens], natural log)
+ *   dq                  float32 [B, q_tokens, H, D] (the reference accumulates and returns grad_q in float32, :361, :413)
+ *   dk, dv              tensor dtype, [B, kv_grad_end - kv_grad_start, H, D]: gradients of keys kv_grad_start ..
+ *                       kv_grad_end - 1; a proper sub-range is the reference's grad_only_new_kv (:362-364); an empty
+ *                       range produces dq only
+ *   workspace           sfm_dense_bwd_workspace_bytes (one float per batch, head and query) */
+typedef struct sfm_dense_bwd_desc {
+    sfm_dense_desc fwd;
+    int64_t dq_stride[3];
+    int64_t dkv_stride[3];
+    int64_t kv_grad_start;
+    int64_t kv_grad_end;
+} sfm_dense_bwd_desc;
+
+int sfm_dense_bwd_workspace_bytes(const sfm_dense_bwd_desc* desc, size_t* bytes);
+int sfm_dense_bwd(const sfm_dense_bwd_desc* desc, const void* q, const void* k, const void* v, const void* out, const float* lse,
+                  const void* dout, float* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream);
+
 typedef struct sfm_prologue_desc {
     int32_t dtype;            /* SFM_BF16 | SFM_F16 | SFM_F32 */
     int32_t B, S, H, D;       /* S new tokens (= F*h*w), model dim C = H*D */

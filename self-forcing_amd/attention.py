@@ -25,6 +25,87 @@ def _dense_desc(q, k, v, out, sm_scale):
     return d
 
 
+def _dense_fwd(q, k, v, sm_scale, want_lse):
+    out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty((q.shape[0], q.shape[2], q.shape[1]), dtype=torch.float32, device=q.device) if want_lse else None
+    d = _dense_desc(q, k, v, out, sm_scale)
+    with torch.cuda.device(q.device):
+        _l.check(_l.load().sfm_dense_fwd(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                         lse.data_ptr() if want_lse else None, _stream(q)))
+    return out, lse
+
+
+def _dense_bwd(q, k, v, out, lse, dout, sm_scale, kv0=0, kv1=None):
+    """Raw call of sfm_dense_bwd: (dq float32, dk, dv); dk, dv cover keys [kv0, kv1)."""
+    if kv1 is None:
+        kv1 = k.shape[1]
+    if dout.stride() != out.stride():
+        dout = dout.contiguous()
+        out = out.contiguous()
+    dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    dk = torch.empty((k.shape[0], kv1 - kv0, k.shape[2], k.shape[3]), dtype=k.dtype, device=k.device)
+    dv = torch.empty_like(dk)
+    bd = _l.DenseBwdDesc()
+    bd.fwd = _dense_desc(q, k, v, out, sm_scale)
+    bd.dq_stride = _l.strides3(dq)
+    bd.dkv_stride = _l.strides3(dk)
+    bd.kv_grad_start, bd.kv_grad_end = kv0, kv1
+    n = C.c_size_t(0)
+    _l.check(_l.load().sfm_dense_bwd_workspace_bytes(C.byref(bd), C.byref(n)))
+    ws = torch.empty(n.value, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        _l.check(_l.load().sfm_dense_bwd(C.byref(bd), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                                         dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), n.value,
+                                         _stream(q)))
+    return dq, dk, dv
+
+
+class _DenseFn(torch.autograd.Function):
+    """attention under autograd: keeps q, k, v, the output and its log-sum-exp, as `_attention.forward` does
+    (attn_patch.py:346-351)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, sm_scale):
+        out, lse = _dense_fwd(q, k, v, sm_scale, True)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.sm_scale = sm_scale
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        dq, dk, dv = _dense_bwd(q, k, v, out, lse, dout, ctx.sm_scale)
+        return dq.to(q.dtype), dk, dv, None
+
+
+class _DenseCacheFn(torch.autograd.Function):
+    """full_attention_with_kv_cache under autograd (`_attention`, attn_patch.py:305-413): the caches are written in place
+    and saved by reference; with grad_only_new_kv only the keys written by this call get gradients (:362-364)."""
+
+    @staticmethod
+    def forward(ctx, q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, sm_scale, grad_only_new_kv):
+        out, lse = _dense_cache_fwd(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, sm_scale, True)
+        ctx.save_for_backward(q, k_cache, v_cache, out, lse)
+        ctx.cfg = (start_idx, end_idx, sm_scale, grad_only_new_kv)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k_cache, v_cache, out, lse = ctx.saved_tensors
+        start_idx, end_idx, sm_scale, grad_only_new_kv = ctx.cfg
+        if grad_only_new_kv:
+            dq, dk_new, dv_new = _dense_bwd(q, k_cache, v_cache, out, lse, dout, sm_scale, start_idx, end_idx)
+            dk_cache = dv_cache = None
+        else:
+            dq, dk_cache, dv_cache = _dense_bwd(q, k_cache, v_cache, out, lse, dout, sm_scale)
+            dk_new, dv_new = dk_cache[:, start_idx:end_idx], dv_cache[:, start_idx:end_idx]
+        return dq.to(q.dtype), dk_cache, dv_cache, dk_new, dv_new, None, None, None, None
+
+
+def _needs_grad(*ts):
+    return torch.is_grad_enabled() and any(t.requires_grad for t in ts)
+
+
 def attention(q, k, v, q_lens=None, k_lens=None, dropout_p=0., softmax_scale=None, q_scale=None, causal=False,
               window_size=(-1, -1), deterministic=False, dtype=torch.bfloat16, fa_version=None, return_lse=False):
     """softmax(q k^T * scale) v on [B, L, H, D] tensors; inputs are cast to `dtype` like the reference does."""
@@ -40,20 +121,25 @@ def attention(q, k, v, q_lens=None, k_lens=None, dropout_p=0., softmax_scale=Non
     q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** -0.5
-    out = torch.empty(q.shape, dtype=dtype, device=q.device)
-    lse = torch.empty((q.shape[0], q.shape[2], q.shape[1]), dtype=torch.float32, device=q.device) if return_lse else None
-    d = _dense_desc(q, k, v, out, softmax_scale)
-    with torch.cuda.device(q.device):
-        _l.check(_l.load().sfm_dense_fwd(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
-                                         lse.data_ptr() if return_lse else None, _stream(q)))
+    if _needs_grad(q, k, v):
+        if return_lse:
+            raise NotImplementedError("return_lse is not differentiable")
+        return _DenseFn.apply(q, k, v, softmax_scale)
+    out, lse = _dense_fwd(q, k, v, softmax_scale, return_lse)
     return (out, lse) if return_lse else out
 
 
 def full_attention_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, sm_scale=None,
                                  grad_only_new_kv=False):
     """k_cache/v_cache[:, start_idx:end_idx] = new_k/new_v (in place), then dense attention over the view."""
-    if torch.is_grad_enabled() and (q.requires_grad or new_k.requires_grad or new_v.requires_grad):
-        raise NotImplementedError("forward only: call under torch.no_grad()")
+    if sm_scale is None:
+        sm_scale = q.shape[-1] ** -0.5
+    if _needs_grad(q, k_cache, v_cache, new_k, new_v):
+        return _DenseCacheFn.apply(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, sm_scale, grad_only_new_kv)
+    return _dense_cache_fwd(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, sm_scale, False)[0]
+
+
+def _dense_cache_fwd(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, sm_scale, want_lse):
     _check4("q", q)
     for name, t in (("k_cache", k_cache), ("v_cache", v_cache), ("new_k", new_k), ("new_v", new_v)):
         _check4(name, t, q.dtype, q.device)
@@ -63,12 +149,11 @@ def full_attention_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, e
         raise ValueError("new_k does not hold end_idx - start_idx tokens")
     if new_k.stride() != new_v.stride():
         new_k, new_v = new_k.contiguous(), new_v.contiguous()
-    if sm_scale is None:
-        sm_scale = q.shape[-1] ** -0.5
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    lse = torch.empty((q.shape[0], q.shape[2], q.shape[1]), dtype=torch.float32, device=q.device) if want_lse else None
     d = _dense_desc(q, k_cache, v_cache, out, sm_scale)
     with torch.cuda.device(q.device):
         _l.check(_l.load().sfm_full_attention_with_kv_cache(
             C.byref(d), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), new_k.data_ptr(), new_v.data_ptr(),
-            _l.strides3(new_k), start_idx, end_idx, out.data_ptr(), None, _stream(q)))
-    return out
+            _l.strides3(new_k), start_idx, end_idx, out.data_ptr(), lse.data_ptr() if want_lse else None, _stream(q)))
+    return out, lse

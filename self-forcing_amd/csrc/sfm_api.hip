@@ -720,6 +720,63 @@ int sfm_full_attention_with_kv_cache(const sfm_dense_desc* desc, const void* q, 
     return launch_dense(*desc, q, k_cache, v_cache, out, lse, (hipStream_t)stream);
 }
 
+static int check_dense_bwd(const sfm_dense_bwd_desc* bd) {
+    if (!bd) {
+        set_error("desc is NULL");
+        return SFM_ERR_NULL;
+    }
+    int rc = check_dense(&bd->fwd);
+    if (rc) return rc;
+    if (!dense_bwd_supported(bd->fwd.dtype, bd->fwd.D)) {
+        set_error("dense backward: bf16 / fp16 tensors with head_dim 64 or 128 only");
+        return SFM_ERR_UNSUPPORTED;
+    }
+    if (bd->kv_grad_start < 0 || bd->kv_grad_end > bd->fwd.kv_tokens || bd->kv_grad_start > bd->kv_grad_end) {
+        set_error("kv gradient range [%lld, %lld) outside [0, %d)", (long long)bd->kv_grad_start, (long long)bd->kv_grad_end,
+                  bd->fwd.kv_tokens);
+        return SFM_ERR_RANGE;
+    }
+    if ((rc = check_strides("dq", bd->dq_stride, bd->fwd.q_tokens, bd->fwd.H, bd->fwd.D, bd->fwd.B, 4))) return rc;
+    if (bd->kv_grad_end > bd->kv_grad_start &&
+        (rc = check_strides("dk/dv", bd->dkv_stride, bd->kv_grad_end - bd->kv_grad_start, bd->fwd.H, bd->fwd.D, bd->fwd.B, 2)))
+        return rc;
+    return SFM_OK;
+}
+
+int sfm_dense_bwd_workspace_bytes(const sfm_dense_bwd_desc* desc, size_t* bytes) {
+    if (!bytes) {
+        set_error("bytes is NULL");
+        return SFM_ERR_NULL;
+    }
+    int rc = check_dense_bwd(desc);
+    if (rc) return rc;
+    *bytes = ((size_t)desc->fwd.B * desc->fwd.H * desc->fwd.q_tokens * sizeof(float) + 255) / 256 * 256;
+    return SFM_OK;
+}
+
+int sfm_dense_bwd(const sfm_dense_bwd_desc* desc, const void* q, const void* k, const void* v, const void* out, const float* lse,
+                  const void* dout, float* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_dense_bwd(desc);
+    if (rc) return rc;
+    const bool want_kv = desc->kv_grad_end > desc->kv_grad_start;
+    if (!q || !k || !v || !out || !lse || !dout || !dq || (want_kv && (!dk || !dv))) {
+        set_error("q, k, v, out, lse, dout, dq (and dk, dv for a non-empty key range) must be non-NULL");
+        return SFM_ERR_NULL;
+    }
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(dout) || !aligned16(dq) ||
+        !aligned16(dk) || !aligned16(dv) || (((uintptr_t)lse) & 3)) {
+        set_error("tensors must be 16-byte aligned (lse: 4-byte)");
+        return SFM_ERR_ALIGN;
+    }
+    const size_t need = (size_t)desc->fwd.B * desc->fwd.H * desc->fwd.q_tokens * sizeof(float);
+    if (!workspace || (((uintptr_t)workspace) & 255) || workspace_bytes < need) {
+        set_error("workspace must be non-NULL, 256-byte aligned and hold at least %zu bytes", need);
+        return SFM_ERR_WORKSPACE;
+    }
+    return launch_dense_bwd(desc->fwd, desc->dq_stride, desc->dkv_stride, desc->kv_grad_start, desc->kv_grad_end, q, k, v, out, lse,
+                            dout, dq, dk, dv, (float*)workspace, (hipStream_t)stream);
+}
+
 int sfm_qk_prologue(const sfm_prologue_desc* d, const void* xq, const void* xk, const void* xv, const void* wq,
                     const void* wk, const double* rope_cos_sin, int32_t rope_max_pos, void* q_out, void* k_cache,
                     void* v_cache, void* stream) {

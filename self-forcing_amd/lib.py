@@ -21,7 +21,7 @@ SYMBOLS = [
     "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
     "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm",
-    "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_probe_mfma_bf16", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_last_error", "sfm_version",
+    "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_dense_bwd_workspace_bytes", "sfm_dense_bwd", "sfm_probe_mfma_bf16", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_last_error", "sfm_version",
 ]
 
 
@@ -57,6 +57,11 @@ class DenseDesc(C.Structure):
                 ("o_stride", C.c_int64 * 3)]
 
 
+class DenseBwdDesc(C.Structure):
+    _fields_ = [("fwd", DenseDesc), ("dq_stride", C.c_int64 * 3), ("dkv_stride", C.c_int64 * 3),
+                ("kv_grad_start", C.c_int64), ("kv_grad_end", C.c_int64)]
+
+
 class PrologueDesc(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("B", C.c_int32), ("S", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
                 ("F", C.c_int32), ("h", C.c_int32), ("w", C.c_int32), ("start_frame", C.c_int32),
@@ -90,6 +95,8 @@ def load():
                                           C.POINTER(C.c_float), C.POINTER(C.c_float)]
     lib.sfm_monarch_bwd_workspace_bytes.argtypes = [C.POINTER(MonarchBwdDesc), C.c_int32, C.POINTER(C.c_size_t)]
     lib.sfm_monarch_bwd.argtypes = [C.POINTER(MonarchBwdDesc), P, P, P, P, P, P, P, P, C.c_size_t, P]
+    lib.sfm_dense_bwd_workspace_bytes.argtypes = [C.POINTER(DenseBwdDesc), C.POINTER(C.c_size_t)]
+    lib.sfm_dense_bwd.argtypes = [C.POINTER(DenseBwdDesc), P, P, P, P, P, P, P, P, P, P, C.c_size_t, P]
     lib.sfm_monarch_stats_bytes.argtypes = [C.POINTER(MonarchDesc), C.POINTER(C.c_size_t)]
     lib.sfm_monarch_fwd_stats.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, P, C.c_size_t, P]
     lib.sfm_monarch_bwd_saved.argtypes = [C.POINTER(MonarchBwdDesc), P, P, P, P, P, P, P, P, P, P, C.c_size_t, P]
