@@ -185,24 +185,62 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (t + 1 < nt) stage(t + 1);
         const char* kt = lds + (t & 1) * 2 * T::kBytes;
         const char* vt = kt + T::kBytes;
+        // Four stages per tile, each a run of MFMAs with its A operands read two ahead (ring) and a slice of the softmax
+        // backward of the half tile before it pinned beside every MFMA:
+        //   1  logits and dP of keys 0..31           2  those of keys 32..63 | softmax backward of keys 0..31
+        //   3  dQ^T += K^T dS of keys 0..31 | softmax backward of keys 32..63          4  dQ^T += K^T dS of keys 32..63
+        constexpr int NA = 2 * T::DS, NO = 2 * T::DT;       // MFMAs of a half's products / of a half's output
+        constexpr int VA = 16 / NA, VO = 16 / NO;           // values of the softmax backward beside each of them
         f32x16 s[2], dp[2];
-        tile_products<E, D>(kt, vt, a_off, qb, gb, s, dp);
-        u32x4 pb[4];
+        u32x4 pb[4], ring[4];
+        const bool ragged = 64 * t + 64 > p.Skv;            // uniform: only the last tile can hold keys past the end
+        auto read_prod = [&](int tl, int j) {               // j even: K rows for the logits, odd: V rows for dP
+            return *(const u32x4*)(((j & 1) ? vt : kt) + tl * 32 * T::kPitch + (a_off ^ (uint32_t)((j >> 1) << 5)));
+        };
+        auto read_out = [&](int tl, int j) { return tile_tr<D>(kt, tr[j % T::DT][0], tr[j % T::DT][1], 2 * tl + j / T::DT); };
+        auto soft = [&](int tl, int v) {
+            float pv = fast_exp2(fmaf(s[tl][v], sc2, -lse2));
+            if (ragged) pv = 64 * t + 32 * tl + 8 * (v >> 2) + 4 * hf + (v & 3) < p.Skv ? pv : 0.f;
+            s[tl][v] = pv * (dp[tl][v] - dl);               // dS^T[l, i]
+            if (v & 1) pb[2 * tl + (v >> 3)][(v >> 1) & 3] = pack2<E>(s[tl][v - 1], s[tl][v]);
+        };
 #pragma unroll
-        for (int tl = 0; tl < 2; ++tl) {
+        for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int l = 64 * t + 32 * tl + 8 * (v >> 2) + 4 * hf + (v & 3);
-                const float pv = l < p.Skv ? fast_exp2(s[tl][v] * sc2 - lse2) : 0.f;
-                s[tl][v] = pv * (dp[tl][v] - dl);           // dS^T[l, i]
-            }
-            pack_steps<E>(s[tl], pb[2 * tl], pb[2 * tl + 1]);
+            for (int v = 0; v < 16; ++v) s[tl][v] = dp[tl][v] = 0.f;
+        ring[0] = read_prod(0, 0);
+        ring[1] = read_prod(0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < NA; ++j) {                      // stage 1
+            ring[(j + 2) % 4] = j + 2 < NA ? read_prod(0, j + 2) : read_prod(1, j + 2 - NA);
+            if (j & 1) dp[0] = E::mfma32(ring[j % 4], gb[j >> 1], dp[0]);
+            else s[0] = E::mfma32(ring[j % 4], qb[j >> 1], s[0]);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        // dQ^T[d, i] += sum_l K^T[d, l] dS^T[l, i]
 #pragma unroll
-        for (int st = 0; st < 4; ++st)
+        for (int j = 0; j < NA; ++j) {                      // stage 2
+            ring[(NA + j + 2) % 4] = j + 2 < NA ? read_prod(1, j + 2) : read_out(0, j + 2 - NA);
+            if (j & 1) dp[1] = E::mfma32(ring[(NA + j) % 4], gb[j >> 1], dp[1]);
+            else s[1] = E::mfma32(ring[(NA + j) % 4], qb[j >> 1], s[1]);
 #pragma unroll
-            for (int dt = 0; dt < T::DT; ++dt) acc[dt] = E::mfma32(tile_tr<D>(kt, tr[dt][0], tr[dt][1], st), pb[st], acc[dt]);
+            for (int v = VA * j; v < VA * (j + 1); ++v) soft(0, v);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NO; ++j) {                      // stage 3
+            ring[(2 * NA + j + 2) % 4] = j + 2 < NO ? read_out(0, j + 2) : read_out(1, j + 2 - NO);
+            acc[j % T::DT] = E::mfma32(ring[(2 * NA + j) % 4], pb[j / T::DT], acc[j % T::DT]);
+#pragma unroll
+            for (int v = VO * j; v < VO * (j + 1); ++v) soft(1, v);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NO; ++j) {                      // stage 4
+            if (j + 2 < NO) ring[(2 * NA + NO + j + 2) % 4] = read_out(1, j + 2);
+            acc[j % T::DT] = E::mfma32(ring[(2 * NA + NO + j) % 4], pb[2 + j / T::DT], acc[j % T::DT]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
     if (i < p.Sq) {
         float* row = p.dq + (int64_t)b * p.dqs[0] + (int64_t)i * p.dqs[1] + (int64_t)h * p.dqs[2] + 4 * hf;
