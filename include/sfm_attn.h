@@ -172,7 +172,7 @@ int sfm_full_attention_with_kv_cache(const sfm_dense_desc* desc, const void* q, 
  *   dk, dv              tensor dtype, [B, kv_grad_end - kv_grad_start, H, D]: gradients of keys kv_grad_start ..
  *                       kv_grad_end - 1; a proper sub-range is the reference's grad_only_new_kv (:362-364); an empty
  *                       range produces dq only
- *   workspace           sfm_dense_bwd_workspace_bytes (one float per batch, head and query) */
+ *   workspace           sfm_dense_bwd_workspace_bytes (two floats per batch, head and query) */
 typedef struct sfm_dense_bwd_desc {
     sfm_dense_desc fwd;
     int64_t dq_stride[3];

@@ -13,11 +13,12 @@
 // come out transposed, [streamed row, own row], one own row per lane, which is directly the B operand of the gradient
 // products whose A operands are transposing LDS reads (ds_read_tr16_b64) of the streamed tile.
 //   dq kernel:  own = 32 queries per wave (4 waves, 128 queries per workgroup), streamed = K and V tiles.
-//   dkv kernel: own = 32 keys per pair of waves (the two waves of a pair take half of the head dim of dK and dV each and
-//               both recompute the logits: the accumulators of a full head dim do not fit beside the operands),
-//               streamed = q and dO tiles plus the tile's log-sum-exp and delta values.
+//   dkv kernel: own = 32 keys per wave (4 waves, 128 keys per workgroup), streamed = q and dO tiles plus the tile's
+//               log-sum-exp and delta values; three tiles in LDS, one wave per SIMD.
 
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "sfm_attn.h"
 #include "sfm_common.hpp"
@@ -28,7 +29,8 @@ namespace {
 struct DenseBwdArgs {
     const char *q, *k, *v, *out, *dout;
     const float* lse;        // [B][H][Sq], natural log
-    float* delta;            // [B][H][Sq]
+    float* lse2;             // [B][H][Sq], the same in base-2 units (scratch)
+    float* delta;            // [B][H][Sq] (scratch)
     float* dq;
     char *dk, *dv;
     int64_t qs[3], ks[3], vs[3], os[3], dqs[3], dks[3];      // batch, token, head; in elements
@@ -54,7 +56,7 @@ __device__ __forceinline__ int db_swz(int r) {
     return CPR >= 16 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
 }
 
-// delta[b][h][i] = dO_i . O_i: 16-byte chunks, D / 8 consecutive lanes per row
+// delta[b][h][i] = dO_i . O_i (16-byte chunks, D / 8 consecutive lanes per row) and the log-sum-exp in base-2 units
 template <class E, int D>
 __global__ __launch_bounds__(256) void dense_bwd_delta_kernel(DenseBwdArgs p) {
     constexpr int CH = D / 8, RPB = 256 / CH;
@@ -76,7 +78,10 @@ __global__ __launch_bounds__(256) void dense_bwd_delta_kernel(DenseBwdArgs p) {
     }
 #pragma unroll
     for (int o = 1; o < CH; o <<= 1) dot += __shfl_xor(dot, o);
-    if (ch == 0 && row < total) p.delta[row] = dot;
+    if (ch == 0 && row < total) {
+        p.delta[row] = dot;
+        p.lse2[row] = p.lse[row] * kLog2e;
+    }
 }
 
 // Shared pieces of the two kernels.  A tile is 64 rows of D elements, row pitch 2 D bytes.
@@ -139,7 +144,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         qb[ds] = *(const u32x4*)(qrow + 32 * ds);
         gb[ds] = *(const u32x4*)(grow + 32 * ds);
     }
-    const float lse2 = p.lse[(int64_t)bh * p.Sq + ic] * kLog2e;
+    const float lse2 = p.lse2[(int64_t)bh * p.Sq + ic];
     const float dl = p.delta[(int64_t)bh * p.Sq + ic];
     const float sc2 = p.scale * kLog2e;
 
@@ -178,8 +183,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
 
     const int nt = (p.Skv + 63) / 64;
-    stage(0);
-    for (int t = 0; t < nt; ++t) {
+    // one tile; RAGGED (only the last tile can be) masks the keys past the end
+    auto tile = [&](int t, auto ragged_c) {
+        constexpr bool ragged = decltype(ragged_c)::value;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();                                   // tile t is in LDS; every wave is done with tile t - 1
         if (t + 1 < nt) stage(t + 1);
@@ -193,7 +199,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         constexpr int VA = 16 / NA, VO = 16 / NO;           // values of the softmax backward beside each of them
         f32x16 s[2], dp[2];
         u32x4 pb[4], ring[4];
-        const bool ragged = 64 * t + 64 > p.Skv;            // uniform: only the last tile can hold keys past the end
         auto read_prod = [&](int tl, int j) {               // j even: K rows for the logits, odd: V rows for dP
             return *(const u32x4*)(((j & 1) ? vt : kt) + tl * 32 * T::kPitch + (a_off ^ (uint32_t)((j >> 1) << 5)));
         };
@@ -241,7 +246,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             acc[j % T::DT] = E::mfma32(ring[(2 * NA + NO + j) % 4], pb[2 + j / T::DT], acc[j % T::DT]);
             __builtin_amdgcn_sched_barrier(0);
         }
-    }
+    };
+    stage(0);
+    for (int t = 0; t + 1 < nt; ++t) tile(t, std::false_type{});
+    if (p.Skv % 64) tile(nt - 1, std::true_type{});
+    else tile(nt - 1, std::false_type{});
     if (i < p.Sq) {
         float* row = p.dq + (int64_t)b * p.dqs[0] + (int64_t)i * p.dqs[1] + (int64_t)h * p.dqs[2] + 4 * hf;
 #pragma unroll
@@ -255,18 +264,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// One wave per SIMD: the wave's K and V rows (64 registers), dK^T and dV^T of a full head dim (128) and two half tiles
+// of logits and dP do not fit 256 registers, and with the MFMAs' operands read ahead and the softmax backward pinned
+// beside them a second wave would add little.
 template <class E, int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void dense_bwd_dkv_kernel(DenseBwdArgs p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void dense_bwd_dkv_kernel(DenseBwdArgs p) {
     using T = Tile<D>;
-    constexpr int DH = T::DT / 2;                          // head-dim blocks of 32 per wave
-    constexpr int oStat = 4 * T::kBytes;                   // [buffer][lse 64 floats | delta 64 floats]
+    constexpr int kBuf = 3;                                // tiles in LDS: the one in use and two on their way
+    constexpr int oStat = kBuf * 2 * T::kBytes;            // [buffer][lse 64 floats | delta 64 floats | 128 unused]
     extern __shared__ __attribute__((aligned(256))) char lds[];          // [buffer][q tile | dO tile], then the row values
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
     const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int kg = wave >> 1, dh = wave & 1;
     const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
-    const int l = p.kv0 + blockIdx.x * 64 + kg * 32 + m;
+    const int l = p.kv0 + blockIdx.x * 128 + wave * 32 + m;
     const int lc = min(l, p.kv1 - 1);
 
     const char* krow = p.k + ((int64_t)b * p.ks[0] + (int64_t)lc * p.ks[1] + (int64_t)h * p.ks[2]) * 2 + 16 * hf;
@@ -281,11 +292,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     const char* qbase = p.q + ((int64_t)b * p.qs[0] + (int64_t)h * p.qs[2]) * 2;
     const char* gbase = p.dout + ((int64_t)b * p.os[0] + (int64_t)h * p.os[2]) * 2;
-    const float* lsep = p.lse + (int64_t)bh * p.Sq;
+    const float* lsep = p.lse2 + (int64_t)bh * p.Sq;
     const float* dlp = p.delta + (int64_t)bh * p.Sq;
     const uint32_t qrb = (uint32_t)(p.qs[1] * 2), grb = (uint32_t)(p.os[1] * 2);
+    // every wave issues the same number of loads per tile (T::CPR / 2 + 1), so that one count waits for a tile
     auto stage = [&](int t) {
-        const uint32_t dst = lds0 + (uint32_t)(t & 1) * 2 * T::kBytes;
+        const uint32_t dst = lds0 + (uint32_t)(t % kBuf) * 2 * T::kBytes;
         for (int g = wave; g < T::CPR; g += 4) {
             const int P = g * 64 + lane;
             const int r = P / T::CPR, c = (P % T::CPR) ^ db_swz<T::CPR>(r);
@@ -294,69 +306,125 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             db_load_lds16(gbase, row * grb + (uint32_t)c * 16, dst + T::kBytes + (uint32_t)g * 1024);
         }
         const uint32_t row = (uint32_t)min(64 * t + lane, p.Sq - 1);
-        if (wave == 0) db_load_lds4(lsep, row * 4, lds0 + oStat + (uint32_t)(t & 1) * 512);
-        if (wave == 1) db_load_lds4(dlp, row * 4, lds0 + oStat + (uint32_t)(t & 1) * 512 + 256);
+        db_load_lds4((wave & 1) ? dlp : lsep, row * 4, lds0 + oStat + (uint32_t)(t % kBuf) * 1024 + (uint32_t)wave * 256);
     };
     const uint32_t a_off = (uint32_t)m * T::kPitch + (uint32_t)((hf ^ db_swz<T::CPR>(m)) << 4);
-    uint32_t tr[DH][2];
+    uint32_t tr[T::DT][2];
     {
         const int s16 = lane & 15, g16 = lane >> 4;
         const int rl = 4 * hf + (s16 >> 2);
         const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
 #pragma unroll
-        for (int dtl = 0; dtl < DH; ++dtl)
+        for (int dt = 0; dt < T::DT; ++dt)
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 const int r = rl + 8 * half;
-                tr[dtl][half] = (uint32_t)(r * T::kPitch + (((4 * (dh * DH + dtl) + cl) ^ db_swz<T::CPR>(r)) << 4) + (s16 & 1) * 8);
+                tr[dt][half] = (uint32_t)(r * T::kPitch + (((4 * dt + cl) ^ db_swz<T::CPR>(r)) << 4) + (s16 & 1) * 8);
             }
     }
 
-    f32x16 dka[DH], dva[DH];
+    f32x16 dka[T::DT], dva[T::DT];
 #pragma unroll
-    for (int dtl = 0; dtl < DH; ++dtl)
+    for (int dt = 0; dt < T::DT; ++dt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) dka[dtl][v] = dva[dtl][v] = 0.f;
+        for (int v = 0; v < 16; ++v) dka[dt][v] = dva[dt][v] = 0.f;
 
     const int nt = (p.Sq + 63) / 64;
-    stage(0);
-    for (int t = 0; t < nt; ++t) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();                                   // tile t is in LDS; every wave is done with tile t - 1
-        if (t + 1 < nt) stage(t + 1);
-        const char* qt = lds + (t & 1) * 2 * T::kBytes;
-        const char* gt = qt + T::kBytes;
-        const char* st_ = lds + oStat + (t & 1) * 512;
-        f32x16 s[2], dp[2];
-        tile_products<E, D>(qt, gt, a_off, kb, vb, s, dp);     // S[i, l] and dP[i, l]: lane = key, registers = queries
-        u32x4 pb[4], sb[4];
-#pragma unroll
-        for (int tl = 0; tl < 2; ++tl) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const f32x4 ls = *(const f32x4*)(st_ + (32 * tl + 8 * g + 4 * hf) * 4);
-                const f32x4 dl = *(const f32x4*)(st_ + 256 + (32 * tl + 8 * g + 4 * hf) * 4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int v = 4 * g + e;
-                    const int i = 64 * t + 32 * tl + 8 * g + 4 * hf + e;
-                    const float pv = i < p.Sq ? fast_exp2(s[tl][v] * sc2 - ls[e] * kLog2e) : 0.f;
-                    s[tl][v] = pv;
-                    dp[tl][v] = pv * (dp[tl][v] - dl[e]);
-                }
-            }
-            pack_steps<E>(s[tl], pb[2 * tl], pb[2 * tl + 1]);
-            pack_steps<E>(dp[tl], sb[2 * tl], sb[2 * tl + 1]);
+    // one tile; RAGGED (only the last tile can be) masks the queries past the end
+    auto tile = [&](int t, auto ragged_c) {
+        constexpr bool ragged = decltype(ragged_c)::value;
+        // tile t has landed when at most the loads of tile t + 1 are outstanding
+        if (t + 1 < nt) {
+            if (T::CPR == 16) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
-        // dV^T[d, l] += sum_i dO^T[d, i] P[i, l];  dK^T[d, l] += sum_i q^T[d, i] dS[i, l]
-#pragma unroll
-        for (int st = 0; st < 4; ++st)
-#pragma unroll
-            for (int dtl = 0; dtl < DH; ++dtl) {
-                dva[dtl] = E::mfma32(tile_tr<D>(gt, tr[dtl][0], tr[dtl][1], st), pb[st], dva[dtl]);
-                dka[dtl] = E::mfma32(tile_tr<D>(qt, tr[dtl][0], tr[dtl][1], st), sb[st], dka[dtl]);
+        __syncthreads();                                   // tile t is in LDS; every wave is done with tile t - 1
+        if (t + 2 < nt) stage(t + 2);
+        const char* qt = lds + (t % kBuf) * 2 * T::kBytes;
+        const char* gt = qt + T::kBytes;
+        const char* st_ = lds + oStat + (t % kBuf) * 1024;
+
+        // Four stages per tile as in the dq kernel; lane = key, registers = queries:
+        //   1  S, dP of queries 0..31            2  those of queries 32..63 | softmax backward of queries 0..31
+        //   3  dV^T += dO^T P, dK^T += q^T dS of queries 0..31 | softmax backward of queries 32..63      4  the same of queries 32..63
+        constexpr int NA = 2 * T::DS, NO = 4 * T::DT;
+        constexpr int VA = 16 / NA > 0 ? 16 / NA : 1, VO = 16 / NO > 0 ? 16 / NO : 1;
+        f32x16 s[2], dp[2];
+        u32x4 pb[4], sb[4], ring[4];
+        auto read_prod = [&](int tl, int j) {               // j even: q rows for S, odd: dO rows for dP
+            return *(const u32x4*)(((j & 1) ? gt : qt) + tl * 32 * T::kPitch + (a_off ^ (uint32_t)((j >> 1) << 5)));
+        };
+        // output MFMA j of a half: step st = 2 tl + j / (2 DT), head-dim block dt = (j / 2) % DT, j even: dV (dO^T), odd: dK (q^T)
+        auto read_out = [&](int tl, int j) {
+            const int dt = (j >> 1) % T::DT;
+            return tile_tr<D>((j & 1) ? qt : gt, tr[dt][0], tr[dt][1], 2 * tl + j / (2 * T::DT));
+        };
+        f32x4 ls4, dl4;                                     // row values of the four queries v & ~3 .. + 3
+        auto soft = [&](int tl, int v) {
+            const int r = 32 * tl + 8 * (v >> 2) + 4 * hf + (v & 3);
+            if ((v & 3) == 0) {
+                ls4 = *(const f32x4*)(st_ + r * 4);
+                dl4 = *(const f32x4*)(st_ + 256 + r * 4);
             }
-    }
+            float pv = fast_exp2(fmaf(s[tl][v], sc2, -ls4[v & 3]));
+            if (ragged) pv = 64 * t + r < p.Sq ? pv : 0.f;
+            s[tl][v] = pv;
+            dp[tl][v] = pv * (dp[tl][v] - dl4[v & 3]);
+            if (v & 1) {
+                pb[2 * tl + (v >> 3)][(v >> 1) & 3] = pack2<E>(s[tl][v - 1], s[tl][v]);
+                sb[2 * tl + (v >> 3)][(v >> 1) & 3] = pack2<E>(dp[tl][v - 1], dp[tl][v]);
+            }
+        };
+        auto out_mfma = [&](int tl, int j, const u32x4& a) {
+            const int dt = (j >> 1) % T::DT, st = 2 * tl + j / (2 * T::DT);
+            if (j & 1) dka[dt] = E::mfma32(a, sb[st], dka[dt]);
+            else dva[dt] = E::mfma32(a, pb[st], dva[dt]);
+        };
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s[tl][v] = dp[tl][v] = 0.f;
+        ring[0] = read_prod(0, 0);
+        ring[1] = read_prod(0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < NA; ++j) {                      // stage 1
+            ring[(j + 2) % 4] = j + 2 < NA ? read_prod(0, j + 2) : read_prod(1, j + 2 - NA);
+            if (j & 1) dp[0] = E::mfma32(ring[j % 4], vb[j >> 1], dp[0]);
+            else s[0] = E::mfma32(ring[j % 4], kb[j >> 1], s[0]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NA; ++j) {                      // stage 2
+            ring[(NA + j + 2) % 4] = j + 2 < NA ? read_prod(1, j + 2) : read_out(0, j + 2 - NA);
+            if (j & 1) dp[1] = E::mfma32(ring[(NA + j) % 4], vb[j >> 1], dp[1]);
+            else s[1] = E::mfma32(ring[(NA + j) % 4], kb[j >> 1], s[1]);
+#pragma unroll
+            for (int v = VA * j; v < VA * (j + 1) && v < 16; ++v) soft(0, v);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NO; ++j) {                      // stage 3
+            ring[(2 * NA + j + 2) % 4] = j + 2 < NO ? read_out(0, j + 2) : read_out(1, j + 2 - NO);
+            out_mfma(0, j, ring[(2 * NA + j) % 4]);
+#pragma unroll
+            for (int v = VO * j; v < VO * (j + 1) && v < 16; ++v) soft(1, v);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < NO; ++j) {                      // stage 4
+            if (j + 2 < NO) ring[(2 * NA + NO + j + 2) % 4] = read_out(1, j + 2);
+            out_mfma(1, j, ring[(2 * NA + NO + j) % 4]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    stage(0);
+    if (nt > 1) stage(1);
+    for (int t = 0; t + 1 < nt; ++t) tile(t, std::false_type{});
+    if (p.Sq % 64) tile(nt - 1, std::true_type{});
+    else tile(nt - 1, std::false_type{});
     // lane (key, hf) holds head-dim 32 dt + 8 g + 4 hf + 0..3; the half swap leaves 8 consecutive ones per lane
     const int64_t obase = ((int64_t)b * p.dks[0] + (int64_t)(lc - p.kv0) * p.dks[1] + (int64_t)h * p.dks[2]) * 2;
     auto store = [&](char* dst, const f32x16& a, int dt, float sc) {
@@ -370,9 +438,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     };
 #pragma unroll
-    for (int dtl = 0; dtl < DH; ++dtl) {
-        store(p.dk, dka[dtl], dh * DH + dtl, p.scale);
-        store(p.dv, dva[dtl], dh * DH + dtl, 1.f);
+    for (int dt = 0; dt < T::DT; ++dt) {
+        store(p.dk, dka[dt], dt, p.scale);
+        store(p.dv, dva[dt], dt, 1.f);
     }
 }
 
@@ -382,7 +450,7 @@ int launch_t(const DenseBwdArgs& a, hipStream_t stream) {
     const int64_t rows = (int64_t)a.B * a.H * a.Sq;
     constexpr int RPB = 256 / (D / 8);
     hipLaunchKernelGGL((dense_bwd_delta_kernel<E, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, stream, a);
-    const size_t lds_dq = 4 * T::kBytes, lds_dkv = 4 * T::kBytes + 1024;
+    const size_t lds_dq = 4 * T::kBytes, lds_dkv = 6 * T::kBytes + 3 * 1024;
     if (lds_dkv > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)dense_bwd_dkv_kernel<E, D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dkv);
         if (e == hipSuccess)
@@ -394,7 +462,7 @@ int launch_t(const DenseBwdArgs& a, hipStream_t stream) {
     }
     hipLaunchKernelGGL((dense_bwd_dq_kernel<E, D>), dim3((a.Sq + 127) / 128, a.B * a.H), dim3(256), lds_dq, stream, a);
     if (a.kv1 > a.kv0)
-        hipLaunchKernelGGL((dense_bwd_dkv_kernel<E, D>), dim3((a.kv1 - a.kv0 + 63) / 64, a.B * a.H), dim3(256), lds_dkv, stream, a);
+        hipLaunchKernelGGL((dense_bwd_dkv_kernel<E, D>), dim3((a.kv1 - a.kv0 + 127) / 128, a.B * a.H), dim3(256), lds_dkv, stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("dense backward: launch failed: %s", hipGetErrorString(e));
@@ -409,14 +477,14 @@ bool dense_bwd_supported(int dtype, int D) { return (dtype == SFM_BF16 || dtype 
 
 int launch_dense_bwd(const sfm_dense_desc& d, const int64_t* dq_stride, const int64_t* dkv_stride, int64_t kv0, int64_t kv1,
                      const void* q, const void* k, const void* v, const void* out, const float* lse, const void* dout, float* dq,
-                     void* dk, void* dv, float* delta, hipStream_t stream) {
+                     void* dk, void* dv, float* scratch, hipStream_t stream) {
     if (!dense_bwd_supported(d.dtype, d.D)) {
         set_error("dense backward: bf16 / fp16 tensors with head_dim 64 or 128 only");
         return SFM_ERR_UNSUPPORTED;
     }
     DenseBwdArgs a;
     a.q = (const char*)q; a.k = (const char*)k; a.v = (const char*)v; a.out = (const char*)out; a.dout = (const char*)dout;
-    a.lse = lse; a.delta = delta; a.dq = dq; a.dk = (char*)dk; a.dv = (char*)dv;
+    a.lse = lse; a.delta = scratch; a.lse2 = scratch + (int64_t)d.B * d.H * d.q_tokens; a.dq = dq; a.dk = (char*)dk; a.dv = (char*)dv;
     int64_t bad = 0;
     for (int i = 0; i < 3; ++i) {
         a.qs[i] = d.q_stride[i]; a.ks[i] = d.k_stride[i]; a.vs[i] = d.v_stride[i]; a.os[i] = d.o_stride[i];

@@ -750,7 +750,7 @@ int sfm_dense_bwd_workspace_bytes(const sfm_dense_bwd_desc* desc, size_t* bytes)
     }
     int rc = check_dense_bwd(desc);
     if (rc) return rc;
-    *bytes = ((size_t)desc->fwd.B * desc->fwd.H * desc->fwd.q_tokens * sizeof(float) + 255) / 256 * 256;
+    *bytes = ((size_t)2 * desc->fwd.B * desc->fwd.H * desc->fwd.q_tokens * sizeof(float) + 255) / 256 * 256;
     return SFM_OK;
 }
 
@@ -768,7 +768,7 @@ int sfm_dense_bwd(const sfm_dense_bwd_desc* desc, const void* q, const void* k, 
         set_error("tensors must be 16-byte aligned (lse: 4-byte)");
         return SFM_ERR_ALIGN;
     }
-    const size_t need = (size_t)desc->fwd.B * desc->fwd.H * desc->fwd.q_tokens * sizeof(float);
+    const size_t need = (size_t)2 * desc->fwd.B * desc->fwd.H * desc->fwd.q_tokens * sizeof(float);
     if (!workspace || (((uintptr_t)workspace) & 255) || workspace_bytes < need) {
         set_error("workspace must be non-NULL, 256-byte aligned and hold at least %zu bytes", need);
         return SFM_ERR_WORKSPACE;

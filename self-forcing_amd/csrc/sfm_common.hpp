@@ -204,11 +204,11 @@ int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, i
                              void* dv, const int64_t* dks, int64_t row0, const TokMap& kmap, int H, int unit0, int f0, int f1,
                              hipStream_t stream);
 
-// backward of the dense attention (dense_attn_bwd.hip); delta is B*H*q_tokens floats of scratch
+// backward of the dense attention (dense_attn_bwd.hip); scratch is 2*B*H*q_tokens floats
 bool dense_bwd_supported(int dtype, int D);
 int launch_dense_bwd(const sfm_dense_desc& d, const int64_t* dq_stride, const int64_t* dkv_stride, int64_t kv0, int64_t kv1,
                      const void* q, const void* k, const void* v, const void* out, const float* lse, const void* dout, float* dq,
-                     void* dk, void* dv, float* delta, hipStream_t stream);
+                     void* dk, void* dv, float* scratch, hipStream_t stream);
 
 void set_error(const char* fmt, ...);
 int cu_count();                                  // compute units of the current device (cached per thread)
