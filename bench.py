@@ -138,6 +138,19 @@ def op_level(torch, sfa, args):
         bwd[name] = (time.perf_counter() - t0) * 1e3 / 3
     bwd_ms = bwd["saved"]
 
+    # backward of the dense fallback at the same shape (all keys, and the new chunk's keys only)
+    from self_forcing_amd.attention import _dense_bwd, _dense_fwd
+    dout_kept, dlse = _dense_fwd(q, kc, vc, D ** -0.5, True)
+    dense_bwd = {}
+    for name, rng in (("all_keys", (0, SKV)), ("new_chunk_keys", (SKV - SQ, SKV))):
+        _dense_bwd(q, kc, vc, dout_kept, dlse, do, D ** -0.5, *rng)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            _dense_bwd(q, kc, vc, dout_kept, dlse, do, D ** -0.5, *rng)
+        torch.cuda.synchronize()
+        dense_bwd[name] = (time.perf_counter() - t0) * 1e3 / 3
+
     # what the matrix pipes sustain on this machine (independent MFMAs only), to read the dense figure against
     probe = C.c_float(0)
     L.check(lib.sfm_probe_mfma_bf16(20000, stream, C.byref(probe)))
@@ -168,7 +181,8 @@ def op_level(torch, sfa, args):
         "monarch_bwd": {"workload": "gradients of q and of all 21 cached K/V frames at the same shape",
                         "ms_per_call": bwd_ms, "ms_per_call_recomputing_statistics": bwd["recompute"]},
         "dense_fallback": {"ms_per_call": dense_ms, "tflops": dense_tfl, "mfma_frac": dense_tfl / MFMA_BF16_PEAK_TFLOPS,
-                           "mfma_probe_tflops": probe.value, "frac_of_probe": dense_tfl / probe.value},
+                           "mfma_probe_tflops": probe.value, "frac_of_probe": dense_tfl / probe.value,
+                           "bwd_ms_per_call": dense_bwd["all_keys"], "bwd_ms_per_call_new_chunk_keys": dense_bwd["new_chunk_keys"]},
         "roofline": {"kernel": "monarch_step1_kernel (configs[1] shape)", "bound": "hbm", "achieved": s1_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s1_gbs / HBM_PEAK_GBS,
                      "algorithmic_bytes": STEP1_BYTES, "traffic": MEASURED_TRAFFIC["monarch_step1_kernel"],

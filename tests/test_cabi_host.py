@@ -133,6 +133,44 @@ def test_row_statistics_size_and_argument_checks():
     assert lib.sfm_monarch_bwd_saved(C.byref(bd), fake, fake, fake, fake, fake, None, fake, fake, fake, fake, 1 << 40, None) == -1
 
 
+def test_dense_backward_argument_checks():
+    lib = L.load()
+    bd = L.DenseBwdDesc()
+    d = bd.fwd
+    d.dtype, d.B, d.H, d.D, d.q_tokens, d.kv_tokens, d.sm_scale = L.SFM_BF16, 1, 2, 128, 100, 300, 128 ** -0.5
+    for name, toks in (("q_stride", 100), ("k_stride", 300), ("v_stride", 300), ("o_stride", 100)):
+        setattr(d, name, (C.c_int64 * 3)(toks * 256, 256, 128))
+    bd.dq_stride = (C.c_int64 * 3)(100 * 256, 256, 128)
+    bd.dkv_stride = (C.c_int64 * 3)(300 * 256, 256, 128)
+    bd.kv_grad_start, bd.kv_grad_end = 0, 300
+    n = C.c_size_t(0)
+    assert lib.sfm_dense_bwd_workspace_bytes(C.byref(bd), C.byref(n)) == 0 and n.value == 1792      # 2 x 2 x 100 floats, rounded to 256
+    fake = 0x10000
+    ok = [fake] * 9
+    call = lambda args, ws=fake, nb=1792: lib.sfm_dense_bwd(C.byref(bd), *args, ws, nb, None)
+    for i in range(9):
+        args = list(ok)
+        args[i] = None
+        assert call(args) == -1
+    args = list(ok)
+    args[0] = fake + 2
+    assert call(args) == -7
+    assert call(ok, None) == -6 and call(ok, fake, 1599) == -6 and call(ok, fake + 16) == -6
+    bd.kv_grad_end = 301
+    assert call(ok) == -4
+    bd.kv_grad_start, bd.kv_grad_end = 200, 100
+    assert call(ok) == -4
+    bd.kv_grad_start, bd.kv_grad_end = 0, 300
+    d.D = 32
+    for name, toks in (("q_stride", 100), ("k_stride", 300), ("v_stride", 300), ("o_stride", 100)):
+        setattr(d, name, (C.c_int64 * 3)(toks * 64, 64, 32))
+    assert call(ok) == -9                              # head_dim 32 has a forward only
+    d.D, d.dtype = 128, L.SFM_F32
+    for name, toks in (("q_stride", 100), ("k_stride", 300), ("v_stride", 300), ("o_stride", 100)):
+        setattr(d, name, (C.c_int64 * 3)(toks * 256, 256, 128))
+    assert call(ok) == -9
+
+
 def test_kv_cache_op_range_checks_happen_before_any_write():
     lib = L.load()
     d = _desc()
