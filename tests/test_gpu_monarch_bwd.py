@@ -59,6 +59,22 @@ def test_no_cache_fp32_gradients(tiling, h, w, bwd_path):
     _close(vd.grad, vr.grad, torch.float32)
 
 
+@pytest.mark.parametrize("tiling,h,w", [((1, 1, 1), 4, 8), ((1, 2, 1), 6, 8), ((3, 1, 1), 4, 8), ((1, 1, 2), 3, 16), ((3, 2, 2), 4, 16)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_no_cache_16bit_gradients_over_the_tilings(tiling, h, w, dtype):
+    """Token-order k, v (no cache): the fused kernels read q, k, v rows through the tiling's index maps."""
+    F, H, D = 3, 2, 64
+    q0, do = (randn((1, F * h * w, H, D), 180 + i, dtype) for i in range(2))
+    k0, v0 = (randn((1, 2 * F * h * w, H, D), 182 + i, dtype) for i in range(2))
+    qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
+    monarch.monarch_attn(qr, kr, vr, *tiling, h, w).backward(do.double())
+    qd, kd, vd = _leaf(q0, DEV), _leaf(k0, DEV), _leaf(v0, DEV)
+    mattn.monarch_attn(qd, kd, vd, *tiling, h, w).backward(do.to(DEV))
+    _close(qd.grad, qr.grad, dtype)
+    _close(kd.grad, kr.grad, dtype)
+    _close(vd.grad, vr.grad, dtype)
+
+
 def test_block_causal_fp32_gradients(bwd_path):
     h, w, F = 3, 8, 4
     q0, k0, v0, do = (randn((1, F * h * w, 2, 64), 110 + i, torch.float32) for i in range(4))
