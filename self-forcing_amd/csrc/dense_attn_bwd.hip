@@ -352,7 +352,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         constexpr int NA = 2 * T::DS, NO = 4 * T::DT;
         constexpr int VA = 16 / NA > 0 ? 16 / NA : 1, VO = 16 / NO > 0 ? 16 / NO : 1;
         f32x16 s[2], dp[2];
-        u32x4 pb[4], sb[4], ring[4];
+        constexpr int kAhead = 4, kRing = 8;                // A operands read this many MFMAs ahead
+        u32x4 pb[4], sb[4], ring[kRing];
         auto read_prod = [&](int tl, int j) {               // j even: q rows for S, odd: dO rows for dP
             return *(const u32x4*)(((j & 1) ? gt : qt) + tl * 32 * T::kPitch + (a_off ^ (uint32_t)((j >> 1) << 5)));
         };
@@ -386,37 +387,37 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
             for (int v = 0; v < 16; ++v) s[tl][v] = dp[tl][v] = 0.f;
-        ring[0] = read_prod(0, 0);
-        ring[1] = read_prod(0, 1);
+#pragma unroll
+        for (int j = 0; j < kAhead; ++j) ring[j] = read_prod(0, j);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < NA; ++j) {                      // stage 1
-            ring[(j + 2) % 4] = j + 2 < NA ? read_prod(0, j + 2) : read_prod(1, j + 2 - NA);
-            if (j & 1) dp[0] = E::mfma32(ring[j % 4], vb[j >> 1], dp[0]);
-            else s[0] = E::mfma32(ring[j % 4], kb[j >> 1], s[0]);
+            ring[(j + kAhead) % kRing] = j + kAhead < NA ? read_prod(0, j + kAhead) : read_prod(1, j + kAhead - NA);
+            if (j & 1) dp[0] = E::mfma32(ring[j % kRing], vb[j >> 1], dp[0]);
+            else s[0] = E::mfma32(ring[j % kRing], kb[j >> 1], s[0]);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int j = 0; j < NA; ++j) {                      // stage 2
-            ring[(NA + j + 2) % 4] = j + 2 < NA ? read_prod(1, j + 2) : read_out(0, j + 2 - NA);
-            if (j & 1) dp[1] = E::mfma32(ring[(NA + j) % 4], vb[j >> 1], dp[1]);
-            else s[1] = E::mfma32(ring[(NA + j) % 4], kb[j >> 1], s[1]);
+            ring[(NA + j + kAhead) % kRing] = j + kAhead < NA ? read_prod(1, j + kAhead) : read_out(0, j + kAhead - NA);
+            if (j & 1) dp[1] = E::mfma32(ring[(NA + j) % kRing], vb[j >> 1], dp[1]);
+            else s[1] = E::mfma32(ring[(NA + j) % kRing], kb[j >> 1], s[1]);
 #pragma unroll
             for (int v = VA * j; v < VA * (j + 1) && v < 16; ++v) soft(0, v);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int j = 0; j < NO; ++j) {                      // stage 3
-            ring[(2 * NA + j + 2) % 4] = j + 2 < NO ? read_out(0, j + 2) : read_out(1, j + 2 - NO);
-            out_mfma(0, j, ring[(2 * NA + j) % 4]);
+            ring[(2 * NA + j + kAhead) % kRing] = j + kAhead < NO ? read_out(0, j + kAhead) : read_out(1, j + kAhead - NO);
+            out_mfma(0, j, ring[(2 * NA + j) % kRing]);
 #pragma unroll
             for (int v = VO * j; v < VO * (j + 1) && v < 16; ++v) soft(1, v);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int j = 0; j < NO; ++j) {                      // stage 4
-            if (j + 2 < NO) ring[(2 * NA + NO + j + 2) % 4] = read_out(1, j + 2);
-            out_mfma(1, j, ring[(2 * NA + NO + j) % 4]);
+            if (j + kAhead < NO) ring[(2 * NA + NO + j + kAhead) % kRing] = read_out(1, j + kAhead);
+            out_mfma(1, j, ring[(2 * NA + NO + j) % kRing]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
