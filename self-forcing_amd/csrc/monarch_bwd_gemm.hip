@@ -392,7 +392,7 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // Scratch of a pass over n units, in bytes (all sub-buffers 256-byte aligned).
 struct Layout {
-    size_t Qk, Qa, dOa, Oa, Kk, Vk, S1f, dRb, Rb, dS1, Kbar, Y, dKbar, dY, c, dc, S2f, dLmf, L, dS2, dQa, dQk, dKk, dVk, total;
+    size_t Qk, Qa, dOa, Kk, Vk, S1f, dRb, Rb, dS1, Kbar, Y, dKbar, dY, c, dc, S2f, dLmf, L, dS2, dQa, dQk, dKk, dVk, total;
 };
 
 // dtype code of the fused kernels for operand type E, or -1 (fp32 operands stay on the GEMMs)
@@ -412,7 +412,9 @@ struct Parts {
 Parts make_parts(const MonarchArgs& p, int dtype, const int64_t* dks) {
     Parts f;
     const bool h16 = dtype == SFM_BF16 || dtype == SFM_F16;
-    f.left = h16 && monarch_bwd_left_supported(dtype, p.D, p.b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
+    const bool q_rows_ok = (p.qs[0] | p.qs[1] | p.qs[2] | p.os[0] | p.os[1] | p.os[2]) % 8 == 0 &&       // 16-byte rows of q, dout, out
+                           (int64_t)p.na * p.b1 * p.b2 * p.qs[1] * 2 < ((int64_t)1 << 32);
+    f.left = h16 && q_rows_ok && monarch_bwd_left_supported(dtype, p.D, p.b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
     f.fwd = f.left && monarch_mfma_supported(dtype, p.D, p.b2) && getenv("SFM_BWD_FWD_GEMM") == nullptr;
     f.dqa = f.left && getenv("SFM_BWD_DQA_GEMM") == nullptr;
     const bool direct_ok = (dks[0] | dks[1] | dks[2] | p.vs[0] | p.vs[1] | p.vs[2]) % 8 == 0;      // 16-byte rows of v, dk, dv
@@ -427,10 +429,9 @@ Layout make_layout(const MonarchArgs& p, int n, size_t e, const Parts& f) {
     Layout l;
     size_t o = 0;
     auto take = [&](bool used, size_t bytes) { size_t at = o; o += used ? align256(bytes) : 0; return at; };
-    l.Qk = take(true, n * MQ * D * e);
-    l.Qa = take(true, n * MQ * D * e);
-    l.dOa = take(true, n * MQ * D * e);
-    l.Oa = take(f.left, n * MQ * D * e);
+    l.Qk = take(!f.fwd || !f.right, n * MQ * D * e);
+    l.Qa = take(!f.left, n * MQ * D * e);
+    l.dOa = take(!f.left, n * MQ * D * e);
     l.Kk = take(true, n * MK * D * e);
     l.Vk = take(!f.right, n * MK * D * e);
     l.S1f = take(!f.fwd, n * p.b1 * AJ * NL * 4);
@@ -518,15 +519,16 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
         constexpr int kPer = 8 / sizeof(T);
         const int64_t tq = (int64_t)n * MQ * (D / kPer), tk = (int64_t)n * MK * (D / kPer);
         const unsigned gq = (unsigned)((tq + 255) / 256), gk = (unsigned)((tk + 255) / 256);
-        hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.Qk), p.q, p.qs[0], p.qs[1], p.qs[2], p.qmap,
-                           na, H, D, p.unit0, 0, tq);
-        hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.Qa), p.q, p.qs[0], p.qs[1], p.qs[2], p.qmap,
-                           na, H, D, p.unit0, 1, tq);
-        hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.dOa), g.dout, g.dos[0], g.dos[1], g.dos[2],
-                           p.qmap, na, H, D, p.unit0, 1, tq);
-        if (saved)
-            hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.Oa), g.fout, g.dos[0], g.dos[1], g.dos[2],
+        // the fused kernels read q, dout (and out) rows where the callers' tensors have them
+        if (!fused_fwd || !fused_right)
+            hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.Qk), p.q, p.qs[0], p.qs[1], p.qs[2], p.qmap,
+                               na, H, D, p.unit0, 0, tq);
+        if (!fused_left) {
+            hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.Qa), p.q, p.qs[0], p.qs[1], p.qs[2], p.qmap,
+                               na, H, D, p.unit0, 1, tq);
+            hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.dOa), g.dout, g.dos[0], g.dos[1], g.dos[2],
                                p.qmap, na, H, D, p.unit0, 1, tq);
+        }
         hipLaunchKernelGGL((gather_rows<E>), dim3(gk), dim3(256), 0, stream, (T*)(ws + lay.Kk), p.k, p.ks[0], p.ks[1], p.ks[2], p.kmap,
                            nf, H, D, p.unit0, 0, tk);
         if (!fused_right)                               // the fused right-factor kernel reads v where it is
@@ -569,10 +571,10 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     if (fused_left) {
         // 4-7 in one kernel: statistics and gradients of the left factor without the [i x r] matrices in memory
         if (!cx.status)
-            cx.status = launch_monarch_bwd_left(left_dtype<E>(), D, n, b1, b2, AJ, nf, p.causal, s, ws + lay.Qa, ws + lay.dOa, ws + lay.Kbar,
-                                                ws + lay.Y, (const float*)(ws + lay.c), fused_fwd ? 1 : 0, ws + lay.dKbar, ws + lay.dY,
-                                                (float*)(ws + lay.dc), ws + lay.dS2, ds2_ld, saved ? ws + lay.Oa : nullptr,
-                                                saved ? g.fstats : nullptr, (b1 + 31) / 32 * 32, p.unit0, stream);
+            cx.status = launch_monarch_bwd_left(left_dtype<E>(), D, n, b1, b2, AJ, nf, p.causal, s, p.q, p.qs, g.dout, saved ? g.fout : nullptr,
+                                                g.dos, p.qmap, H, p.unit0, ws + lay.Kbar, ws + lay.Y, (const float*)(ws + lay.c),
+                                                fused_fwd ? 1 : 0, ws + lay.dKbar, ws + lay.dY, (float*)(ws + lay.dc), ws + lay.dS2, ds2_ld,
+                                                saved ? g.fstats : nullptr, (b1 + 31) / 32 * 32, stream);
     } else {
         // 4, 5. per unit and (a, j): S2 = q_i . Kbar_r, dLm = dO_i . Y_r; the [RR x D] matrix of column aj is every AJ-th row
         for (int u = 0; u < n && !cx.status; ++u) {
@@ -611,7 +613,7 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     if (fused_right) {
         if (!cx.status)
             cx.status = launch_monarch_bwd_right(left_dtype<E>(), D, nt, b1, b2, AJ, nf, s, ws + lay.Kk, p.v, p.vs, ws + lay.Rb,
-                                                 ws + lay.dKbar, ws + lay.dY, (const float*)(ws + lay.dc), ws + lay.Qk, ws + lay.dS1, g.dk,
+                                                 ws + lay.dKbar, ws + lay.dY, (const float*)(ws + lay.dc), p.q, p.qs, p.qmap, ws + lay.dS1, g.dk,
                                                  g.dv, g.dks, g.dk_row0, p.kmap, H, p.unit0, g.kv_f0, g.kv_f1, stream);
     } else {
         // 9. dR block = dKbar block . K block^T + dY block . V block^T per t

@@ -23,8 +23,12 @@ namespace sfm {
 namespace {
 
 struct LeftArgs {
-    const uint16_t* qa;      // [u][aj][b1][D]
-    const uint16_t* doa;     // [u][aj][b1][D]
+    const char* q;           // callers' tensors: row i of (unit, a, j) is token qmap.row(a, i) + j; strides batch, token, head
+    const char* dout;        // (in elements); out, optional, shares dout's strides
+    const char* out;
+    int64_t qs[3], os[3];
+    TokMap qmap;
+    int H;
     const uint16_t* kbar;    // row r of (u, aj) at ((u * RR + r) * AJ + aj) * D
     const uint16_t* y;
     const float* c;          // c_rows == 0: [u][aj][RR], natural log units; c_rows == 1: [(u * RR + r) * AJ + aj], log2 units
@@ -34,8 +38,7 @@ struct LeftArgs {
     float* dc;               // [u][aj][RR]
     uint16_t* ds2;           // [u][aj][b1][ds2_ld], ds2_ld >= RR
     int ds2_ld;
-    const uint16_t* oa;      // optional, with stats: the forward's output rows [u][aj][b1][D]
-    const float* stats;      // log2-sum-exp of the logits of row (unit, aj, i) at ((unit0 + u) * AJ + aj) * stats_ld + i
+    const float* stats;      // optional, with out:      // log2-sum-exp of the logits of row (unit, aj, i) at ((unit0 + u) * AJ + aj) * stats_ld + i
     int stats_ld, unit0;
     int b1, b2, AJ, nf, RR, causal;
     float scale;
@@ -67,19 +70,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     float* dls = (float*)(dos + 32 * kPitch);
     const bool saved = p.stats != nullptr;                // uniform: the forward's output and row statistics are at hand
     {
-        const uint16_t* qg = p.qa + uaj * b1 * D;
-        const uint16_t* dg = p.doa + uaj * b1 * D;
-        const uint16_t* og = saved ? p.oa + uaj * b1 * D : dg;
+        const int unit = p.unit0 + u, bb = unit / p.H, hh = unit % p.H;
+        const int a_q = aj / p.b2, j_q = aj % p.b2;
+        const char* qg = p.q + ((int64_t)bb * p.qs[0] + (int64_t)hh * p.qs[2]) * 2;
+        const char* dg = p.dout + ((int64_t)bb * p.os[0] + (int64_t)hh * p.os[2]) * 2;
+        const char* og = saved ? p.out + ((int64_t)bb * p.os[0] + (int64_t)hh * p.os[2]) * 2 : dg;
         constexpr int CH = D / 8;
         for (int cidx = lane; cidx < 32 * CH; cidx += 64) {
             const int r = cidx / CH, ch = cidx % CH;
             u32x4 a = {0u, 0u, 0u, 0u}, b = a;
             float dot = 0.f;
             if (r < b1) {
-                a = *(const u32x4*)(qg + r * D + ch * 8);
-                b = *(const u32x4*)(dg + r * D + ch * 8);
+                const int64_t tok = p.qmap.row(a_q, r) + j_q;
+                a = *(const u32x4*)(qg + tok * p.qs[1] * 2 + ch * 16);
+                b = *(const u32x4*)(dg + tok * p.os[1] * 2 + ch * 16);
                 if (saved) {                              // sum_r L dLm of row i is dO_i . O_i
-                    const u32x4 o = *(const u32x4*)(og + r * D + ch * 8);
+                    const u32x4 o = *(const u32x4*)(og + tok * p.os[1] * 2 + ch * 16);
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         dot += E::to_float((uint16_t)(b[e] & 0xffffu)) * E::to_float((uint16_t)(o[e] & 0xffffu)) +
@@ -428,15 +434,21 @@ bool monarch_bwd_left_supported(int dtype, int D, int b1) {
     return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b1 >= 1 && b1 <= 32;
 }
 
-int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* qa,
-                            const void* doa, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy,
-                            float* dc, void* ds2, int ds2_ld, const void* oa, const float* stats, int stats_ld, int unit0,
-                            hipStream_t stream) {
+int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* q,
+                            const int64_t* qs, const void* dout, const void* out, const int64_t* os, const TokMap& qmap, int H,
+                            int unit0, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy, float* dc,
+                            void* ds2, int ds2_ld, const float* stats, int stats_ld, hipStream_t stream) {
     LeftArgs a;
     a.ds2_ld = ds2_ld;
-    a.oa = (const uint16_t*)oa; a.stats = oa ? stats : nullptr; a.stats_ld = stats_ld; a.unit0 = unit0;
+    a.q = (const char*)q; a.dout = (const char*)dout; a.out = (const char*)out;
+    for (int i = 0; i < 3; ++i) {
+        a.qs[i] = qs[i];
+        a.os[i] = os[i];
+    }
+    a.qmap = qmap;
+    a.H = H;
+    a.stats = out ? stats : nullptr; a.stats_ld = stats_ld; a.unit0 = unit0;
     a.c_rows = c_rows;
-    a.qa = (const uint16_t*)qa; a.doa = (const uint16_t*)doa;
     a.kbar = (const uint16_t*)kbar; a.y = (const uint16_t*)y;
     a.c = c;
     a.dkbar = (uint16_t*)dkbar; a.dy = (uint16_t*)dy;

@@ -40,7 +40,9 @@ struct RightArgs {
     const char* dkbar;       // [t][AJ][D]
     const char* dy;
     const float* dc;         // [u][AJ][RR]
-    const char* qk;          // [(u, k)][AJ][D]
+    const char* q;           // caller's tensor: row (a, j) of (unit, k) is token qmap.row(a, k) + j, strides qs0, qs1, qs2
+    int64_t qs0, qs1, qs2;
+    TokMap qmap;
     uint16_t* ds1;           // [(u, k)][AJ][nf * b2]
     uint16_t* dk;            // caller's tensors: row kmap.row(f, k) + l - row0, strides s0 (batch), s1 (row), s2 (head)
     uint16_t* dv;
@@ -197,7 +199,17 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
     }
     __syncthreads();                                                     // K, V, dKbar, dY tiles are free
     // the query rows of (unit, k) take the place of the dY tile while the softmax backward runs
-    if (want) stage(p.qk + uk * AJ * kPitch, kPitch, AJ * CPR, oH, c_d{});
+    if (want) {
+        const char* qbase = p.q + ((int64_t)(unit / p.H) * p.qs0 + (int64_t)(unit % p.H) * p.qs2) * 2;
+        const uint32_t qrb = (uint32_t)(p.qs1 * 2);
+        const int nchunks = AJ * CPR;
+        for (int g = wave; g * 64 < nchunks; g += kWaves) {
+            const int P = min(g * 64 + lane, nchunks - 1);
+            const int r = P / CPR, c = (P % CPR) ^ br_swz<CPR>(r);
+            const uint32_t tok = (uint32_t)(p.qmap.row(r / b2, k) + r % b2);
+            br_load_lds16(qbase, tok * qrb + (uint32_t)(c * 16), lds0 + oH + (uint32_t)g * 1024);
+        }
+    }
 
     // ---- phase 1, softmax backward.  R[col][l] for the l this lane holds: l = 32 tl + 8 g + 4 hf + 0..3, 8 bytes of chunk 4 tl + g
     float rv[16];
@@ -275,9 +287,9 @@ bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ) {
 }
 
 int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, float scale, const void* kk, const void* v,
-                             const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* qk, void* ds1, void* dk,
-                             void* dv, const int64_t* dks, int64_t row0, const TokMap& kmap, int H, int unit0, int f0, int f1,
-                             hipStream_t stream) {
+                             const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* q,
+                             const int64_t* qs, const TokMap& qmap, void* ds1, void* dk, void* dv, const int64_t* dks, int64_t row0,
+                             const TokMap& kmap, int H, int unit0, int f0, int f1, hipStream_t stream) {
     if ((dks[0] | dks[1] | dks[2] | vs[0] | vs[1] | vs[2]) % 8 || ((uintptr_t)dk | (uintptr_t)dv | (uintptr_t)v) % 16 ||
         (int64_t)(b2 - 1) * vs[1] * 2 + 2 * D > 0xffffffffll) {
         set_error("monarch backward (right factor): v / dk / dv strides must be multiples of 8 elements and the pointers 16-byte aligned");
@@ -288,7 +300,8 @@ int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, i
     a.v = (const char*)v; a.vs0 = vs[0]; a.vs1 = vs[1]; a.vs2 = vs[2];
     a.dkbar = (const char*)dkbar; a.dy = (const char*)dy;
     a.dc = dc;
-    a.qk = (const char*)qk;
+    a.q = (const char*)q; a.qs0 = qs[0]; a.qs1 = qs[1]; a.qs2 = qs[2];
+    a.qmap = qmap;
     a.ds1 = (uint16_t*)ds1;
     a.dk = (uint16_t*)dk; a.dv = (uint16_t*)dv;
     a.s0 = dks[0]; a.s1 = dks[1]; a.s2 = dks[2]; a.row0 = row0;

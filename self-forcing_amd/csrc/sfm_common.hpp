@@ -186,23 +186,24 @@ size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits, const
 int launch_monarch_bwd_gemm(const MonarchBwdArgs& g, int dtype, int nunits, void* workspace, hipStream_t stream);
 // step 1 of the MFMA forward alone, with the scratch strides of `a` and, if a.rb is set, the right factor written out
 int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream);
-// fused left-factor part of the backward (monarch_bwd_left.hip); operands in the GEMM path's scratch layouts
+// fused left-factor part of the backward (monarch_bwd_left.hip): q, dout (and out, with stats) are the callers' tensors,
+// 16-byte aligned rows; everything else in the GEMM path's scratch layouts
 bool monarch_bwd_left_supported(int dtype, int D, int b1);
-int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* qa,
-                            const void* doa, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy,
-                            float* dc, void* ds2, int ds2_ld, const void* oa, const float* stats, int stats_ld, int unit0,
-                            hipStream_t stream);
+int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* q,
+                            const int64_t* qs, const void* dout, const void* out, const int64_t* os, const TokMap& qmap, int H,
+                            int unit0, const void* kbar, const void* y, const float* c, int c_rows, void* dkbar, void* dy, float* dc,
+                            void* ds2, int ds2_ld, const float* stats, int stats_ld, hipStream_t stream);
 // dq rows (caller's layout) = s dS2 Kbar per (unit, a, j) + the right factor's dQk; same limits as the left kernel
 int launch_monarch_bwd_dqa(int dtype, int D, int n, int b1, int b2, int AJ, int nf, float scale, const void* kbar, const void* ds2,
                            int ds2_ld, const float* dqk, float* dq, const int64_t* dqs, const TokMap& map, int H, int unit0,
                            hipStream_t stream);
 // fused right-factor part of the backward (monarch_bwd_right.hip): per tile t = (unit, k, f) the dS1 block (scratch, for
-// dQ = s dS1 K) and the finished dK / dV rows of kv block-frames [f0, f1) in the caller's tensors; v is the caller's tensor too
+// dQ = s dS1 K) and the finished dK / dV rows of kv block-frames [f0, f1) in the caller's tensors; q and v are the caller's tensors too
 bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ);
 int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, float scale, const void* kk, const void* v,
-                             const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* qk, void* ds1, void* dk,
-                             void* dv, const int64_t* dks, int64_t row0, const TokMap& kmap, int H, int unit0, int f0, int f1,
-                             hipStream_t stream);
+                             const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* q,
+                             const int64_t* qs, const TokMap& qmap, void* ds1, void* dk, void* dv, const int64_t* dks, int64_t row0,
+                             const TokMap& kmap, int H, int unit0, int f0, int f1, hipStream_t stream);
 
 // backward of the dense attention (dense_attn_bwd.hip); scratch is 2*B*H*q_tokens floats
 bool dense_bwd_supported(int dtype, int D);
