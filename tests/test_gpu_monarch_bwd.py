@@ -207,6 +207,28 @@ def test_each_fused_part_can_fall_back_to_the_library_chain(switch, monkeypatch)
     _close(vd.grad, vr.grad, dtype)
 
 
+def test_480p_block_shape_new_frame_gradients_only():
+    """b1 = 30, b2 = 52, D = 128: one query frame against a cache of three frames whose last one arrives with the call;
+    grad_only_new_kv, so that the right-factor kernel skips the gradient products of two of the three block-frames."""
+    h, w, H, D = 30, 52, 1, 128
+    dtype = torch.bfloat16
+    n = h * w
+    q0, do = (randn((1, n, H, D), 190 + i, dtype) for i in range(2))
+    k_old, v_old = (randn((1, 2 * n, H, D), 192 + i, dtype) for i in range(2))
+    k_new, v_new = (randn((1, n, H, D), 194 + i, dtype) for i in range(2))
+    qr, kor, vor, knr, vnr = (_leaf(t.double()) for t in (q0, k_old, v_old, k_new, v_new))
+    monarch.monarch_attn(qr, torch.cat([kor, knr], 1), torch.cat([vor, vnr], 1), 1, 1, 1, h, w).backward(do.double())
+    qd, knd, vnd = _leaf(q0, DEV), _leaf(k_new, DEV), _leaf(v_new, DEV)
+    kc = torch.zeros(1, 3 * n, H, D, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    kc[:, :2 * n], vc[:, :2 * n] = k_old.to(DEV), v_old.to(DEV)
+    out = mattn.monarch_attn_with_kv_cache(qd, kc, vc, knd, vnd, 2 * n, 3 * n, 1, 1, 1, h, w, grad_only_new_kv=True)
+    out.backward(do.to(DEV))
+    _close(qd.grad, qr.grad, dtype)
+    _close(knd.grad, knr.grad, dtype)
+    _close(vnd.grad, vnr.grad, dtype)
+
+
 def test_descriptor_errors():
     q = randn((1, 64, 1, 32), 140, torch.float32).to(DEV).requires_grad_(True)
     with pytest.raises(NotImplementedError):
