@@ -1,5 +1,5 @@
-// Right-factor part of the Monarch backward on gfx950 MFMA (bf16 / fp16, head_dim 64 or 128, b2 <= 64 a multiple of 4,
-// at most 160 (a, j) columns).
+// Right-factor part of the Monarch backward on gfx950 MFMA (bf16 / fp16, head_dim 64 or 128, b2 <= 64 a multiple of 4;
+// at most 480 (a, j) columns, taken 160 at a time).
 //
 // Replaces, per tile t = (unit, k, f), the small batched products and the row kernel of the GEMM chain
 //     dR[aj, l]  = dKbar[aj,:] . K[l,:] + dY[aj,:] . V[l,:]
@@ -69,7 +69,10 @@ __device__ __forceinline__ int br_swz(int r) {
 
 constexpr int kWaves = 16, kThreads = 64 * kWaves;
 
-template <class E, int D>
+// NP: passes over the tile, 160 columns each (with more than one the dS1 tile has LDS of its own).  The passes are
+// written out one after the other: as a loop, the invariant LDS addresses of all the transposing reads get hoisted
+// out of it and spill.
+template <class E, int D, int NP>
 __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p) {
     constexpr int DS = D / 16, DT = D / 32;
     constexpr int CPR = D / 8;                            // chunks per row of the D-wide tiles
@@ -78,9 +81,12 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
     constexpr int kG = kMaxAJ * kPitch;                   // dKbar or dY tile, 160 rows
     constexpr int kR = kMaxAJ * 128;                      // R tile, 160 rows of 64
     constexpr int oK = 0, oV = kKV, oG = 2 * kKV, oH = 2 * kKV + kG, oR = 2 * kKV + 2 * kG;
-    // dS1 tile (like R): over the K / V tiles after phase 1 where it fits there (head_dim 128), else behind the R tile
-    constexpr int oS = kR <= 2 * kKV ? 0 : oR + kR;
-    constexpr int oDot = oR + kR + (kR <= 2 * kKV ? 0 : kR);              // float [2][160]: per-column partial sums of the two l halves
+    // dS1 tile (like R): over the K / V tiles after phase 1 where it fits there and they are not needed again (head_dim
+    // 128, all columns in one pass), else behind the R tile
+    constexpr bool MULTI = NP > 1;
+    constexpr bool s_over_kv = kR <= 2 * kKV && !MULTI;
+    constexpr uint32_t oS = s_over_kv ? 0 : oR + kR;
+    constexpr uint32_t oDot = oR + kR + (s_over_kv ? 0 : kR);             // float [2][160]: per-column partial sums of the two l halves
     extern __shared__ __attribute__((aligned(256))) char lds[];
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
 
@@ -108,26 +114,6 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
     stage(p.kk + t * b2 * kPitch, kPitch, b2 * CPR, oK, c_d{});
     stage(p.v + ((int64_t)(unit / p.H) * p.vs0 + (int64_t)(unit % p.H) * p.vs2 + p.kmap.row(f, k) * p.vs1) * 2, (uint32_t)(p.vs1 * 2),
           b2 * CPR, oV, c_d{});
-    stage(p.dkbar + t * AJ * kPitch, kPitch, AJ * CPR, oG, c_d{});
-    stage(p.dy + t * AJ * kPitch, kPitch, AJ * CPR, oH, c_d{});
-    stage(p.rb + t * AJ * 128, 128, AJ * 8, oR, c_r{});
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    // rows past the end of a tile are zero, so that they add nothing to any contraction
-    {
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        for (int i = tid; i < (64 - b2) * CPR; i += kThreads) {
-            *(u32x4*)(lds + oK + b2 * kPitch + i * 16) = z;
-            *(u32x4*)(lds + oV + b2 * kPitch + i * 16) = z;
-        }
-        for (int i = tid; i < (kMaxAJ - AJ) * CPR; i += kThreads) {
-            *(u32x4*)(lds + oG + AJ * kPitch + i * 16) = z;
-            *(u32x4*)(lds + oH + AJ * kPitch + i * 16) = z;
-        }
-        for (int i = tid; i < (kMaxAJ - AJ) * 8; i += kThreads) *(u32x4*)(lds + oR + AJ * 128 + i * 16) = z;
-    }
-    __syncthreads();
-
     const bool want = f >= p.f0 && f < p.f1;                             // uniform: dK / dV of this kv block-frame are asked for
 
     // phase 2 operands: C^T[d, l] = sum_aj A^T[d, aj] B[aj, l]; a wave owns 32 head-dim rows x 32 key rows of dV (waves
@@ -137,9 +123,7 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
     const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
     const uint32_t sub = (uint32_t)(s16 & 1) * 8;
     const int dt = wave % DT, lb = (wave / DT) & 1, which = wave / (2 * DT);      // which: 0 dV, 1 dK, else idle
-    auto product = [&](uint32_t oA, uint32_t oB, f32x16& acc) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+    auto product = [&](uint32_t oA, uint32_t oB, f32x16& acc) {      // acc += ...
         const int ca = 4 * dt + cl, cb = 4 * lb + cl;
 #pragma unroll
         for (int ks = 0; ks < kMaxAJ / 16; ++ks) {
@@ -168,10 +152,41 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
         }
     };
 
-    // ---- phase 1 (waves 0..9 = (32 columns aj, 32 rows l) blocks of dS1), products: dR^T
-    const bool active = wave < 10;
+    const bool active = wave < 10;                                       // phase 1: waves 0..9 = (32 columns, 32 rows l) blocks of dS1
     const int cblk = wave % 5, tl = (wave / 5) & 1;
-    const int col = 32 * cblk + m;                                       // < 160
+    const int col = 32 * cblk + m;                                       // column within the pass, < 160
+    const char* qbase = p.q + ((int64_t)(unit / p.H) * p.qs0 + (int64_t)(unit % p.H) * p.qs2) * 2;
+    const uint32_t qrb = (uint32_t)(p.qs1 * 2);
+    f32x16 acc, accq;                                                    // dV^T, or R^T dKbar and dS1^T q of dK^T
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = accq[v] = 0.f;
+
+    // the tile's columns (a, j), up to 160 per pass
+    auto pass = [&](auto pi_c) {
+    constexpr int pi = decltype(pi_c)::value;
+    constexpr int c0 = pi * kMaxAJ;
+    const int nrows = MULTI ? min(kMaxAJ, AJ - c0) : AJ;
+    stage(p.dkbar + (t * AJ + c0) * kPitch, kPitch, nrows * CPR, oG, c_d{});
+    stage(p.dy + (t * AJ + c0) * kPitch, kPitch, nrows * CPR, oH, c_d{});
+    stage(p.rb + (t * AJ + c0) * 128, 128, nrows * 8, oR, c_r{});
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (nrows < kMaxAJ || c0 == 0) {                                     // rows past the end are zero: they add nothing to any contraction
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        if (c0 == 0)                                                     // K, V rows past b2: what the logits pick up there is masked, but must be finite
+            for (int i = tid; i < (64 - b2) * CPR; i += kThreads) {
+                *(u32x4*)(lds + oK + b2 * kPitch + i * 16) = z;
+                *(u32x4*)(lds + oV + b2 * kPitch + i * 16) = z;
+            }
+        for (int i = tid; i < (kMaxAJ - nrows) * CPR; i += kThreads) {
+            *(u32x4*)(lds + oG + nrows * kPitch + i * 16) = z;
+            *(u32x4*)(lds + oH + nrows * kPitch + i * 16) = z;
+        }
+        for (int i = tid; i < (kMaxAJ - nrows) * 8; i += kThreads) *(u32x4*)(lds + oR + nrows * 128 + i * 16) = z;
+        __syncthreads();
+    }
+
+    // ---- phase 1, products: dR^T
     f32x16 dr;
 #pragma unroll
     for (int v = 0; v < 16; ++v) dr[v] = 0.f;
@@ -188,11 +203,10 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
             dr = E::mfma32(av, bh, dr);
         }
     }
-    // ---- phase 2, the products that only need the loaded tiles: dV = R^T dY (finished), R^T dKbar
-    f32x16 acc;
+    // ---- phase 2, the products that only need the loaded tiles: dV += R^T dY, dK += R^T dKbar
     if (want) {
         if (which == 0) {
-            product(oH, oR, acc);                                        // stored at the end: a store in flight would hold up the wait for the query rows
+            product(oH, oR, acc);
         } else if (which == 1) {
             product(oG, oR, acc);
         }
@@ -200,13 +214,12 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
     __syncthreads();                                                     // K, V, dKbar, dY tiles are free
     // the query rows of (unit, k) take the place of the dY tile while the softmax backward runs
     if (want) {
-        const char* qbase = p.q + ((int64_t)(unit / p.H) * p.qs0 + (int64_t)(unit % p.H) * p.qs2) * 2;
-        const uint32_t qrb = (uint32_t)(p.qs1 * 2);
-        const int nchunks = AJ * CPR;
+        const int nchunks = nrows * CPR;
         for (int g = wave; g * 64 < nchunks; g += kWaves) {
             const int P = min(g * 64 + lane, nchunks - 1);
             const int r = P / CPR, c = (P % CPR) ^ br_swz<CPR>(r);
-            const uint32_t tok = (uint32_t)(p.qmap.row(r / b2, k) + r % b2);
+            const int aj = c0 + r;
+            const uint32_t tok = (uint32_t)(p.qmap.row(aj / b2, k) + aj % b2);
             br_load_lds16(qbase, tok * qrb + (uint32_t)(c * 16), lds0 + oH + (uint32_t)g * 1024);
         }
     }
@@ -215,7 +228,7 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
     float rv[16];
     float dot = 0.f;
     if (active) {
-        const float dcv = col < AJ ? p.dc[(u * AJ + col) * ((int64_t)nf * p.b1) + (int64_t)k * nf + f] : 0.f;
+        const float dcv = c0 + col < AJ ? p.dc[(u * AJ + c0 + col) * ((int64_t)nf * p.b1) + (int64_t)k * nf + f] : 0.f;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const int c = 4 * tl + g;
@@ -255,23 +268,30 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
     // dS1 to memory for dQ = s dS1 K: row aj is b2 consecutive elements, 8-byte pieces, consecutive lanes along a row
     {
         const int ppr = b2 / 4;                                          // pieces per row
-        uint16_t* out = p.ds1 + uk * AJ * ((int64_t)nf * b2) + (int64_t)f * b2;
-        for (int i = tid; i < AJ * ppr; i += kThreads) {
+        uint16_t* out = p.ds1 + (uk * AJ + c0) * ((int64_t)nf * b2) + (int64_t)f * b2;
+        for (int i = tid; i < nrows * ppr; i += kThreads) {
             const int row = i / ppr, pc = i % ppr;
             const u32x2 w = *(const u32x2*)(lds + oS + row * 128 + (((pc >> 1) ^ br_swz<8>(row)) << 4) + 8 * (pc & 1));
             *(u32x2*)(out + (int64_t)row * nf * b2 + 4 * pc) = w;
         }
     }
-    if (!want) return;
-    if ((AJ * CPR) % 64) {                                               // the last load spilled copies of a chunk into the zero rows
-        const u32x4 z = {0u, 0u, 0u, 0u};
-        for (int i = tid; i < (kMaxAJ - AJ) * CPR; i += kThreads) *(u32x4*)(lds + oH + AJ * kPitch + i * 16) = z;
-        __syncthreads();
+    if (want) {
+        if ((nrows * CPR) % 64) {                                        // the last load spilled copies of a chunk into the zero rows
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            for (int i = tid; i < (kMaxAJ - nrows) * CPR; i += kThreads) *(u32x4*)(lds + oH + nrows * kPitch + i * 16) = z;
+            __syncthreads();
+        }
+        // ---- phase 2, the product that needs dS1: dS1^T q
+        if (which == 1) product(oH, oS, accq);
     }
-    // ---- phase 2, the product that needs dS1: dK = R^T dKbar + s dS1^T q
+    if (pi + 1 < NP) __syncthreads();                                    // every wave is done with this pass's rows
+    };
+    pass(std::integral_constant<int, 0>{});
+    if constexpr (NP > 1) pass(std::integral_constant<int, 1>{});
+    if constexpr (NP > 2) pass(std::integral_constant<int, 2>{});
+    if (!want) return;
+    // dK = R^T dKbar + s dS1^T q
     if (which == 1) {
-        f32x16 accq;
-        product(oH, oS, accq);
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[v] += p.scale * accq[v];
         store(p.dk, acc);
@@ -283,7 +303,8 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
 }  // namespace
 
 bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ) {
-    return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 >= 4 && b2 <= 64 && b2 % 4 == 0 && AJ <= kMaxAJ;
+    // up to three passes of 160 columns over a tile
+    return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 >= 4 && b2 <= 64 && b2 % 4 == 0 && AJ <= 3 * kMaxAJ;
 }
 
 int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, float scale, const void* kk, const void* v,
@@ -309,11 +330,15 @@ int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, i
     a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.nf = nf; a.H = H; a.unit0 = unit0; a.f0 = f0; a.f1 = f1;
     a.scale = scale;
     const size_t kv = (size_t)2 * 64 * 2 * D, rt = (size_t)kMaxAJ * 128;
-    const size_t ldsb = kv + (size_t)2 * kMaxAJ * 2 * D + rt + (rt <= kv ? 0 : rt) + 2 * kMaxAJ * 4;
+    const size_t ldsb = kv + (size_t)2 * kMaxAJ * 2 * D + rt + (rt <= kv && AJ <= kMaxAJ ? 0 : rt) + 2 * kMaxAJ * 4;
+    const int np = (AJ + kMaxAJ - 1) / kMaxAJ;                         // 1, 2 or 3 (monarch_bwd_right_supported)
     const void* fn = nullptr;
-    if (dtype == SFM_BF16) fn = D == 128 ? (const void*)monarch_bwd_right_kernel<BF16, 128> : (const void*)monarch_bwd_right_kernel<BF16, 64>;
-    else fn = D == 128 ? (const void*)monarch_bwd_right_kernel<F16, 128> : (const void*)monarch_bwd_right_kernel<F16, 64>;
-    if (ldsb > 64 * 1024) {
+#define SFM_RIGHT_FN(E, D) \
+    (np == 1 ? (const void*)monarch_bwd_right_kernel<E, D, 1> : np == 2 ? (const void*)monarch_bwd_right_kernel<E, D, 2> : (const void*)monarch_bwd_right_kernel<E, D, 3>)
+    if (dtype == SFM_BF16) fn = D == 128 ? SFM_RIGHT_FN(BF16, 128) : SFM_RIGHT_FN(BF16, 64);
+    else fn = D == 128 ? SFM_RIGHT_FN(F16, 128) : SFM_RIGHT_FN(F16, 64);
+#undef SFM_RIGHT_FN
+    if (ldsb > 48 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsb);
         if (e != hipSuccess) {
             set_error("monarch backward (right factor): cannot reserve %zu bytes of LDS: %s", ldsb, hipGetErrorString(e));
@@ -321,12 +346,11 @@ int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, i
         }
     }
     const dim3 grid((unsigned)ntiles);
-    if (dtype == SFM_BF16) {
-        if (D == 128) hipLaunchKernelGGL((monarch_bwd_right_kernel<BF16, 128>), grid, dim3(kThreads), ldsb, stream, a);
-        else hipLaunchKernelGGL((monarch_bwd_right_kernel<BF16, 64>), grid, dim3(kThreads), ldsb, stream, a);
-    } else {
-        if (D == 128) hipLaunchKernelGGL((monarch_bwd_right_kernel<F16, 128>), grid, dim3(kThreads), ldsb, stream, a);
-        else hipLaunchKernelGGL((monarch_bwd_right_kernel<F16, 64>), grid, dim3(kThreads), ldsb, stream, a);
+    void* kargs[] = {(void*)&a};
+    hipError_t le = hipLaunchKernel(fn, grid, dim3(kThreads), kargs, ldsb, stream);
+    if (le != hipSuccess) {
+        set_error("monarch backward (right factor): launch failed: %s", hipGetErrorString(le));
+        return SFM_ERR_HIP;
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

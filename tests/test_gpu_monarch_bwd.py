@@ -146,7 +146,8 @@ def test_480p_block_shape_bf16_one_head(bwd_path):
 @pytest.mark.parametrize("h,w,Fq,Fk,D,causal,dtype", [
     (4, 52, 3, 3, 128, True, torch.bfloat16),      # 156 (a, j) columns: every fused kernel, last column block partial
     (4, 52, 3, 5, 64, False, torch.float16),
-    (4, 52, 4, 4, 64, True, torch.bfloat16),       # 208 columns: the right factor's blocks stay on the library products
+    (4, 52, 4, 4, 64, True, torch.bfloat16),       # 208 columns: two passes of the right-factor kernel over each tile
+    (4, 52, 7, 7, 128, False, torch.float16),      # 364 columns: three passes
     (5, 6, 2, 3, 64, False, torch.bfloat16),       # b2 = 6, not a multiple of 4: likewise
 ])
 def test_16bit_gradients_across_the_fused_kernels_limits(h, w, Fq, Fk, D, causal, dtype):
