@@ -407,6 +407,7 @@ struct Parts {
     bool fwd;      // 1-3: the forward's MFMA step 1 recomputes Kbar, Y, c and R straight into the scratch ([t][aj] rows)
     bool dqa;      // 8 and the scatter of dq: dQ of the left factor in its own kernel, which also adds the right factor's part
     bool right;    // 9, the right factor's softmax backward, 11-13 and the scatter of dk / dv in one kernel per tile t
+    bool dqk;      // 10 in a kernel that reads K where the caller has it (with `right`: no gathered copy of K is needed)
 };
 
 Parts make_parts(const MonarchArgs& p, int dtype, const int64_t* dks) {
@@ -417,9 +418,11 @@ Parts make_parts(const MonarchArgs& p, int dtype, const int64_t* dks) {
     f.left = h16 && q_rows_ok && monarch_bwd_left_supported(dtype, p.D, p.b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
     f.fwd = f.left && monarch_mfma_supported(dtype, p.D, p.b2) && getenv("SFM_BWD_FWD_GEMM") == nullptr;
     f.dqa = f.left && getenv("SFM_BWD_DQA_GEMM") == nullptr;
-    const bool direct_ok = (dks[0] | dks[1] | dks[2] | p.vs[0] | p.vs[1] | p.vs[2]) % 8 == 0;      // 16-byte rows of v, dk, dv
+    const bool direct_ok = (dks[0] | dks[1] | dks[2] | p.vs[0] | p.vs[1] | p.vs[2] | p.ks[0] | p.ks[1] | p.ks[2]) % 8 == 0 &&      // 16-byte rows of k, v, dk, dv
+                           (int64_t)p.nf * p.b1 * p.b2 * p.ks[1] * 2 < ((int64_t)1 << 32);
     f.right = f.fwd && direct_ok && monarch_bwd_right_supported(dtype, p.D, p.b2, p.na * p.b2) &&
               getenv("SFM_BWD_RIGHT_GEMM") == nullptr;
+    f.dqk = f.right && monarch_bwd_dqk_supported(dtype, p.D, p.b2, p.na * p.b2) && getenv("SFM_BWD_DQK_GEMM") == nullptr;
     return f;
 }
 
@@ -432,7 +435,7 @@ Layout make_layout(const MonarchArgs& p, int n, size_t e, const Parts& f) {
     l.Qk = take(!f.fwd || !f.right, n * MQ * D * e);
     l.Qa = take(!f.left, n * MQ * D * e);
     l.dOa = take(!f.left, n * MQ * D * e);
-    l.Kk = take(true, n * MK * D * e);
+    l.Kk = take(!f.dqk, n * MK * D * e);
     l.Vk = take(!f.right, n * MK * D * e);
     l.S1f = take(!f.fwd, n * p.b1 * AJ * NL * 4);
     l.dRb = take(!f.right, n * p.b1 * AJ * NL * 4);
@@ -529,8 +532,9 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
             hipLaunchKernelGGL((gather_rows<E>), dim3(gq), dim3(256), 0, stream, (T*)(ws + lay.dOa), g.dout, g.dos[0], g.dos[1], g.dos[2],
                                p.qmap, na, H, D, p.unit0, 1, tq);
         }
-        hipLaunchKernelGGL((gather_rows<E>), dim3(gk), dim3(256), 0, stream, (T*)(ws + lay.Kk), p.k, p.ks[0], p.ks[1], p.ks[2], p.kmap,
-                           nf, H, D, p.unit0, 0, tk);
+        if (!parts.dqk)
+            hipLaunchKernelGGL((gather_rows<E>), dim3(gk), dim3(256), 0, stream, (T*)(ws + lay.Kk), p.k, p.ks[0], p.ks[1], p.ks[2], p.kmap,
+                               nf, H, D, p.unit0, 0, tk);
         if (!fused_right)                               // the fused right-factor kernel reads v where it is
             hipLaunchKernelGGL((gather_rows<E>), dim3(gk), dim3(256), 0, stream, (T*)(ws + lay.Vk), p.v, p.vs[0], p.vs[1], p.vs[2], p.kmap,
                            nf, H, D, p.unit0, 0, tk);
@@ -612,7 +616,7 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     }
     if (fused_right) {
         if (!cx.status)
-            cx.status = launch_monarch_bwd_right(left_dtype<E>(), D, nt, b1, b2, AJ, nf, s, ws + lay.Kk, p.v, p.vs, ws + lay.Rb,
+            cx.status = launch_monarch_bwd_right(left_dtype<E>(), D, nt, b1, b2, AJ, nf, s, p.k, p.ks, p.v, p.vs, ws + lay.Rb,
                                                  ws + lay.dKbar, ws + lay.dY, (const float*)(ws + lay.dc), p.q, p.qs, p.qmap, ws + lay.dS1, g.dk,
                                                  g.dv, g.dks, g.dk_row0, p.kmap, H, p.unit0, g.kv_f0, g.kv_f1, stream);
     } else {
@@ -629,7 +633,13 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
         hipLaunchKernelGGL((softmax_right_bwd<E>), dim3((unsigned)((nseg + 3) / 4)), dim3(256), 0, stream, (const float*)(ws + lay.S1f),
                            (const float*)(ws + lay.dRb), (const float*)(ws + lay.dc), (T*)(ws + lay.dS1), b1, AJ, nf, b2, s, nseg);
     // 10. dQ (right factor) = s dS1 K per (u, k)
-    gemm(cx, false, false, AJ, D, NL, s, 0.f, dS1_uk, Kk_uk, dQk_uk, tE, tF, nuk);
+    if (parts.dqk) {
+        if (!cx.status)
+            cx.status = launch_monarch_bwd_dqk(left_dtype<E>(), D, nuk, b1, b2, AJ, nf, s, p.k, p.ks, p.kmap, ws + lay.dS1,
+                                               (float*)(ws + lay.dQk), H, p.unit0, stream);
+    } else {
+        gemm(cx, false, false, AJ, D, NL, s, 0.f, dS1_uk, Kk_uk, dQk_uk, tE, tF, nuk);
+    }
     if (!fused_right) {
         // 11. dK = s dS1^T q per (u, k)
         gemm(cx, true, false, NL, D, AJ, s, 0.f, dS1_uk, Qk_uk, dKk_uk, tE, tF, nuk);

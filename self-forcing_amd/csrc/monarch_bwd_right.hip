@@ -33,9 +33,9 @@ namespace {
 constexpr int kMaxAJ = 160;
 
 struct RightArgs {
-    const char* kk;          // [t][b2][D]
-    const char* v;           // caller's tensor: row kmap.row(f, k) + l, strides vs0 (batch), vs1 (row), vs2 (head), in elements
-    int64_t vs0, vs1, vs2;
+    const char* kk;          // callers' tensors: row kmap.row(f, k) + l, strides (batch, row, head) in elements
+    const char* v;
+    int64_t ks0, ks1, ks2, vs0, vs1, vs2;
     const char* rb;          // [t][AJ][64]
     const char* dkbar;       // [t][AJ][D]
     const char* dy;
@@ -111,7 +111,8 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
     using c_d = std::integral_constant<int, CPR>;
     using c_r = std::integral_constant<int, 8>;
     const int unit = p.unit0 + (int)u;
-    stage(p.kk + t * b2 * kPitch, kPitch, b2 * CPR, oK, c_d{});
+    stage(p.kk + ((int64_t)(unit / p.H) * p.ks0 + (int64_t)(unit % p.H) * p.ks2 + p.kmap.row(f, k) * p.ks1) * 2, (uint32_t)(p.ks1 * 2),
+          b2 * CPR, oK, c_d{});
     stage(p.v + ((int64_t)(unit / p.H) * p.vs0 + (int64_t)(unit % p.H) * p.vs2 + p.kmap.row(f, k) * p.vs1) * 2, (uint32_t)(p.vs1 * 2),
           b2 * CPR, oV, c_d{});
     const bool want = f >= p.f0 && f < p.f1;                             // uniform: dK / dV of this kv block-frame are asked for
@@ -300,6 +301,120 @@ __global__ __launch_bounds__(kThreads) void monarch_bwd_right_kernel(RightArgs p
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// dQ of the right factor: dQk[(u, k)][aj, :] = s sum_{f, l} dS1[(u, k)][aj, (f, l)] K[(f, k, l), :], float, for the
+// left-factor dQ kernel to add.  One workgroup per (unit, k), one wave per 32 columns (a, j); the K rows of the nf
+// block-frames stream through LDS 64 at a time straight from the caller's tensor (global_load_lds_dwordx4, double
+// buffered, chunk swizzle) and come back transposed as the B operand [n = d, k = (f, l)]; the A operand is dS1 straight
+// from memory, two 8-byte pieces per step in the order in which the transposing reads deliver the rows.
+struct DqkArgs {
+    const char* k;           // caller's tensor: row kmap.row(f, k) + l, strides ks0 (batch), ks1 (row), ks2 (head), in elements
+    int64_t ks0, ks1, ks2;
+    TokMap kmap;
+    const uint16_t* ds1;     // [(u, k)][AJ][nf * b2]
+    float* dqk;              // [(u, k)][AJ][D]
+    int b1, b2, AJ, nf, H, unit0;
+    float scale;
+};
+
+template <class E, int D>
+__global__ __launch_bounds__(1024) void monarch_bwd_dqk_kernel(DqkArgs p) {
+    constexpr int DT = D / 32, CPR = D / 8;
+    constexpr int kPitch = 2 * D;
+    constexpr int kTile = 64 * kPitch;
+    extern __shared__ __attribute__((aligned(256))) char lds[];          // two tiles of 64 K rows
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
+
+    const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nwaves = __builtin_amdgcn_readfirstlane((int)blockDim.x >> 6);
+    const int64_t uk = blockIdx.x;
+    const int k = (int)(uk % p.b1);
+    const int unit = p.unit0 + (int)(uk / p.b1);
+    const int b2 = p.b2, AJ = p.AJ, NL = p.nf * b2;
+    const int nt = (NL + 63) / 64;
+
+    const char* kbase = p.k + ((int64_t)(unit / p.H) * p.ks0 + (int64_t)(unit % p.H) * p.ks2) * 2;
+    const uint32_t krb = (uint32_t)(p.ks1 * 2);
+    // LDS position P (16-byte units) of a tile holds chunk (P % CPR) ^ swz(row) of row P / CPR; row x of the flat (f, l)
+    // axis is token kmap.row(x / b2, k) + x % b2 (rows past the end repeat the last one; dS1 is zero there)
+    auto stage = [&](int t) {
+        for (int g = wave; g < CPR; g += nwaves) {
+            const int P = g * 64 + lane;
+            const int r = P / CPR, c = (P % CPR) ^ br_swz<CPR>(r);
+            const int x = min(64 * t + r, NL - 1);
+            const uint32_t tok = (uint32_t)(p.kmap.row(x / b2, k) + x % b2);
+            br_load_lds16(kbase, tok * krb + (uint32_t)(c * 16), lds0 + (uint32_t)(t & 1) * kTile + (uint32_t)g * 1024);
+        }
+    };
+    // dS1 pieces of row aj = 32 wave + m: x = 64 t + 16 ks + 4 hf + {0..3} and + 8 + {0..3}
+    const int aj = min(32 * wave + m, AJ - 1);
+    const uint16_t* arow = p.ds1 + (uk * AJ + aj) * (int64_t)NL + 4 * hf;
+    auto load_a = [&](int t, u32x4 (&a)[4]) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const int x0 = 64 * t + 16 * ks + 4 * hf;
+            u32x2 lo = {0u, 0u}, hi = {0u, 0u};
+            if (x0 + 4 <= NL) lo = *(const u32x2*)(arow + 64 * t + 16 * ks);           // NL is a multiple of 4: whole pieces
+            if (x0 + 12 <= NL) hi = *(const u32x2*)(arow + 64 * t + 16 * ks + 8);
+            a[ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
+    };
+    uint32_t tr[DT][2];
+    {
+        const int s16 = lane & 15, g16 = lane >> 4;
+        const int rl = 4 * hf + (s16 >> 2);
+        const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int r = rl + 8 * half;             // swz depends on r mod 16 only
+                tr[dt][half] = (uint32_t)(r * kPitch + (((4 * dt + cl) ^ br_swz<CPR>(r)) << 4) + (s16 & 1) * 8);
+            }
+    }
+    f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[dt][v] = 0.f;
+
+    u32x4 acur[4], anext[4];
+    stage(0);
+    load_a(0, acur);
+    for (int t = 0; t < nt; ++t) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();                                   // tile t is in LDS; every wave is done with tile t - 1
+        if (t + 1 < nt) {
+            stage(t + 1);
+            load_a(t + 1, anext);
+        }
+        const char* tile = lds + (t & 1) * kTile;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const u32x2 lo = br_read_tr(tile, tr[dt][0] + ks * 16 * kPitch);
+                const u32x2 hi = br_read_tr(tile, tr[dt][1] + ks * 16 * kPitch);
+                const u32x4 bop = {lo.x, lo.y, hi.x, hi.y};
+                acc[dt] = E::mfma32(acur[ks], bop, acc[dt]);
+            }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) acur[ks] = anext[ks];
+    }
+    // lane (d = 32 dt + m) holds rows aj = 32 wave + 8 g + 4 hf + e
+    float* out = p.dqk + uk * AJ * D;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int row = 32 * wave + 8 * (v >> 2) + 4 * hf + (v & 3);
+        if (row < AJ) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) out[(int64_t)row * D + 32 * dt + m] = acc[dt][v] * p.scale;
+        }
+    }
+}
+
 }  // namespace
 
 bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ) {
@@ -307,18 +422,20 @@ bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ) {
     return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 >= 4 && b2 <= 64 && b2 % 4 == 0 && AJ <= 3 * kMaxAJ;
 }
 
-int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, float scale, const void* kk, const void* v,
-                             const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* q,
+int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, float scale, const void* kk,
+                             const int64_t* ks, const void* v, const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* q,
                              const int64_t* qs, const TokMap& qmap, void* ds1, void* dk, void* dv, const int64_t* dks, int64_t row0,
                              const TokMap& kmap, int H, int unit0, int f0, int f1, hipStream_t stream) {
-    if ((dks[0] | dks[1] | dks[2] | vs[0] | vs[1] | vs[2]) % 8 || ((uintptr_t)dk | (uintptr_t)dv | (uintptr_t)v) % 16 ||
-        (int64_t)(b2 - 1) * vs[1] * 2 + 2 * D > 0xffffffffll) {
-        set_error("monarch backward (right factor): v / dk / dv strides must be multiples of 8 elements and the pointers 16-byte aligned");
+    if ((dks[0] | dks[1] | dks[2] | vs[0] | vs[1] | vs[2] | ks[0] | ks[1] | ks[2]) % 8 ||
+        ((uintptr_t)dk | (uintptr_t)dv | (uintptr_t)v | (uintptr_t)kk) % 16 || (int64_t)(b2 - 1) * vs[1] * 2 + 2 * D > 0xffffffffll ||
+        (int64_t)(b2 - 1) * ks[1] * 2 + 2 * D > 0xffffffffll) {
+        set_error("monarch backward (right factor): k / v / dk / dv strides must be multiples of 8 elements and the pointers 16-byte aligned");
         return SFM_ERR_STRIDE;
     }
     RightArgs a;
     a.kk = (const char*)kk; a.rb = (const char*)rb;
     a.v = (const char*)v; a.vs0 = vs[0]; a.vs1 = vs[1]; a.vs2 = vs[2];
+    a.ks0 = ks[0]; a.ks1 = ks[1]; a.ks2 = ks[2];
     a.dkbar = (const char*)dkbar; a.dy = (const char*)dy;
     a.dc = dc;
     a.q = (const char*)q; a.qs0 = qs[0]; a.qs1 = qs[1]; a.qs2 = qs[2];
@@ -355,6 +472,42 @@ int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, i
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("monarch backward (right factor): launch failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+// at most 16 waves of 32 columns each
+bool monarch_bwd_dqk_supported(int dtype, int D, int b2, int AJ) {
+    return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 % 4 == 0 && AJ <= 512;
+}
+
+int launch_monarch_bwd_dqk(int dtype, int D, int64_t nuk, int b1, int b2, int AJ, int nf, float scale, const void* k, const int64_t* ks,
+                           const TokMap& kmap, const void* ds1, float* dqk, int H, int unit0, hipStream_t stream) {
+    if ((ks[0] | ks[1] | ks[2]) % 8 || ((uintptr_t)k) % 16 || (int64_t)nf * b1 * b2 * ks[1] * 2 > 0xffffffffll) {
+        set_error("monarch backward (dQ of the right factor): k rows must be 16-byte aligned and a (batch, head) slice under 4 GiB");
+        return SFM_ERR_STRIDE;
+    }
+    DqkArgs a;
+    a.k = (const char*)k; a.ks0 = ks[0]; a.ks1 = ks[1]; a.ks2 = ks[2];
+    a.kmap = kmap;
+    a.ds1 = (const uint16_t*)ds1;
+    a.dqk = dqk;
+    a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.nf = nf; a.H = H; a.unit0 = unit0;
+    a.scale = scale;
+    const int nwaves = (AJ + 31) / 32;
+    const size_t ldsb = (size_t)2 * 64 * 2 * D;
+    const dim3 grid((unsigned)nuk), block((unsigned)(64 * nwaves));
+    if (dtype == SFM_BF16) {
+        if (D == 128) hipLaunchKernelGGL((monarch_bwd_dqk_kernel<BF16, 128>), grid, block, ldsb, stream, a);
+        else hipLaunchKernelGGL((monarch_bwd_dqk_kernel<BF16, 64>), grid, block, ldsb, stream, a);
+    } else {
+        if (D == 128) hipLaunchKernelGGL((monarch_bwd_dqk_kernel<F16, 128>), grid, block, ldsb, stream, a);
+        else hipLaunchKernelGGL((monarch_bwd_dqk_kernel<F16, 64>), grid, block, ldsb, stream, a);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("monarch backward (dQ of the right factor): launch failed: %s", hipGetErrorString(e));
         return SFM_ERR_HIP;
     }
     return SFM_OK;

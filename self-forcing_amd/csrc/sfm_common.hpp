@@ -198,12 +198,17 @@ int launch_monarch_bwd_dqa(int dtype, int D, int n, int b1, int b2, int AJ, int 
                            int ds2_ld, const float* dqk, float* dq, const int64_t* dqs, const TokMap& map, int H, int unit0,
                            hipStream_t stream);
 // fused right-factor part of the backward (monarch_bwd_right.hip): per tile t = (unit, k, f) the dS1 block (scratch, for
-// dQ = s dS1 K) and the finished dK / dV rows of kv block-frames [f0, f1) in the caller's tensors; q and v are the caller's tensors too
+// dQ = s dS1 K) and the finished dK / dV rows of kv block-frames [f0, f1) in the caller's tensors; q, k and v are the caller's tensors too
 bool monarch_bwd_right_supported(int dtype, int D, int b2, int AJ);
-int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, float scale, const void* kk, const void* v,
-                             const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* q,
+int launch_monarch_bwd_right(int dtype, int D, int64_t ntiles, int b1, int b2, int AJ, int nf, float scale, const void* kk,
+                             const int64_t* ks, const void* v, const int64_t* vs, const void* rb, const void* dkbar, const void* dy, const float* dc, const void* q,
                              const int64_t* qs, const TokMap& qmap, void* ds1, void* dk, void* dv, const int64_t* dks, int64_t row0,
                              const TokMap& kmap, int H, int unit0, int f0, int f1, hipStream_t stream);
+
+// dQ of the right factor (monarch_bwd_right.hip): dqk[(u, k)][aj][:] = s sum_{f, l} dS1 K, float; k is the caller's tensor
+bool monarch_bwd_dqk_supported(int dtype, int D, int b2, int AJ);
+int launch_monarch_bwd_dqk(int dtype, int D, int64_t nuk, int b1, int b2, int AJ, int nf, float scale, const void* k, const int64_t* ks,
+                           const TokMap& kmap, const void* ds1, float* dqk, int H, int unit0, hipStream_t stream);
 
 // backward of the dense attention (dense_attn_bwd.hip); scratch is 2*B*H*q_tokens floats
 bool dense_bwd_supported(int dtype, int D);

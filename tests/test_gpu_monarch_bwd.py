@@ -190,7 +190,7 @@ def test_backward_with_and_without_the_forwards_saved_tensors(causal):
     assert stats32 is None
 
 
-@pytest.mark.parametrize("switch", ["SFM_BWD_LEFT_GEMM", "SFM_BWD_FWD_GEMM", "SFM_BWD_DQA_GEMM", "SFM_BWD_RIGHT_GEMM"])
+@pytest.mark.parametrize("switch", ["SFM_BWD_LEFT_GEMM", "SFM_BWD_FWD_GEMM", "SFM_BWD_DQA_GEMM", "SFM_BWD_RIGHT_GEMM", "SFM_BWD_DQK_GEMM"])
 def test_each_fused_part_can_fall_back_to_the_library_chain(switch, monkeypatch):
     """The measurement switches that put one fused part back on the batched GEMMs + row kernels (what also runs for
     shapes a fused kernel does not take): same gradients, and the workspace query follows the switch."""
