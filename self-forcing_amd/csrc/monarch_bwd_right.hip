@@ -18,7 +18,7 @@
 //            phase 1 is done with them), contraction over the columns aj.  The products with R run right after the
 //            logits of phase 1; the query rows of (unit, k) then load over the dY tile while the softmax backward runs.  dK and dV leave in the tensor dtype, straight to the caller's rows; tiles whose
 //            kv block-frame is outside the wanted range skip phase 2.
-// dS1 is also written to memory (16 bit) for dQ = s dS1 K, which contracts over f across tiles and stays a library GEMM.
+// dS1 is also written to memory (16 bit) for dQ = s dS1 K, which contracts over f across tiles (monarch_bwd_dqk_kernel below).
 
 #include <hip/hip_runtime.h>
 
