@@ -110,9 +110,12 @@ typedef struct sfm_monarch_bwd_desc {
 } sfm_monarch_bwd_desc;
 
 int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t heads_per_pass, size_t* bytes);
-/* 1 when the backward runs as batched rocBLAS GEMMs + row kernels (rocBLAS found at run time and SFM_BWD_SIMT
- * unset), 0 when it runs the fp32 SIMT kernels.  The first GEMM call on a device creates a rocBLAS handle,
- * which allocates; every other entry point of this header allocates nothing.  No counterpart in the reference. */
+/* 1 when rocBLAS was found at run time and SFM_BWD_SIMT is unset.  The backward is a chain of parts, each a fused
+ * MFMA kernel where the problem allows (16-bit tensors, head_dim 64 / 128, b1 <= 32, b2 <= 64 a multiple of 4, at
+ * most 480 (a, j) columns) and batched rocBLAS GEMMs + row kernels otherwise; when every part is fused the chain
+ * runs with or without rocBLAS, else without rocBLAS the fp32 SIMT kernels run.  The first GEMM call on a device
+ * creates a rocBLAS handle, which allocates; every other entry point of this header allocates nothing.  No
+ * counterpart in the reference. */
 int sfm_monarch_bwd_uses_gemm(void);
 int sfm_monarch_bwd(const sfm_monarch_bwd_desc* desc, const void* q, const void* k, const void* v, const void* dout,
                     float* dq, void* dk, void* dv, void* workspace, size_t workspace_bytes, void* stream);

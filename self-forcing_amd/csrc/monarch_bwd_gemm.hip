@@ -46,6 +46,7 @@ bool blas_load() {
     std::lock_guard<std::mutex> lock(g_blas_mutex);
     if (g_blas.tried) return g_blas.ok;
     g_blas.tried = true;
+    if (getenv("SFM_NO_ROCBLAS") != nullptr) return false;             // for tests: behave as where the library is absent
     void* lib = dlopen("librocblas.so.5", RTLD_NOW | RTLD_GLOBAL);
     if (!lib) lib = dlopen("/opt/rocm/lib/librocblas.so.5", RTLD_NOW | RTLD_GLOBAL);
     if (!lib) lib = dlopen("librocblas.so", RTLD_NOW | RTLD_GLOBAL);
@@ -463,6 +464,7 @@ struct Ctx {
     rocblas_handle h;
     char* ws;
     int status;
+    hipStream_t stream;
 };
 
 // one operand of a batched product: byte offset of batch 0 in the scratch, leading dimension and batch stride in elements
@@ -475,6 +477,11 @@ struct Op {
 void gemm(Ctx& cx, bool ta, bool tb, int M, int N, int K, float alpha, float beta, const Op& A, const Op& B, const Op& C,
           rocblas_datatype tab, rocblas_datatype tc, int batch) {
     if (cx.status) return;
+    if (!cx.h && (!blas_load() || !(cx.h = blas_handle(cx.stream)))) {
+        set_error("rocBLAS is needed for this shape and could not be loaded (or its handle not created)");
+        cx.status = SFM_ERR_UNSUPPORTED;
+        return;
+    }
     // column-major view: C^T[N,M] = op(B)^T op(A)^T
     void* c = cx.ws + C.off;
     rocblas_status st = g_blas.gemm(cx.h, tb ? rocblas_operation_transpose : rocblas_operation_none,
@@ -496,11 +503,7 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
     const Parts parts = make_parts(p, left_dtype<E>() >= 0 ? left_dtype<E>() : SFM_F32, g.dks);
     const Layout lay = make_layout(p, n, e, parts);
     char* ws = (char*)workspace;
-    Ctx cx{blas_handle(stream), ws, 0};
-    if (!cx.h) {
-        set_error("could not create a rocBLAS handle");
-        return SFM_ERR_HIP;
-    }
+    Ctx cx{nullptr, ws, 0, stream};                      // the rocBLAS handle is made by the first product that needs it
     const int b1 = p.b1, b2 = p.b2, nf = p.nf, na = p.na, D = p.D, H = p.H;
     const int AJ = na * b2, RR = nf * b1, NL = nf * b2;
     const int64_t MQ = (int64_t)b1 * AJ, MK = (int64_t)b1 * NL;
@@ -676,12 +679,17 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
 
 bool monarch_bwd_gemm_available() { return blas_load(); }
 
+bool monarch_bwd_all_fused(const MonarchArgs& p, int dtype, const int64_t* dkv_stride) {
+    const Parts f = make_parts(p, dtype, dkv_stride);
+    return f.left && f.fwd && f.dqa && f.right && f.dqk;
+}
+
 size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits, const int64_t* dkv_stride) {
     return make_layout(p, nunits, dtype == SFM_F32 ? 4 : 2, make_parts(p, dtype, dkv_stride)).total;
 }
 
 int launch_monarch_bwd_gemm(const MonarchBwdArgs& g, int dtype, int nunits, void* workspace, hipStream_t stream) {
-    if (!blas_load()) {
+    if (!monarch_bwd_all_fused(g.p, dtype, g.dks) && !blas_load()) {
         set_error("rocBLAS could not be loaded");
         return SFM_ERR_UNSUPPORTED;
     }

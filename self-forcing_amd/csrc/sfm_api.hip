@@ -412,6 +412,17 @@ static bool bwd_uses_gemm() {
 
 int sfm_monarch_bwd_uses_gemm(void) { return bwd_uses_gemm() ? 1 : 0; }
 
+// The chain of fused kernels and library products runs when rocBLAS is there, and also without it when every part of
+// the chain has a fused kernel for this problem.
+static bool bwd_uses_chain(const sfm_monarch_bwd_desc* desc, const MonarchPlan& pl) {
+    const char* e = getenv("SFM_BWD_SIMT");
+    if (e && atoi(e) != 0) return false;
+    if (monarch_bwd_gemm_available()) return true;
+    MonarchArgs a;
+    init_args(&desc->fwd, pl, &a);
+    return monarch_bwd_all_fused(a, desc->fwd.dtype, desc->dkv_stride);
+}
+
 int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t heads_per_pass, size_t* bytes) {
     if (!bytes) {
         set_error("bytes is NULL");
@@ -425,7 +436,7 @@ int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t he
         set_error("heads_per_pass must be >= 0");
         return SFM_ERR_SHAPE;
     }
-    if (bwd_uses_gemm()) {
+    if (bwd_uses_chain(desc, pl)) {
         MonarchArgs a;
         init_args(&desc->fwd, pl, &a);
         int n = heads_per_pass > 0 ? (heads_per_pass > pl.units ? pl.units : heads_per_pass) : pl.units;
@@ -483,7 +494,7 @@ static int monarch_bwd_impl(const sfm_monarch_bwd_desc* desc, const void* q, con
         set_error("workspace must be non-NULL and 256-byte aligned");
         return SFM_ERR_WORKSPACE;
     }
-    if (bwd_uses_gemm()) {
+    if (bwd_uses_chain(desc, pl)) {
         MonarchBwdArgs g;
         memset(&g, 0, sizeof(g));
         init_args(&desc->fwd, pl, &g.p);

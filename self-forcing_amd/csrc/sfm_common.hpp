@@ -182,6 +182,8 @@ bool monarch_mfma_supported(int dtype, int D, int b2);
 int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
 int launch_monarch_bwd(const MonarchBwdArgs& g, int dtype, int nunits, hipStream_t stream);
 bool monarch_bwd_gemm_available();
+// every part of the chain runs as a fused kernel for this problem: no library GEMM is called
+bool monarch_bwd_all_fused(const MonarchArgs& p, int dtype, const int64_t* dkv_stride);
 size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits, const int64_t* dkv_stride);
 int launch_monarch_bwd_gemm(const MonarchBwdArgs& g, int dtype, int nunits, void* workspace, hipStream_t stream);
 // step 1 of the MFMA forward alone, with the scratch strides of `a` and, if a.rb is set, the right factor written out

@@ -230,6 +230,37 @@ def test_480p_block_shape_new_frame_gradients_only():
     _close(vnd.grad, vnr.grad, dtype)
 
 
+def test_fused_chain_runs_without_rocblas():
+    """Where every part of the chain has a fused kernel no library product is called: a process that cannot load rocBLAS
+    (SFM_NO_ROCBLAS) gets the same gradients, bit for bit, as this one."""
+    import os
+    import subprocess
+    import sys
+    h, w, F, H, D = 4, 20, 2, 2, 64
+    code = f"""
+import sys, torch
+sys.path.insert(0, {os.path.dirname(os.path.abspath(__file__))!r}); sys.path.insert(0, {os.path.dirname(os.path.dirname(os.path.abspath(__file__)))!r})
+import self_forcing_amd as sfa
+from gpu_util import randn
+assert sfa.lib.load().sfm_monarch_bwd_uses_gemm() == int(sys.argv[1])
+q, do = (randn((1, {F * h * w}, {H}, {D}), 230 + i, torch.bfloat16).cuda() for i in range(2))
+k, v = (randn((1, {3 * h * w}, {H}, {D}), 232 + i, torch.bfloat16).cuda() for i in range(2))
+q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+sfa.monarch_attn.monarch_attn(q, k, v, 1, 1, 1, {h}, {w}).backward(do)
+print("SUM", *(float(t.grad.double().abs().sum()) for t in (q, k, v)))
+"""
+    outs = []
+    for no_blas in (False, True):
+        env = dict(os.environ)
+        env.pop("SFM_NO_ROCBLAS", None)
+        if no_blas:
+            env["SFM_NO_ROCBLAS"] = "1"
+        r = subprocess.run([sys.executable, "-c", code, "0" if no_blas else "1"], env=env, capture_output=True, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        outs.append([ln for ln in r.stdout.splitlines() if ln.startswith("SUM")][0])
+    assert outs[0] == outs[1]
+
+
 def test_descriptor_errors():
     q = randn((1, 64, 1, 32), 140, torch.float32).to(DEV).requires_grad_(True)
     with pytest.raises(NotImplementedError):
