@@ -1,4 +1,6 @@
-// Monarch attention backward as batched library GEMMs plus small element-wise kernels.
+// Monarch attention backward: the chain of its parts.  Each part runs as a fused MFMA kernel where the problem
+// allows (monarch_bwd_left.hip, monarch_bwd_right.hip, step 1 of monarch_mfma.hip; make_parts() decides) and
+// otherwise as batched library GEMMs plus small element-wise kernels, which is what this file holds.
 //
 // Every contraction of the backward (and of the forward it recomputes) is a plain matrix product once q, k, v
 // are gathered into block-row-major copies: per (unit, block row k) the logits are [a*b2 x D] . [D x f*b2],
@@ -9,7 +11,8 @@
 // softmaxes, the entropy term and their backward are row kernels in between.  Replaces _z_bwd_preprocess,
 // _z_bwd, _al_cl_y_bwd and their orchestration (wan/modules/monarch_attn.py:852-886, 1034-1222, 403-596,
 // 1326-1470, 1566-1693).  rocBLAS is resolved with dlopen on first use, so the library itself does not
-// depend on it; without it the fp32 SIMT kernels of monarch_generic.hip are used.
+// depend on it; without it the chain still runs where every part is fused, and the fp32 SIMT kernels of
+// monarch_generic.hip otherwise.
 //
 // Formulas (s = sm_scale, per unit): S1 = s q.k, R = softmax_l S1, Kbar = R K, Y = R V, c = sum_l R ln R,
 // S2 = s q.Kbar - c, L = softmax_(f,k) S2, O = L Y;
