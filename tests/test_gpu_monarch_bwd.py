@@ -168,10 +168,10 @@ def test_16bit_gradients_across_the_fused_kernels_limits(h, w, Fq, Fk, D, causal
 def test_backward_with_and_without_the_forwards_saved_tensors(causal):
     """sfm_monarch_bwd recomputes the left factor's row statistics; sfm_monarch_bwd_saved takes them (and the output)
     from sfm_monarch_fwd_stats.  Both against the float64 oracle, and the forward with statistics against the plain one."""
-    h, w, F, H, D = 4, 52, 3, 2, 128
+    h, w, F, H, D = 4, 52, 3, 3, 128
     dtype = torch.bfloat16
-    q0, do = (randn((1, F * h * w, H, D), 160 + i, dtype) for i in range(2))
-    k0, v0 = (randn((1, F * h * w, H, D), 162 + i, dtype) for i in range(2))
+    q0, do = (randn((2, F * h * w, H, D), 160 + i, dtype) for i in range(2))
+    k0, v0 = (randn((2, F * h * w, H, D), 162 + i, dtype) for i in range(2))
     kw = {"block_causal_size": h * w} if causal else {}
     qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
     monarch.monarch_attn(qr, kr, vr, 1, 1, 1, h, w, **kw).backward(do.double())
@@ -180,7 +180,10 @@ def test_backward_with_and_without_the_forwards_saved_tensors(causal):
     out, stats = mattn._monarch_fwd_stats(qd, kd, vd, tiling, D ** -0.5, 0, cbf)
     assert stats is not None and stats.dtype == torch.float32
     assert torch.equal(out, mattn.monarch_attn(qd, kd, vd, *tiling, **kw))
-    for kept in ({}, {"out": out, "stats": stats}):
+    # the statistics do not depend on how many (batch, head) units a pass of the forward takes
+    out4, stats4 = mattn._monarch_fwd_stats(qd, kd, vd, tiling, D ** -0.5, 0, cbf, heads_per_pass=4)
+    assert torch.equal(out, out4) and torch.equal(stats, stats4)
+    for kept in ({}, {"out": out, "stats": stats}, {"out": out, "stats": stats, "heads_per_pass": 4}):
         dq, dk, dv = mattn._monarch_bwd(qd, kd, vd, dod, tiling, D ** -0.5, 0, cbf, **kept)
         _close(dq, qr.grad, dtype)
         _close(dk, kr.grad, dtype)
