@@ -182,7 +182,9 @@ def test_backward_with_and_without_the_forwards_saved_tensors(causal):
     assert torch.equal(out, mattn.monarch_attn(qd, kd, vd, *tiling, **kw))
     # the statistics do not depend on how many (batch, head) units a pass of the forward takes
     out4, stats4 = mattn._monarch_fwd_stats(qd, kd, vd, tiling, D ** -0.5, 0, cbf, heads_per_pass=4)
-    assert torch.equal(out, out4) and torch.equal(stats, stats4)
+    # (one float per block row, rows padded to 32 per (unit, a, j): the padding is never written)
+    valid = lambda st: st.view(2 * H, F * w, 32)[..., :h]
+    assert torch.equal(out, out4) and torch.equal(valid(stats), valid(stats4))
     for kept in ({}, {"out": out, "stats": stats}, {"out": out, "stats": stats, "heads_per_pass": 4}):
         dq, dk, dv = mattn._monarch_bwd(qd, kd, vd, dod, tiling, D ** -0.5, 0, cbf, **kept)
         _close(dq, qr.grad, dtype)
