@@ -6,19 +6,23 @@
 //     dS1[aj, l] = R (dR + dc ln R - sum_l R (dR + dc ln R))
 //     dK[l, :]   = sum_aj R[aj, l] dKbar[aj,:] + s sum_aj dS1[aj, l] q[aj,:]
 //     dV[l, :]   = sum_aj R[aj, l] dY[aj,:]
-// (wan/modules/monarch_attn.py:403-596 `_al_cl_y_bwd`).  One workgroup per tile: the K and V blocks, the tile's rows of
-// R, dKbar and dY (all contiguous in the backward's scratch) go straight into LDS (global_load_lds_dwordx4, 16-byte
-// chunks XOR-swizzled per row as in the dense attention kernel), rows past the end are zeroed.
+// (wan/modules/monarch_attn.py:403-596 `_al_cl_y_bwd`).  One workgroup per tile: the K and V blocks (52 rows each, read
+// where the callers' tensors have them), and the tile's rows of R, dKbar and dY (contiguous in the backward's scratch)
+// go straight into LDS (global_load_lds_dwordx4, 16-byte chunks XOR-swizzled per row as in the dense attention
+// kernel); rows past the end are zeroed.  A tile with more than 160 columns is taken in passes of 160, the K and V
+// blocks and the accumulators of dK and dV staying where they are.
 // Sixteen waves per workgroup (one workgroup fills the LDS of a compute unit, so the waves have to come from it).
 //   phase 1: wave = 32 columns aj x 32 key rows l (ten waves busy).  dR^T[l, aj] with A = K / V rows, B = dKbar / dY
 //            rows, so that a lane owns one column and the softmax backward is in-lane plus one cross-half add and one
 //            exchange between the two waves of a column through LDS.
 //   phase 2: wave = 32 head-dim rows x 32 key rows of dV or of dK.  C^T[d, l] with both operands from transposing LDS
-//            reads (ds_read_tr16_b64): A = dY^T / dKbar^T / q^T, B = R or dS1 (kept in LDS, 16 bit, over the K / V tiles once
-//            phase 1 is done with them), contraction over the columns aj.  The products with R run right after the
-//            logits of phase 1; the query rows of (unit, k) then load over the dY tile while the softmax backward runs.  dK and dV leave in the tensor dtype, straight to the caller's rows; tiles whose
-//            kv block-frame is outside the wanted range skip phase 2.
-// dS1 is also written to memory (16 bit) for dQ = s dS1 K, which contracts over f across tiles (monarch_bwd_dqk_kernel below).
+//            reads (ds_read_tr16_b64): A = dY^T / dKbar^T / q^T, B = R or dS1 (kept in LDS, 16 bit; with a single pass
+//            over the K / V tiles once phase 1 is done with them), contraction over the columns aj.  The products
+//            with R run right after the logits of phase 1; the query rows of (unit, k) then load over the dY tile
+//            while the softmax backward runs.  dK and dV leave in the tensor dtype, straight to the caller's rows;
+//            tiles whose kv block-frame is outside the wanted range skip phase 2.
+// dS1 is also written to memory (16 bit) for dQ = s dS1 K, which contracts over f across tiles (monarch_bwd_dqk_kernel
+// below).
 
 #include <hip/hip_runtime.h>
 
