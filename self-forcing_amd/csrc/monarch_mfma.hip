@@ -5,8 +5,8 @@
 //  step 1 (right factor; replaces _al_cl_y_fwd, wan/modules/monarch_attn.py:109-253)
 //      work item = tile (unit, key block row k, kv block-frame f) against all (a, j) columns of a chunk of query
 //      block-frames; one workgroup per CU, each taking an equal contiguous share of the tile list.
-//      per tile: stage K[f,k,:,:], V[f,k,:,:] in LDS once (row-major K for the logits, transposed K^T / V^T for
-//      the contractions), and for ALL columns of the chunk
+//      per tile: K[f,k,:,:], V[f,k,:,:] go row-major into LDS once, straight from global memory (the contractions
+//      take K^T / V^T from transposing LDS reads), and for ALL columns of the chunk
 //          S^T[l,(a,j)] = K[f,k,l,:] . Q[a,k,j,:]           (MFMA, wave = 32 (a,j) columns)
 //          R = softmax_l(s S)       cl = sum_l R log2 R      (registers + one cross-half shuffle)
 //          Kbar^T = K^T R^T,  Y^T = V^T R^T                  (MFMA; R^T is fed straight from the
@@ -30,39 +30,54 @@ namespace sfm {
 // ------------------------------------------------------------------------------------------------
 // step 1
 // ------------------------------------------------------------------------------------------------
+// The K and V tiles are staged row-major (64 rows of 2 D bytes, 16-byte chunks XOR-swizzled per row) straight
+// from global memory into LDS (global_load_lds_dwordx4, two buffers per wave group) and the K^T / V^T operands of the
+// contractions are transposing LDS reads (ds_read_tr16_b64): no staging registers, no transposes written to LDS,
+// one barrier per tile.
+typedef short s1_s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2 s1_read_tr(const char* lds, uint32_t off) {
+    s1_s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s1_s16x4 __attribute__((address_space(3)))*)(lds + off));
+    return __builtin_bit_cast(u32x2, v);
+}
+__device__ __forceinline__ void s1_load_lds16(const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
+}
+template <int CPR>
+__device__ __forceinline__ int s1_swz(int r) {
+    return CPR >= 16 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
+}
 template <int D>
 struct S1Lds {
-    static constexpr int kRowPitch = D + 8;    // u16 per row of row-major K   [64][D+8]
-    static constexpr int kTPitch = 72;         // u16 per row of K^T / V^T     [D][64+8]
-    static constexpr int kElems = 64 * kRowPitch + 2 * D * kTPitch;
-    static __host__ __device__ constexpr size_t bytes() { return 2 * (size_t)kElems; }
+    static constexpr int kPitch = 2 * D, kTile = 64 * kPitch;
+    static constexpr int kGroup = 4 * kTile;                 // [buffer][K tile | V tile]
+    static __host__ __device__ constexpr size_t bytes() { return (size_t)kGroup; }
 };
 
+// NT: 32-row tiles of the key axis l (2 when b2 > 32).
 // WR: also write the right factor R (16 bit, 64 values per scratch row) to p.rb; the backward uses it.
-template <class E, int D, bool WR = false>
+template <class E, int D, int NT, bool WR = false>
 __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) void monarch_step1_kernel(MonarchArgs p) {
     using L = S1Lds<D>;
+    constexpr int CPR = D / 8;   // 16-byte chunks of a K/V row
     constexpr int DS = D / 16;   // contraction steps of the logits
-    constexpr int DP = D / 2;    // dword columns of a K/V row
-    extern __shared__ __attribute__((aligned(16))) uint16_t lds_all[];
+    extern __shared__ __attribute__((aligned(256))) char lds_s1[];
 
     // A workgroup is `p.s1_groups` independent wave groups that share nothing but the barriers, each with
     // its own LDS tiles.  Two groups of 5 waves put 3,3,2,2 waves on the four SIMDs, which one group of 5
     // cannot (waves go to SIMDs round-robin).
     const int G = p.s1_groups;
     const int nthreads = blockDim.x / G;                  // threads of one group
+    const int nwaves = nthreads >> 6;
     const int grp = __builtin_amdgcn_readfirstlane(threadIdx.x / nthreads);
     const int tid = threadIdx.x - grp * nthreads;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int m = lane & 31;
     const int hf = lane >> 5;
-    const uint32_t piece = (uint32_t)(4 * ((m >> 3) & 1) + 2 * ((m >> 4) & 1) + hf) * 16;   // see the output stores of step 1
+    const uint32_t piece = (uint32_t)(4 * ((m >> 3) & 1) + 2 * ((m >> 4) & 1) + hf) * 16;   // see the output stores below
 
-    uint16_t* const lds = lds_all + grp * L::kElems;
-    uint16_t* const lds_krow = lds;                                  // [64][D+8]
-    uint16_t* const lds_kt = lds + 64 * L::kRowPitch;                // [D][72]
-    uint16_t* const lds_vt = lds_kt + D * L::kTPitch;                // [D][72]
+    char* const lds = lds_s1 + grp * L::kGroup;
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
 
     // Work items are K/V tiles t = ((ul * b1 + k) * n_achunks + ac) * nf + f, i.e. one kv block row (f, k) of
     // one unit against the query rows Q[a, k, :, :] of one chunk of query block-frames.  The launch has one
@@ -75,15 +90,11 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int rounds = (t1 - t0 + G - 1) / G;
     const int mine = (t1 - t0 - grp + G - 1) / G;         // tiles of this group: t0 + grp, t0 + grp + G, ...
     if (mine <= 0) {                                      // still joins the barriers of the other group
-        for (int r = 0; r < rounds; ++r) {
-            lds_barrier();
-            lds_barrier();
-        }
+        for (int r = 0; r < rounds; ++r) lds_barrier();
         return;
     }
 
     const int b2 = p.b2;
-    const int NT = b2 > 32 ? 2 : 1;                       // 32-row tiles of the key axis l
     const uint32_t qs1 = (uint32_t)p.qs[1], ks1 = (uint32_t)p.ks[1];
     const uint32_t fstep = p.ws_f ? p.ws_f : (uint32_t)p.b1 * p.ws_row;     // scratch rows between consecutive f
 
@@ -103,104 +114,67 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         return x;
     };
 
-    // staging tasks: (sh = 2*s + hf', dword column pc); 8 rows perm_row(s, hf', 0..7) each.  With
-    // D = 128 the 64 lanes of a wave share sh.  A thread without a second task of its own repeats
-    // another thread's (same data to the same LDS words), so that every thread issues the same loads.
-    constexpr int kTasks = 8 * DP;
-    constexpr int kMaxTask = 2;                             // host launches >= kTasks/2 threads
-    const int ntask = (kTasks + nthreads - 1) / nthreads;
-    if (ntask > kMaxTask) return;                           // (checked on the host as well)
-    uint32_t pk[kMaxTask][8], pv[kMaxTask][8];
-    int tsh[kMaxTask];
-    uint32_t tcol[kMaxTask];                                // byte offset of dword column pc
-#pragma unroll
-    for (int t = 0; t < kMaxTask; ++t) {
-        int task = (tid + t * nthreads) % kTasks;
-        int sh = task / DP;
-        if (DP == 64) sh = __builtin_amdgcn_readfirstlane(sh);
-        tsh[t] = sh;
-        tcol[t] = (uint32_t)(task % DP) * 4;
-    }
-
-    // Rows past the end of a short tile (l >= b2) load row b2 - 1 again; their logits are masked below.
-    auto prefetch = [&](const Tile& x) {
+    // Tile x into buffer `buf`: LDS position P (in 16-byte units) holds chunk (P % CPR) ^ swz(row) of row P / CPR.
+    // Rows past the end of a short tile (l >= b2) load row b2 - 1 again; their logits are masked below.  Every wave
+    // issues the same number of loads for every tile, which the partial wait at the top of a round relies on.
+    auto stage = [&](const Tile& x, int buf) {
         const int unit = p.unit0 + x.ul;
         const int b = unit / p.H, h = unit % p.H;
         const char* kg = (const char*)p.k + ((int64_t)b * p.ks[0] + (int64_t)h * p.ks[2]) * 2;
         const char* vg = (const char*)p.v + ((int64_t)b * p.vs[0] + (int64_t)h * p.vs[2]) * 2;
         const uint32_t krow0 = (uint32_t)p.kmap.row(x.f, x.k);        // uniform
-#pragma unroll
-        for (int t = 0; t < kMaxTask; ++t) {
-            if (t < ntask) {
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int l = min(perm_row(tsh[t] >> 1, tsh[t] & 1, e), b2 - 1);
-                    const size_t rowb = (size_t)((krow0 + (uint32_t)l) * ks1) * 2;
-                    pk[t][e] = *(const uint32_t*)(kg + rowb + tcol[t]);
-                    pv[t][e] = *(const uint32_t*)(vg + rowb + tcol[t]);
-                }
-            }
+        const uint32_t dst = lds0 + (uint32_t)buf * 2 * L::kTile;
+        for (int g = wave; g < NT * (CPR / 2); g += nwaves) {         // 1 KB (64 / CPR rows) per step
+            const int P = g * 64 + lane;
+            const int r = P / CPR, c = (P % CPR) ^ s1_swz<CPR>(r);
+            const uint32_t off = (krow0 + (uint32_t)min(r, b2 - 1)) * ks1 * 2 + (uint32_t)c * 16;
+            s1_load_lds16(kg, off, dst + (uint32_t)g * 1024);
+            s1_load_lds16(vg, off, dst + L::kTile + (uint32_t)g * 1024);
         }
     };
-    auto commit = [&]() {
+    // K rows 32 t + m as the logits' A operand
+    const uint32_t a_off = (uint32_t)m * L::kPitch + (uint32_t)((hf ^ s1_swz<CPR>(m)) << 4);
+    // K^T / V^T as the contractions' A operand: rows = head-dim 32 dt + m, 16 key rows per step in the order the
+    // logits' accumulators hold them (two transposing reads of 4 x 4 blocks each)
+    uint32_t tr[D / 32][2];
+    {
+        const int s16 = lane & 15, g16 = lane >> 4;
+        const int rl = 4 * hf + (s16 >> 2);
+        const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
 #pragma unroll
-        for (int t = 0; t < kMaxTask; ++t) {
-            if (t < ntask) {
-                const int pc = tcol[t] >> 2, sh = tsh[t];
+        for (int dt = 0; dt < D / 32; ++dt)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    int l = perm_row(sh >> 1, sh & 1, e);
-                    *(uint32_t*)(lds_krow + l * L::kRowPitch + 2 * pc) = pk[t][e];
-                }
-                u32x4 lo, hi;
-                lo.x = lo16x2(pk[t][0], pk[t][1]); lo.y = lo16x2(pk[t][2], pk[t][3]);
-                lo.z = lo16x2(pk[t][4], pk[t][5]); lo.w = lo16x2(pk[t][6], pk[t][7]);
-                hi.x = hi16x2(pk[t][0], pk[t][1]); hi.y = hi16x2(pk[t][2], pk[t][3]);
-                hi.z = hi16x2(pk[t][4], pk[t][5]); hi.w = hi16x2(pk[t][6], pk[t][7]);
-                *(u32x4*)(lds_kt + (2 * pc) * L::kTPitch + sh * 8) = lo;
-                *(u32x4*)(lds_kt + (2 * pc + 1) * L::kTPitch + sh * 8) = hi;
-                lo.x = lo16x2(pv[t][0], pv[t][1]); lo.y = lo16x2(pv[t][2], pv[t][3]);
-                lo.z = lo16x2(pv[t][4], pv[t][5]); lo.w = lo16x2(pv[t][6], pv[t][7]);
-                hi.x = hi16x2(pv[t][0], pv[t][1]); hi.y = hi16x2(pv[t][2], pv[t][3]);
-                hi.z = hi16x2(pv[t][4], pv[t][5]); hi.w = hi16x2(pv[t][6], pv[t][7]);
-                *(u32x4*)(lds_vt + (2 * pc) * L::kTPitch + sh * 8) = lo;
-                *(u32x4*)(lds_vt + (2 * pc + 1) * L::kTPitch + sh * 8) = hi;
+            for (int half = 0; half < 2; ++half) {
+                const int r = rl + 8 * half;
+                tr[dt][half] = (uint32_t)(r * L::kPitch + (((4 * dt + cl) ^ s1_swz<CPR>(r)) << 4) + (s16 & 1) * 8);
             }
-        }
-    };
+    }
 
     const float sc2 = p.scale * kLog2e;
+    const f32x16 kZero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // Everything from the logits to the output stores runs without a branch, and a lane whose column
     // index is past the chunk's last column works on that last column again (same values to the same
-    // addresses).  The number of stores between a prefetch and the wait for it is then the same on
-    // every path, so that wait leaves the stores in flight instead of draining them.
+    // addresses).  The number of stores after a tile's loads is then the same on every path, so that the
+    // wait for the loads can leave those stores in flight instead of draining them.
     u32x4 qb[DS];                                          // logits operand (B): this lane's query row
     uint32_t crow[4] = {0, 0, 0, 0};                       // byte offsets in the (f, k) slab of the four scratch rows this lane stores to
     uint32_t cloff = 0;                                    // same for cl
     int qkey = -1;
 
-    // Makes the compiler wait here for loads into the given registers.  The waits it places are the most
-    // cautious over all paths that reach a use; closing a load's wait on the rarely taken path (kernel
-    // entry, change of query rows) keeps the wait in the steady-state loop as loose as that path allows.
-    auto settle4 = [](uint32_t& a, uint32_t& b, uint32_t& c, uint32_t& d) { asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d)); };
-
     Tile cur = decode(t0 + grp), nxt = cur;
-    prefetch(cur);
-#pragma unroll
-    for (int t = 0; t < kMaxTask; ++t) {
-        settle4(pk[t][0], pk[t][1], pk[t][2], pk[t][3]);
-        settle4(pk[t][4], pk[t][5], pk[t][6], pk[t][7]);
-        settle4(pv[t][0], pv[t][1], pv[t][2], pv[t][3]);
-        settle4(pv[t][4], pv[t][5], pv[t][6], pv[t][7]);
-    }
+    stage(cur, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     for (int r = 0; r < rounds; ++r) {
         const bool fresh = r < mine;     // in its last round a group may have no tile left: it repeats its previous one
-        lds_barrier();                   // previous iteration finished reading the tiles
-        if (fresh) {
-            cur = nxt;
-            commit();
-        }
+        // Vector memory operations complete in order: this wave's part of tile r has landed when only the Kbar / Y
+        // stores of the round before (the last 8 * D / 64 operations it issued) are outstanding.
+        if (D == 128) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        lds_barrier();                   // tile r is in LDS; every wave has finished reading the tile before it
+        if (fresh) cur = nxt;
+        const char* kt = lds + (r & 1) * 2 * L::kTile;
+        const char* vt = kt + L::kTile;
         const int key = (cur.ul * p.b1 + cur.k) * p.n_achunks + cur.a0;
         if (key != qkey) {
             qkey = key;
@@ -215,7 +189,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
 #pragma unroll
-            for (int ds = 0; ds < DS; ++ds) asm volatile("" : "+v"(qb[ds]));
+            for (int ds = 0; ds < DS; ++ds) asm volatile("" : "+v"(qb[ds]));      // waited for here, before the tile loads below
             cloff = (uint32_t)(ca * b2 + cj) * p.ws_aj * 4;
 #pragma unroll
             for (int rb = 0; rb < 4; ++rb) {
@@ -224,49 +198,40 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 crow[rb] = (uint32_t)((cur.a0 + sa) * b2 + (sg - sa * b2)) * p.ws_aj * (D * 2) + piece;
             }
         }
-        {
+        if (r + 1 < rounds) {
             // the tile after this one; past the end of the share the current tile is loaded again and dropped
             const int tn = t0 + grp + (r + 1) * G;
             nxt = decode(tn < t1 ? tn : t0 + grp + (mine - 1) * G);
-            prefetch(nxt);
+            stage(nxt, (r + 1) & 1);
         }
-        lds_barrier();                   // K/V tiles visible
 
         const uint32_t srow = (uint32_t)cur.ul * p.ws_unit + (uint32_t)cur.k * p.ws_row + (uint32_t)cur.f * fstep;
 
-        u32x4 pb[4];                     // R^T as B operands, 16 contraction rows per step
+        u32x4 pb[2 * NT];                // R^T as B operands, 16 contraction rows per step
         {
-            f32x16 s[2];
+            f32x16 s[NT];
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < NT; ++t)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) s[t][v] = 0.f;
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                if (t < NT) {
-                    const uint16_t* arow = lds_krow + (32 * t + m) * L::kRowPitch + 8 * hf;
-#pragma unroll
-                    for (int ds = 0; ds < DS; ++ds) {
-                        u32x4 a = *(const u32x4*)(arow + 16 * ds);
-                        s[t] = E::mfma32(a, qb[ds], s[t]);
-                    }
+                for (int ds = 0; ds < DS; ++ds) {
+                    const u32x4 a = *(const u32x4*)(kt + 32 * t * L::kPitch + (a_off ^ (uint32_t)(ds << 5)));
+                    s[t] = E::mfma32(a, qb[ds], ds ? s[t] : kZero);
                 }
-            }
-            // block softmax over l (rows of S^T): 16*NT values here, the rest in lane ^ 32
+            // block softmax over l (rows of S^T): 16 NT values here, the rest in lane ^ 32
             float mx = -INFINITY;
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < NT; ++t)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     int l = 32 * t + 8 * (v >> 2) + 4 * hf + (v & 3);
-                    float zz = (t < NT && l < b2) ? s[t][v] * sc2 : kMaskLogit;
+                    float zz = l < b2 ? s[t][v] * sc2 : kMaskLogit;
                     s[t][v] = zz;
                     mx = fmaxf(mx, zz);
                 }
             mx = xhalf_max(mx);
             float sum = 0.f, ent = 0.f;
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < NT; ++t)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     float zz = s[t][v];
@@ -280,7 +245,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             const float inv_l = 1.f / sum;
             // R = e / sum is rounded to 16 bit once, as the reference's right factor is
 #pragma unroll
-            for (int st = 0; st < 4; ++st) {
+            for (int st = 0; st < 2 * NT; ++st) {
                 const int t = st >> 1, v0 = 8 * (st & 1);
                 pb[st].x = pack2<E>(s[t][v0 + 0] * inv_l, s[t][v0 + 1] * inv_l);
                 pb[st].y = pack2<E>(s[t][v0 + 2] * inv_l, s[t][v0 + 3] * inv_l);
@@ -294,13 +259,11 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 // 12..15; exchanging the lower half's second pair with the upper half's first leaves 8 consecutive values
                 char* rrow = (char*)p.rb + ((size_t)srow + cloff / 4) * 128 + 16 * hf;
 #pragma unroll
-                for (int st = 0; st < 4; ++st) {
-                    if (st < 2 * NT) {
-                        auto rx = __builtin_amdgcn_permlane32_swap(pb[st].x, pb[st].z, false, false);
-                        auto ry = __builtin_amdgcn_permlane32_swap(pb[st].y, pb[st].w, false, false);
-                        const u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
-                        *(u32x4*)(rrow + 32 * st) = w;
-                    }
+                for (int st = 0; st < 2 * NT; ++st) {
+                    auto rx = __builtin_amdgcn_permlane32_swap(pb[st].x, pb[st].z, false, false);
+                    auto ry = __builtin_amdgcn_permlane32_swap(pb[st].y, pb[st].w, false, false);
+                    const u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+                    *(u32x4*)(rrow + 32 * st) = w;
                 }
             }
         }
@@ -314,7 +277,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         // (c & 7) + 8 rb, so that one store instruction writes 128 contiguous bytes of each of 8 rows.
 #pragma unroll
         for (int which = 0; which < 2; ++which) {
-            const uint16_t* tbase = which == 0 ? lds_kt : lds_vt;
+            const char* tbase = which == 0 ? kt : vt;
             char* og = (char*)(which == 0 ? p.kbar : p.y) + (size_t)srow * (D * 2);
 #pragma unroll
             for (int dp = 0; dp < D / 64; ++dp) {
@@ -324,14 +287,11 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                     const int dt = 2 * dp + dl;
                     f32x16 acc;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-                    const uint16_t* arow = tbase + (32 * dt + m) * L::kTPitch + 8 * hf;
-#pragma unroll
-                    for (int st = 0; st < 4; ++st) {
-                        if (st < 2 * NT) {
-                            u32x4 a = *(const u32x4*)(arow + 16 * st);
-                            acc = E::mfma32(a, pb[st], acc);
-                        }
+                    for (int st = 0; st < 2 * NT; ++st) {
+                        const u32x2 lo = s1_read_tr(tbase, tr[dt][0] + st * 16 * L::kPitch);
+                        const u32x2 hi = s1_read_tr(tbase, tr[dt][1] + st * 16 * L::kPitch);
+                        const u32x4 a = {lo.x, lo.y, hi.x, hi.y};
+                        acc = E::mfma32(a, pb[st], st ? acc : kZero);
                     }
 #pragma unroll
                     for (int gp = 0; gp < 2; ++gp) {
@@ -345,8 +305,8 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                     // lane bit 4 <-> gp: slot 0 then holds rows (c & 15), slot 1 rows (c & 15) + 16
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        auto r = __builtin_amdgcn_permlane16_swap(w[dl][0][q], w[dl][1][q], false, false);
-                        w[dl][0][q] = r[0]; w[dl][1][q] = r[1];
+                        auto x = __builtin_amdgcn_permlane16_swap(w[dl][0][q], w[dl][1][q], false, false);
+                        w[dl][0][q] = x[0]; w[dl][1][q] = x[1];
                     }
                 }
                 // lane bit 3 <-> block within the pair
@@ -360,7 +320,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                         lo[q] = (uint32_t)__builtin_amdgcn_update_dpp((int)a, (int)b, 0x128, 0xf, 0xc, false);
                         hi[q] = (uint32_t)__builtin_amdgcn_update_dpp((int)b, (int)a, 0x128, 0xf, 0x3, false);
                     }
-// Non-temporal: the rows are read exactly once, by step 2, after the whole grid has finished.
+                    // Non-temporal: the rows are read exactly once, by step 2, after the whole grid has finished.
                     // Ordinary stores leave them dirty in the caches and their write-back then competes with
                     // step 2's reads (measured at 4680 x 32760, 12 heads: step 1 +15 us, step 2 -45 us).
                     __builtin_nontemporal_store(lo, (u32x4*)(og + crow[2 * r4 + 0] + 128 * dp));
@@ -591,20 +551,22 @@ int cu_count() {
     return cached;
 }
 
+// Enqueues step 1 (with the right factor written too when a.rb is set).
 template <class E, int D>
-static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const StepEvents* ev) {
+static int enqueue_step1(const MonarchArgs& a, int nunits, hipStream_t stream) {
     const int ncols = a.a_chunk * a.b2;
     const int ntiles = (ncols + 31) / 32;
-    const int nwaves = ntiles < 4 ? 4 : ntiles;   // at least 4 waves so that K/V staging is <= 2 tasks per thread
-    if (ntiles < 1 || nwaves > 8 || (8 * (D / 2) + nwaves * 64 - 1) / (nwaves * 64) > 2) {
+    const int nwaves = ntiles < 4 ? 4 : ntiles;   // a wave per 32 (a, j) columns, at least 4 to share the tile loads
+    if (ntiles < 1 || nwaves > 8) {
         set_error("internal: step-1 launch shape (a_chunk=%d, b2=%d)", a.a_chunk, a.b2);
         return SFM_ERR_UNSUPPORTED;
     }
     const int groups = nwaves <= 5 ? 2 : 1;             // wave groups per workgroup (<= 10 waves in all)
     const size_t lds1 = S1Lds<D>::bytes() * groups;
+    const void* fn = a.b2 > 32 ? (a.rb ? (const void*)monarch_step1_kernel<E, D, 2, true> : (const void*)monarch_step1_kernel<E, D, 2, false>)
+                               : (a.rb ? (const void*)monarch_step1_kernel<E, D, 1, true> : (const void*)monarch_step1_kernel<E, D, 1, false>);
     if (lds1 > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)monarch_step1_kernel<E, D>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1);
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1);
         if (e != hipSuccess) {
             set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
             return SFM_ERR_HIP;
@@ -616,9 +578,21 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const 
     // one workgroup per CU (a CU holds one: 3 waves per SIMD), fewer when there are not two tiles for each
     int wgs = a.s1_wgs > 0 ? a.s1_wgs : cu_count();
     if (wgs > (a1.s1_total + groups - 1) / groups) wgs = (a1.s1_total + groups - 1) / groups;
-    dim3 g1(wgs);
+    void* args[] = {&a1};
+    hipError_t e = hipLaunchKernel(fn, dim3(wgs), dim3(nwaves * 64 * groups), args, lds1, stream);
+    if (e != hipSuccess) {
+        set_error("hip launch failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+template <class E, int D>
+static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const StepEvents* ev) {
     if (ev) (void)hipEventRecord(ev->ev[0], stream);
-    hipLaunchKernelGGL((monarch_step1_kernel<E, D>), g1, dim3(nwaves * 64 * groups), lds1, stream, a1);
+    MonarchArgs a0 = a;
+    a0.rb = nullptr;
+    if (int rc = enqueue_step1<E, D>(a0, nunits, stream)) return rc;
     if (ev) (void)hipEventRecord(ev->ev[1], stream);
     const int njg = (a.b2 + 3) / 4;
     dim3 g2(a.na * njg, nunits, (a.b1 + 31) / 32);
@@ -634,36 +608,7 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const 
 
 template <class E, int D>
 static int launch_step1_t(const MonarchArgs& a, int nunits, hipStream_t stream) {
-    const int ncols = a.a_chunk * a.b2;
-    const int ntiles = (ncols + 31) / 32;
-    const int nwaves = ntiles < 4 ? 4 : ntiles;
-    if (ntiles < 1 || nwaves > 8 || (8 * (D / 2) + nwaves * 64 - 1) / (nwaves * 64) > 2) {
-        set_error("internal: step-1 launch shape (a_chunk=%d, b2=%d)", a.a_chunk, a.b2);
-        return SFM_ERR_UNSUPPORTED;
-    }
-    const int groups = nwaves <= 5 ? 2 : 1;
-    const size_t lds1 = S1Lds<D>::bytes() * groups;
-    const void* fn = a.rb ? (const void*)monarch_step1_kernel<E, D, true> : (const void*)monarch_step1_kernel<E, D, false>;
-    if (lds1 > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1);
-        if (e != hipSuccess) {
-            set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
-            return SFM_ERR_HIP;
-        }
-    }
-    MonarchArgs a1 = a;
-    a1.s1_total = a.nf * a.b1 * nunits * a.n_achunks;
-    a1.s1_groups = groups;
-    int wgs = a.s1_wgs > 0 ? a.s1_wgs : cu_count();
-    if (wgs > (a1.s1_total + groups - 1) / groups) wgs = (a1.s1_total + groups - 1) / groups;
-    if (a.rb) hipLaunchKernelGGL((monarch_step1_kernel<E, D, true>), dim3(wgs), dim3(nwaves * 64 * groups), lds1, stream, a1);
-    else hipLaunchKernelGGL((monarch_step1_kernel<E, D, false>), dim3(wgs), dim3(nwaves * 64 * groups), lds1, stream, a1);
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess) {
-        set_error("hip launch failed: %s", hipGetErrorString(err));
-        return SFM_ERR_HIP;
-    }
-    return SFM_OK;
+    return enqueue_step1<E, D>(a, nunits, stream);
 }
 
 int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream) {
