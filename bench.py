@@ -170,6 +170,15 @@ def op_level(torch, sfa, args):
     copy_gbs = 5 * 2 * (1 << 30) / (e0.elapsed_time(e1) * 1e-3) / 1e9
     del src, dst
 
+    # step 1's memory traffic with nothing else (same tile count, rows and scatter, non-temporal stores): what this
+    # machine's memory system takes for the bytes alone
+    tiles, rows_in, rows_out, row_bytes = B * H * B1 * F, B2, A * B2, 2 * D
+    ws = torch.empty(tiles * (2 * rows_in + 2 * rows_out) * row_bytes, dtype=torch.uint8, device=dev)
+    ws.zero_()
+    floor_us = C.c_float(0)
+    L.check(lib.sfm_probe_tile_traffic(tiles, rows_in, rows_out, row_bytes, 1, ws.data_ptr(), ws.numel(), stream, C.byref(floor_us)))
+    del ws
+
     s1_gbs = STEP1_BYTES / (s1_ms * 1e-3) / 1e9
     s2_gbs = STEP2_BYTES / (s2_ms * 1e-3) / 1e9
     tfl = MONARCH_FLOPS / (ms_call * 1e-3) / 1e12
@@ -186,7 +195,8 @@ def op_level(torch, sfa, args):
         "roofline": {"kernel": "monarch_step1_kernel (configs[1] shape)", "bound": "hbm", "achieved": s1_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s1_gbs / HBM_PEAK_GBS,
                      "algorithmic_bytes": STEP1_BYTES, "traffic": MEASURED_TRAFFIC["monarch_step1_kernel"],
-                     "copy_probe_gbs": copy_gbs, "frac_of_copy_probe": s1_gbs / copy_gbs},
+                     "copy_probe_gbs": copy_gbs, "frac_of_copy_probe": s1_gbs / copy_gbs,
+                     "traffic_only_us": floor_us.value, "frac_of_traffic_only": floor_us.value / (s1_ms * 1e3)},
         "roofline_step2": {"kernel": "monarch_step2_kernel (configs[1] shape)", "bound": "hbm", "achieved": s2_gbs,
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s2_gbs / HBM_PEAK_GBS,
                            "algorithmic_bytes": STEP2_BYTES, "traffic": MEASURED_TRAFFIC["monarch_step2_kernel"],

@@ -268,6 +268,16 @@ int sfm_vae_norm_act(int32_t dtype, int32_t T, int32_t H, int32_t W, int32_t C, 
  * reports the dense kernel against it beside the nominal peak. */
 int sfm_probe_mfma_bf16(int32_t iters, void* stream, float* tflops);
 
+/* Measurement aid with no counterpart in the reference: the memory traffic of the Monarch forward's step 1 and nothing
+ * else.  `tiles` work items in equal contiguous shares over two workgroups per compute unit; item t reads 2 x rows_in
+ * rows of row_bytes (contiguous) and writes rows_out rows of row_bytes to each of two matrices, row r of item t at row
+ * index r * tiles + t (the scatter of step 1's scratch), with non-temporal stores if `nontemporal` != 0.  The caller
+ * supplies `workspace` (device memory, 16-byte aligned, >= tiles * (2 rows_in + 2 rows_out) * row_bytes bytes; its
+ * contents are read and overwritten).  Runs on `stream`, waits, and returns the mean duration of one pass in
+ * microseconds: the floor for this traffic on this machine, which bench.py reports beside step 1's own duration. */
+int sfm_probe_tile_traffic(int32_t tiles, int32_t rows_in, int32_t rows_out, int32_t row_bytes, int32_t nontemporal,
+                           void* workspace, size_t workspace_bytes, void* stream, float* us);
+
 /* Thread-local description of the last error returned on this thread ("" if none). */
 const char* sfm_last_error(void);
 

@@ -49,6 +49,34 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(int iters) {
     if (s == 12345.678f) sfm_probe_sink[0] = s;                 // keeps the accumulators alive; never true in practice
 }
 
+// Memory traffic of the Monarch forward's step 1 with nothing else: `tiles` work items in gridDim.x equal contiguous
+// shares; item t reads 2 x rows_in rows of 16 x chunks bytes (contiguous, at t) and writes rows_out rows to each of two
+// matrices, row r of item t at row index r * tiles + t (the scatter of the (a, j)-major scratch).
+template <bool NT>
+__global__ __launch_bounds__(320) void tile_traffic_kernel(const u32x4* in, u32x4* o0, u32x4* o1, int tiles, int rows_in, int rows_out, int chunks) {
+    const int tid = threadIdx.x;
+    const int t0 = (int)((int64_t)blockIdx.x * tiles / gridDim.x), t1 = (int)((int64_t)(blockIdx.x + 1) * tiles / gridDim.x);
+    const int nin = 2 * rows_in * chunks, nout = rows_out * chunks;
+    for (int t = t0; t < t1; ++t) {
+        u32x4 acc = {0u, 0u, 0u, 0u};
+        const u32x4* src = in + (size_t)t * nin;
+        for (int c = tid; c < nin; c += 320) {
+            const u32x4 v = src[c];
+            acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
+        }
+        for (int c = tid; c < nout; c += 320) {
+            const size_t at = ((size_t)(c / chunks) * tiles + t) * chunks + c % chunks;
+            if (NT) {
+                __builtin_nontemporal_store(acc, o0 + at);
+                __builtin_nontemporal_store(acc, o1 + at);
+            } else {
+                o0[at] = acc;
+                o1[at] = acc;
+            }
+        }
+    }
+}
+
 }  // namespace
 }  // namespace sfm
 
@@ -80,5 +108,49 @@ extern "C" int sfm_probe_mfma_bf16(int32_t iters, void* stream, float* tflops) {
     }
     const double flops = (double)wgs * 4 * (double)iters * 16 * (2.0 * 32 * 32 * 16);
     *tflops = (float)(flops / (ms * 1e-3) / 1e12);
+    return SFM_OK;
+}
+
+extern "C" int sfm_probe_tile_traffic(int32_t tiles, int32_t rows_in, int32_t rows_out, int32_t row_bytes, int32_t nontemporal,
+                                      void* workspace, size_t workspace_bytes, void* stream, float* us) {
+    using namespace sfm;
+    if (tiles < 1 || rows_in < 1 || rows_out < 1 || row_bytes < 16 || row_bytes % 16 || workspace == nullptr || us == nullptr) {
+        set_error("sfm_probe_tile_traffic: tiles, rows_in, rows_out >= 1, row_bytes a multiple of 16, workspace and us non-null");
+        return SFM_ERR_RANGE;
+    }
+    const size_t in_bytes = (size_t)tiles * 2 * rows_in * row_bytes, out_bytes = (size_t)tiles * rows_out * row_bytes;
+    if (in_bytes + 2 * out_bytes > workspace_bytes || ((uintptr_t)workspace & 15)) {
+        set_error("sfm_probe_tile_traffic: workspace of %zu bytes, 16-byte aligned, needed", in_bytes + 2 * out_bytes);
+        return SFM_ERR_WORKSPACE;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        set_error("sfm_probe_tile_traffic: hipEventCreate failed");
+        return SFM_ERR_HIP;
+    }
+    const u32x4* in = (const u32x4*)workspace;
+    u32x4* o0 = (u32x4*)((char*)workspace + in_bytes);
+    u32x4* o1 = (u32x4*)((char*)workspace + in_bytes + out_bytes);
+    const int wgs = tiles < 2 * cu_count() ? tiles : 2 * cu_count();
+    const int reps = 5;
+    auto launch = [&] {
+        if (nontemporal) hipLaunchKernelGGL(tile_traffic_kernel<true>, dim3(wgs), dim3(320), 0, st, in, o0, o1, tiles, rows_in, rows_out, row_bytes / 16);
+        else hipLaunchKernelGGL(tile_traffic_kernel<false>, dim3(wgs), dim3(320), 0, st, in, o0, o1, tiles, rows_in, rows_out, row_bytes / 16);
+    };
+    launch();                                                // warm-up
+    (void)hipEventRecord(e0, st);
+    for (int i = 0; i < reps; ++i) launch();
+    (void)hipEventRecord(e1, st);
+    hipError_t e = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (e != hipSuccess || ms <= 0.f) {
+        set_error("sfm_probe_tile_traffic: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    *us = ms * 1e3f / reps;
     return SFM_OK;
 }

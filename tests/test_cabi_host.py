@@ -232,3 +232,17 @@ def test_mfma_probe_rejects_bad_arguments_before_any_launch():
     assert lib.sfm_probe_mfma_bf16(0, None, C.byref(out)) == -4
     assert lib.sfm_probe_mfma_bf16(100, None, None) == -4
     assert b"iters" in lib.sfm_last_error()
+
+
+def test_traffic_probe_rejects_bad_arguments_before_any_launch():
+    lib = L.load()
+    out = C.c_float(0)
+    fake = C.c_void_p(4096)                                   # never dereferenced: every call below fails the checks
+    assert lib.sfm_probe_tile_traffic(0, 52, 156, 256, 1, fake, 1 << 30, None, C.byref(out)) == -4
+    assert lib.sfm_probe_tile_traffic(10, 52, 156, 250, 1, fake, 1 << 30, None, C.byref(out)) == -4
+    assert lib.sfm_probe_tile_traffic(10, 52, 156, 256, 1, None, 1 << 30, None, C.byref(out)) == -4
+    assert lib.sfm_probe_tile_traffic(10, 52, 156, 256, 1, fake, 1 << 30, None, None) == -4
+    need = 10 * (2 * 52 + 2 * 156) * 256
+    assert lib.sfm_probe_tile_traffic(10, 52, 156, 256, 1, fake, need - 1, None, C.byref(out)) == -6
+    assert str(need).encode() in lib.sfm_last_error()
+    assert lib.sfm_probe_tile_traffic(10, 52, 156, 256, 1, C.c_void_p(4100), need, None, C.byref(out)) == -6

@@ -133,3 +133,36 @@ def test_mfma_probe_reports_a_rate():
     out = C.c_float(0)
     L.check(lib.sfm_probe_mfma_bf16(2000, None, C.byref(out)))
     assert 10.0 < out.value < 5000.0       # TFLOP/s; the nominal peak is 2500
+
+
+@pytest.mark.gpu
+def test_traffic_probe_moves_the_bytes_and_reports_a_duration():
+    import ctypes as C
+    from self_forcing_amd import lib as L
+    lib = L.load()
+    tiles, rows_in, rows_out, row_bytes = 300, 52, 156, 256
+    nin = tiles * 2 * rows_in * row_bytes
+    nout = tiles * rows_out * row_bytes
+    for nt in (0, 1):
+        ws = torch.zeros(nin + 2 * nout, dtype=torch.uint8, device="cuda")
+        ws[:nin] = torch.randint(0, 256, (nin,), dtype=torch.uint8, device="cuda")
+        ws[nin:] = 0xEE
+        src = ws[:nin].clone()
+        out = C.c_float(0)
+        L.check(lib.sfm_probe_tile_traffic(tiles, rows_in, rows_out, row_bytes, nt, ws.data_ptr(), ws.numel(), None, C.byref(out)))
+        torch.cuda.synchronize()
+        assert 0.1 < out.value < 1e5           # microseconds per pass
+        assert torch.equal(ws[:nin], src)      # the input region is only read
+        o0 = ws[nin:nin + nout].view(rows_out, tiles, row_bytes // 16, 16)
+        o1 = ws[nin + nout:].view(rows_out, tiles, row_bytes // 16, 16)
+        assert torch.equal(o0, o1)
+        # every 16-byte piece of item t holds the xor of the pieces one thread read: thread x reads pieces x, x + 320, ...
+        pieces = src.view(tiles, 2 * rows_in * row_bytes // 16, 16)
+        t = 7
+        want = torch.zeros(320, 16, dtype=torch.uint8, device="cuda")
+        for c0 in range(0, pieces.shape[1], 320):
+            blk = pieces[t, c0:c0 + 320]
+            want[:blk.shape[0]] ^= blk
+        got = o0[:, t].reshape(-1, 16)          # piece c of the item's output comes from thread c % 320
+        idx = torch.arange(got.shape[0], device="cuda") % 320
+        assert torch.equal(got, want[idx])
