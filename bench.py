@@ -32,7 +32,7 @@ STEP2_BYTES = 2 * ROWS * D * 2 + ROWS * 4 + 2 * SQ * H * D * 2              # re
 
 # HBM bytes per launch measured with rocprofv3 (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 1 GiB
 # device copy in the same run); the runs and raw counters are in profiles/monarch_step{1,2}_c2.md.
-MEASURED_TRAFFIC = {"monarch_step1_kernel": 881.0e6, "monarch_step2_kernel": 647.2e6}
+MEASURED_TRAFFIC = {"monarch_step1_kernel": 881.0e6, "monarch_step2_kernel": 637.6e6}
 
 LAYERS, CHUNKS, PASSES = 30, 7, 5
 

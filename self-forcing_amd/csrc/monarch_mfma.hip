@@ -15,10 +15,11 @@
 //      v_permlane32_swap per dword pair leaves 8 consecutive head-dim elements per lane (16-byte stores).
 //
 //  step 2 (left factor; replaces _z_fwd, monarch_attn.py:698-842)
-//      wave = (unit, a, j): streams its contiguous Kbar / Y rows once,
+//      wave = (unit, a, j): streams its contiguous Kbar / Y rows once, 32 rows at a time, through its own part of
+//      LDS (global_load_lds_dwordx4, one chunk ahead; no barriers: a wave waits for its own loads only),
 //          S2^T[(f,k), i] = Kbar[(f,k),:] . Q[a,i,j,:]  - cl       online softmax over (f,k)
 //          O^T[d, i]     += Y^T[d,(f,k)] P^T[(f,k), i]
-//      Y^T operands are built in registers from dword loads of 8 rows (no LDS, no transpose pass).
+//      with the Y^T operands from transposing LDS reads and the query rows in registers.
 //
 // The running output stays in fp32 for the whole KV range (the reference rounds it to 16 bit
 // between KV chunks, monarch_attn.py:795,838).
@@ -334,22 +335,32 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 // ------------------------------------------------------------------------------------------------
 // step 2
 // ------------------------------------------------------------------------------------------------
+// Per wave: two buffers of [Kbar chunk | Y chunk | cl values], a chunk being 32 scratch rows of 2 D bytes, row-major
+// with the 16-byte pieces XOR-swizzled per row as in step 1.
 template <int D>
 struct S2Lds {
-    static constexpr int kPitch = D + 8;             // u16 per row of a wave's [32][D+8] region
-    static constexpr int kPerWave = 32 * kPitch;
-    static __host__ __device__ constexpr size_t bytes() { return 2 * (size_t)(4 * kPerWave); }
+    static constexpr int kPitch = 2 * D, kTile = 32 * kPitch;
+    static constexpr int kBuf = 2 * kTile + 256;
+    static constexpr int kWave = 2 * kBuf;
+    static __host__ __device__ constexpr size_t bytes() { return 4 * (size_t)kWave; }
 };
 
+__device__ __forceinline__ void s2_load_lds4(const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
+}
+
+// The four waves of a workgroup share nothing: each streams the rows of its own (a, j) through its own part of LDS
+// (global_load_lds_dwordx4, 1 KB contiguous per instruction, one chunk ahead of the one being contracted) and
+// synchronises with its own loads only (vector memory operations complete in order, so waiting until one chunk's
+// worth of them is outstanding means the chunk before has landed).
 template <class E, int D>
 __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
     using L = S2Lds<D>;
-    constexpr int DS = D / 16;
-    constexpr int DPn = D / 64;          // 64-wide head-dim spans, each giving an even and an odd 32-row tile
-    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    constexpr int DS = D / 16, DT = D / 32, CPR = D / 8;
+    extern __shared__ __attribute__((aligned(256))) char lds_s2[];
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int m = lane & 31;
     const int hf = lane >> 5;
@@ -369,93 +380,96 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
     const int r_lim = f_lim * p.b1;
     const int nch = (r_lim + 31) / 32;
 
-    const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj;   // in rows
-    const uint16_t* kb = (const uint16_t*)p.kbar + blk * D;
-    const uint16_t* yb = (const uint16_t*)p.y + blk * D;
-    const float* clp = p.cl + blk;
-    constexpr uint32_t rstride = D;                 // rows of one (a, j) are consecutive (ws_row == 1)
+    const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj;   // in rows; the rows of one (a, j) are consecutive
+    const char* kb = (const char*)p.kbar + blk * (2 * D);
+    const char* yb = (const char*)p.y + blk * (2 * D);
+    const char* clp = (const char*)(p.cl + blk);
 
-    uint16_t* wl = lds + wave * L::kPerWave;
+    char* const wl = lds_s2 + wave * L::kWave;
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)wl;
 
-    // stage the wave's query rows Q[a, i0 + 0..31, j, :] (zero rows past b1)
+    // logits operand (B): this lane's query row Q[a, i0 + m, j, :] (zero past b1)
+    u32x4 qb[DS];
     {
         const uint16_t* qg = (const uint16_t*)p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[2];
-        constexpr int CH = D / 8;                      // 16-byte chunks per row
-        for (int c = lane; c < 32 * CH; c += 64) {
-            int r = c / CH, ch = c % CH;
-            int i = i0 + r;
-            u32x4 w = {0u, 0u, 0u, 0u};
-            if (i < p.b1) w = *(const u32x4*)(qg + (p.qmap.row(a, i) + j) * p.qs[1] + ch * 8);
-            *(u32x4*)(wl + r * L::kPitch + ch * 8) = w;
+        const int i = min(i0 + m, p.b1 - 1);
+        const uint16_t* qrow = qg + (p.qmap.row(a, i) + j) * p.qs[1] + 8 * hf;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) asm volatile("" : "+v"(qb[ds]));       // waited for here, before the first chunk's loads
+        if (i0 + m >= p.b1) {
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds) qb[ds] = u32x4{0u, 0u, 0u, 0u};
         }
     }
-    __syncthreads();
+
+    // chunk n into buffer `buf`: CPR + 1 loads per lane.  Rows past the valid range may hold anything: the last valid
+    // row is read instead (the rows' weights are exactly zero).
+    auto issue = [&](int n, int buf) {
+        const uint32_t dst = lds0 + (uint32_t)buf * L::kBuf;
+#pragma unroll
+        for (int g = 0; g < CPR / 2; ++g) {
+            const int P = g * 64 + lane;
+            const int r = P / CPR, c = (P % CPR) ^ s1_swz<CPR>(r);
+            const uint32_t off = (uint32_t)min(32 * n + r, r_lim - 1) * (2 * D) + (uint32_t)c * 16;
+            s1_load_lds16(kb, off, dst + (uint32_t)g * 1024);
+            s1_load_lds16(yb, off, dst + L::kTile + (uint32_t)g * 1024);
+        }
+        s2_load_lds4(clp, (uint32_t)(32 * n + m) * 4, dst + 2 * L::kTile);     // cl of the chunk's 32 rows (twice)
+    };
+    const uint32_t a_off = (uint32_t)m * L::kPitch + (uint32_t)((hf ^ s1_swz<CPR>(m)) << 4);   // Kbar row m as the logits' A operand
+    uint32_t tr[DT][2];            // Y^T as the output's A operand: transposing reads, as in step 1
+    {
+        const int s16 = lane & 15, g16 = lane >> 4;
+        const int rl = 4 * hf + (s16 >> 2);
+        const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int r = rl + 8 * half;
+                tr[dt][half] = (uint32_t)(r * L::kPitch + (((4 * dt + cl) ^ s1_swz<CPR>(r)) << 4) + (s16 & 1) * 8);
+            }
+    }
 
     const float sc2 = p.scale * kLog2e;
-    f32x16 oacc[DPn][2];
+    const f32x16 kZero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    f32x16 oacc[DT];               // O^T[d = 32 dt + 8 g + 4 hf + e, i = m]
 #pragma unroll
-    for (int dp = 0; dp < DPn; ++dp)
-#pragma unroll
-        for (int par = 0; par < 2; ++par)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) oacc[dp][par][v] = 0.f;
+    for (int dt = 0; dt < DT; ++dt) oacc[dt] = kZero;
     float mrun = -INFINITY, lrun = 0.f;
 
-    u32x4 kcur[DS];
-    f32x4 ccur[4];
-    uint32_t ycur[2][DPn][8];
-
-    auto load_k = [&](int n) {
-        const uint16_t* row = kb + (uint32_t)(32 * n + m) * rstride + 8 * hf;
-#pragma unroll
-        for (int ds = 0; ds < DS; ++ds) kcur[ds] = *(const u32x4*)(row + 16 * ds);
-    };
-    auto load_c = [&](int n) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) ccur[g] = *(const f32x4*)(clp + 32 * n + 8 * g + 4 * hf);
-    };
-    auto load_y = [&](int n) {
-#pragma unroll
-        for (int st = 0; st < 2; ++st)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                int r = 32 * n + perm_row(st, hf, e);
-                const uint16_t* row = yb + (uint32_t)r * rstride + 2 * m;
-#pragma unroll
-                for (int dp = 0; dp < DPn; ++dp) {
-                    uint32_t w = *(const uint32_t*)(row + 64 * dp);
-                    ycur[st][dp][e] = r < r_lim ? w : 0u;     // rows past the valid range may hold anything
-                }
-            }
-    };
-
-    // Single-buffered software pipeline: each operand set is re-loaded for chunk n+1 as soon as
-    // chunk n has consumed it, so that about one chunk of Kbar and Y rows is in flight per wave.
-    load_k(0);
-    load_c(0);
-    load_y(0);
+    issue(0, 0);
     for (int n = 0; n < nch; ++n) {
-        const int nn = min(n + 1, nch - 1);
+        if (n + 1 < nch) {
+            issue(n + 1, (n + 1) & 1);
+            if (D == 128) asm volatile("s_waitcnt vmcnt(17)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        const char* kt = wl + (n & 1) * L::kBuf;
+        const char* yt = kt + L::kTile;
 
         f32x16 s;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = 0.f;
-#pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
-            u32x4 qb = *(const u32x4*)(wl + m * L::kPitch + 16 * ds + 8 * hf);
-            s = E::mfma32(kcur[ds], qb, s);
+            const u32x4 ak = *(const u32x4*)(kt + (a_off ^ (uint32_t)(ds << 5)));
+            s = E::mfma32(ak, qb[ds], ds ? s : kZero);
         }
-        load_k(nn);
+        f32x4 cc[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) cc[g] = *(const f32x4*)(kt + 2 * L::kTile + (8 * g + 4 * hf) * 4);
 
         float mx = -INFINITY;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             int r = 32 * n + 8 * (v >> 2) + 4 * hf + (v & 3);
-            float z = r < r_lim ? s[v] * sc2 - ccur[v >> 2][v & 3] : -INFINITY;
+            float z = r < r_lim ? s[v] * sc2 - cc[v >> 2][v & 3] : -INFINITY;
             s[v] = z;
             mx = fmaxf(mx, z);
         }
-        load_c(nn);
         mx = xhalf_max(mx);
         const float mnew = fmaxf(mrun, mx);        // finite: chunk n has at least one valid row
         const float alpha = exp2f(mrun - mnew);
@@ -476,55 +490,42 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
             pb[st].z = pack2<E>(s[8 * st + 4], s[8 * st + 5]);
             pb[st].w = pack2<E>(s[8 * st + 6], s[8 * st + 7]);
         }
-
 #pragma unroll
-        for (int dp = 0; dp < DPn; ++dp) {
+        for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
-            for (int par = 0; par < 2; ++par)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) oacc[dp][par][v] *= alpha;
+            for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
 #pragma unroll
             for (int st = 0; st < 2; ++st) {
-                const uint32_t* yy = ycur[st][dp];
-                u32x4 ae, ao;
-                ae.x = lo16x2(yy[0], yy[1]); ae.y = lo16x2(yy[2], yy[3]);
-                ae.z = lo16x2(yy[4], yy[5]); ae.w = lo16x2(yy[6], yy[7]);
-                ao.x = hi16x2(yy[0], yy[1]); ao.y = hi16x2(yy[2], yy[3]);
-                ao.z = hi16x2(yy[4], yy[5]); ao.w = hi16x2(yy[6], yy[7]);
-                oacc[dp][0] = E::mfma32(ae, pb[st], oacc[dp][0]);
-                oacc[dp][1] = E::mfma32(ao, pb[st], oacc[dp][1]);
+                const u32x2 lo = s1_read_tr(yt, tr[dt][0] + st * 16 * L::kPitch);
+                const u32x2 hi = s1_read_tr(yt, tr[dt][1] + st * 16 * L::kPitch);
+                const u32x4 ay = {lo.x, lo.y, hi.x, hi.y};
+                oacc[dt] = E::mfma32(ay, pb[st], oacc[dt]);
             }
         }
-        load_y(nn);
     }
 
-    // epilogue: O[i, d] = O^T / l, through the wave's LDS region (the query rows are dead now)
+    // epilogue: O[i, d] = O^T / l, turned through the wave's LDS (the operand buffers are dead: every load has landed)
     const float ltot = xhalf_sum(lrun);
     const float inv = 1.f / ltot;
     if (p.stats != nullptr && hf == 0 && j_ok && i0 + m < p.b1)
         p.stats[((int64_t)unit * (p.na * b2) + a * b2 + j) * p.stats_ld + i0 + m] = mrun + log2f(ltot);
-    __syncthreads();
 #pragma unroll
-    for (int dp = 0; dp < DPn; ++dp)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            // accumulator row mr = 8g + 4hf + v%4 of tile (dp, par) is head-dim 64dp + 2mr + par
-            u32x4 w;
-            w.x = pack2<E>(oacc[dp][0][4 * g + 0] * inv, oacc[dp][1][4 * g + 0] * inv);
-            w.y = pack2<E>(oacc[dp][0][4 * g + 1] * inv, oacc[dp][1][4 * g + 1] * inv);
-            w.z = pack2<E>(oacc[dp][0][4 * g + 2] * inv, oacc[dp][1][4 * g + 2] * inv);
-            w.w = pack2<E>(oacc[dp][0][4 * g + 3] * inv, oacc[dp][1][4 * g + 3] * inv);
-            *(u32x4*)(wl + m * L::kPitch + 64 * dp + 2 * (8 * g + 4 * hf)) = w;
+            u32x2 w;
+            w.x = pack2<E>(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
+            w.y = pack2<E>(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
+            *(u32x2*)(wl + m * L::kPitch + (32 * dt + 8 * g + 4 * hf) * 2) = w;
         }
-    __syncthreads();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     {
         uint16_t* og = (uint16_t*)p.out + (int64_t)b * p.os[0] + (int64_t)h * p.os[2];
-        constexpr int CH = D / 8;
-        for (int c = lane; c < 32 * CH; c += 64) {
-            int r = c / CH, ch = c % CH;
+        for (int c = lane; c < 32 * CPR; c += 64) {
+            int r = c / CPR, ch = c % CPR;
             int i = i0 + r;
             if (i < p.b1 && j_ok) {
-                u32x4 w = *(const u32x4*)(wl + r * L::kPitch + ch * 8);
+                u32x4 w = *(const u32x4*)(wl + r * L::kPitch + ch * 16);
                 *(u32x4*)(og + (p.qmap.row(a, i) + j) * p.os[1] + ch * 8) = w;
             }
         }
@@ -596,6 +597,14 @@ static int launch_t(const MonarchArgs& a, int nunits, hipStream_t stream, const 
     if (ev) (void)hipEventRecord(ev->ev[1], stream);
     const int njg = (a.b2 + 3) / 4;
     dim3 g2(a.na * njg, nunits, (a.b1 + 31) / 32);
+    {
+        hipError_t e = hipFuncSetAttribute((const void*)monarch_step2_kernel<E, D>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)S2Lds<D>::bytes());
+        if (e != hipSuccess) {
+            set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+            return SFM_ERR_HIP;
+        }
+    }
     hipLaunchKernelGGL((monarch_step2_kernel<E, D>), g2, dim3(256), S2Lds<D>::bytes(), stream, a);
     if (ev) (void)hipEventRecord(ev->ev[2], stream);
     hipError_t err = hipGetLastError();
