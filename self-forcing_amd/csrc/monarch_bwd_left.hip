@@ -16,6 +16,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "sfm_attn.h"
 #include "sfm_common.hpp"
 
@@ -50,14 +52,43 @@ __device__ __forceinline__ u32x2 bl_read_tr(const char* lds, uint32_t off) {
     return __builtin_bit_cast(u32x2, v);
 }
 
-template <class E, int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void monarch_bwd_left_kernel(LeftArgs p) {
-    constexpr int DS = D / 16, DT = D / 32;
-    constexpr int kPitch = (D + 8) * 2;                   // bytes per staged row
-    constexpr int kPerWave = 2 * 32 * kPitch + 128;       // q rows, then dO rows, then 32 floats
-    extern __shared__ __attribute__((aligned(16))) char lds[];
+template <int CPR>
+__device__ __forceinline__ int bl_swz(int r) {
+    return CPR >= 16 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
+}
+__device__ __forceinline__ void bl_load_lds16(const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
+}
+// the same with the LDS address as a scalar base plus a compile-time offset (one scalar register for all of a chunk's loads)
+template <int OFF>
+__device__ __forceinline__ void bl_load_lds16_at(const char* base, uint32_t off, uint32_t lds_base) {
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(off), "s"(base), "n"(OFF) : "memory", "m0", "scc");
+}
+template <int OFF>
+__device__ __forceinline__ void bl_load_lds4_at(const char* base, uint32_t off, uint32_t lds_base) {
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_base), "v"(off), "s"(base), "n"(OFF) : "memory", "m0", "scc");
+}
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, m = lane & 31, hf = lane >> 5;
+// LDS per wave: q rows, dO rows, 32 floats, then the chunk being loaded: 32 Kbar rows, 32 Y rows (row-major, 16-byte
+// pieces XOR-swizzled per row) and their 32 c values (twice)
+template <int D>
+struct LeftLds {
+    static constexpr int kPitch = (D + 8) * 2;            // bytes per staged q / dO row
+    static constexpr int kRows = 2 * 32 * kPitch + 128;
+    static constexpr int kTile = 32 * 2 * D;
+    static constexpr int kPerWave = (kRows + 2 * kTile + 256 + 255) / 256 * 256;
+};
+
+template <class E, int D>
+__global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
+    constexpr int DS = D / 16, DT = D / 32, CPR = D / 8;
+    constexpr int kPitch = LeftLds<D>::kPitch;
+    constexpr int kPerWave = LeftLds<D>::kPerWave;
+    constexpr int kTile = LeftLds<D>::kTile;
+    extern __shared__ __attribute__((aligned(256))) char lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ajraw = blockIdx.x * 4 + wave;
     const bool aj_ok = ajraw < p.AJ;
     const int aj = aj_ok ? ajraw : p.AJ - 1;              // a wave past the end repeats the last column and stores nothing
@@ -114,18 +145,51 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const float sc2 = p.scale * kLog2e;
     const int nch = (RR + 31) / 32;
 
+    // A chunk of 32 rows r goes from global memory into the wave's LDS (global_load_lds_dwordx4: a row's 2 D bytes
+    // by consecutive lanes) and from there into the operand registers; the chunk after it is requested as soon as the
+    // registers are filled, and is waited for (with everything else this wave has in flight) before they are filled
+    // again.  Nothing is shared between waves.
+    char* const kt = qs + LeftLds<D>::kRows;
+    const uint32_t kt0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(size_t)(__attribute__((address_space(3))) char*)kt);
+    const char* const kbb = (const char*)kb;
+    const char* const ybb = (const char*)yb;
+    const char* const cpb = (const char*)cp;
+    const uint32_t rsb = (uint32_t)(rstride * 2), csb = (uint32_t)(cstep * 4);
+    auto request_piece = [&](int n, auto g_c) {
+        constexpr int g = decltype(g_c)::value;
+        const int P = g * 64 + lane;
+        const int r = P / CPR, c = (P % CPR) ^ bl_swz<CPR>(r);
+        const uint32_t off = (uint32_t)min(32 * n + r, RR - 1) * rsb + (uint32_t)c * 16;
+        bl_load_lds16_at<g * 1024>(kbb, off, kt0);
+        bl_load_lds16_at<kTile + g * 1024>(ybb, off, kt0);
+    };
+    auto request = [&](int n) {
+        request_piece(n, std::integral_constant<int, 0>{});
+        request_piece(n, std::integral_constant<int, 1>{});
+        request_piece(n, std::integral_constant<int, 2>{});
+        request_piece(n, std::integral_constant<int, 3>{});
+        if constexpr (CPR / 2 > 4) {
+            request_piece(n, std::integral_constant<int, 4>{});
+            request_piece(n, std::integral_constant<int, 5>{});
+            request_piece(n, std::integral_constant<int, 6>{});
+            request_piece(n, std::integral_constant<int, 7>{});
+        }
+        bl_load_lds4_at<2 * kTile>(cpb, (uint32_t)min(32 * n + m, RR - 1) * csb, kt0);
+    };
+    const uint32_t b_off = (uint32_t)m * (2 * D) + (uint32_t)((hf ^ bl_swz<CPR>(m)) << 4);     // row m as a B operand
     u32x4 kcur[DS], ycur[DS];
     float ccur = 0.f;
-    auto load_tile = [&](int n) {
-        const int r = min(32 * n + m, RR - 1);
-        const uint16_t* kr = kb + (int64_t)r * rstride + 8 * hf;
-        const uint16_t* yr = yb + (int64_t)r * rstride + 8 * hf;
+    // fills the operand registers with the chunk that was requested last and requests chunk `next`
+    auto load_tile = [&](int next) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) {
-            kcur[ds] = *(const u32x4*)(kr + 16 * ds);
-            ycur[ds] = *(const u32x4*)(yr + 16 * ds);
+            kcur[ds] = *(const u32x4*)(kt + (b_off ^ (uint32_t)(ds << 5)));
+            ycur[ds] = *(const u32x4*)(kt + kTile + (b_off ^ (uint32_t)(ds << 5)));
         }
-        ccur = cp[(int64_t)r * cstep] * cmul;
+        ccur = *(const float*)(kt + 2 * kTile + m * 4) * cmul;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // the registers are filled: the buffer may be overwritten
+        if (next >= 0) request(next);
     };
     // logits S2[i, r] and dLm[i, r]: lane -> r = 32 n + m, register v -> i = 8 (v >> 2) + 4 hf + (v & 3)
     auto products = [&](f32x16& s, f32x16& d) {
@@ -161,13 +225,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             mloc[v] = -INFINITY;
             lloc[v] = dloc[v] = 0.f;
         }
-        load_tile(0);
+        request(0);
         for (int n = 0; n < nch; ++n) {
+            load_tile(n + 1 < nch ? n + 1 : -1);
             f32x16 s, d;
             products(s, d);
             const float cl2 = ccur;
             const bool ok = row_ok(n);
-            load_tile(min(n + 1, nch - 1));
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const float z = ok ? s[v] * sc2 - cl2 : -INFINITY;
@@ -214,15 +278,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     float* const dcp = p.dc + uaj * RR;
     uint16_t* const ds2p = p.ds2 + uaj * b1 * p.ds2_ld;
 
-    load_tile(0);
+    request(0);
     for (int n = 0; n < nch; ++n) {
+        load_tile(n + 1 < nch ? n + 1 : -1);
         f32x16 s, d;
         products(s, d);
         const float cl2 = ccur;
         const bool ok = row_ok(n);
         const int r = 32 * n + m;
         const bool r_in = r < RR;
-        load_tile(min(n + 1, nch - 1));
         float dsum = 0.f;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -302,13 +366,6 @@ struct DqaArgs {
     float scale;
 };
 
-template <int CPR>
-__device__ __forceinline__ int bl_swz(int r) {
-    return CPR >= 16 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
-}
-__device__ __forceinline__ void bl_load_lds16(const char* base, uint32_t off, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
-}
 
 template <class E, int D>
 __global__ __launch_bounds__(256) void monarch_bwd_dqa_kernel(DqaArgs p) {
@@ -457,7 +514,7 @@ int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int
     a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.nf = nf; a.RR = nf * b1; a.causal = causal;
     a.scale = scale;
     const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n);
-    const size_t ldsb = (size_t)4 * (2 * 32 * (D + 8) * 2 + 128);
+    const size_t ldsb = (size_t)4 * (D == 128 ? LeftLds<128>::kPerWave : LeftLds<64>::kPerWave);
     const void* fn = nullptr;
     if (dtype == SFM_BF16) fn = D == 128 ? (const void*)monarch_bwd_left_kernel<BF16, 128> : (const void*)monarch_bwd_left_kernel<BF16, 64>;
     else fn = D == 128 ? (const void*)monarch_bwd_left_kernel<F16, 128> : (const void*)monarch_bwd_left_kernel<F16, 64>;
