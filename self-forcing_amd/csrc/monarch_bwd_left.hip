@@ -8,7 +8,7 @@
 // r and stays a batched library GEMM.
 //
 // One wave per (unit, a, j); its b1 query rows and their dO rows sit in LDS, the r = (k, f) rows of Kbar and Y stream
-// from global memory 32 at a time, twice: pass 1 for the softmax statistics (row maximum, sum, and sum of L dLm, kept
+// from global memory 32 at a time (through the wave's own part of LDS, global_load_lds_dwordx4), twice: pass 1 for the softmax statistics (row maximum, sum, and sum of L dLm, kept
 // per lane and merged across lanes once at the end), pass 2 for the gradients.  Logits are computed as
 // S2[i, r] (A = query rows, B = Kbar rows), so that a lane owns one r and holds 16 of the i: the accumulator layout
 // is then directly the B operand [n = r, k = i] of dY^T = dO^T L and dKbar^T = s Q^T dS2, whose A operands are
