@@ -68,10 +68,6 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
     return E::pack(lo, hi);
 }
 
-// low / high 16-bit halves of two dwords -> one dword
-__device__ __forceinline__ uint32_t lo16x2(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }
-__device__ __forceinline__ uint32_t hi16x2(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
-
 // v_exp_f32 without the denormal-range fix-up of exp2f(): arguments here are <= 0 and results that
 // underflow may flush to zero.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
