@@ -313,34 +313,69 @@ __global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
             pg[ks].x = pack2<E>(d[8 * ks + 0], d[8 * ks + 1]); pg[ks].y = pack2<E>(d[8 * ks + 2], d[8 * ks + 3]);
             pg[ks].z = pack2<E>(d[8 * ks + 4], d[8 * ks + 5]); pg[ks].w = pack2<E>(d[8 * ks + 6], d[8 * ks + 7]);
         }
-        // dY^T[d, r] = sum_i dO^T[d, i] L[i, r],  dKbar^T[d, r] = s sum_i Q^T[d, i] dS2[i, r], 32 head-dim rows at a time
+        // dY^T[d, r] = sum_i dO^T[d, i] L[i, r],  dKbar^T[d, r] = s sum_i Q^T[d, i] dS2[i, r], 32 head-dim rows at a time.
+        // A lane (r, hf) holds head-dim 32 dt + 8 g + 4 hf + 0..3 of its row r.  A half swap (v_permlane32_swap) leaves 8
+        // consecutive ones per lane; then, over a pair of head-dim blocks, lane bit 4 is traded for the piece pair
+        // (v_permlane16_swap) and lane bit 3 for the block within the pair (a rotation by 8 within rows of 16 lanes),
+        // after which a lane holds the 16-byte piece 4 (bit 3) + 2 (bit 4) + hf of the rows (r & 7) + 8 rb, rb = 0..3:
+        // one store instruction writes 128 contiguous bytes of each of 8 rows.
+        int64_t rowoff[4];
+        bool row_in[4];
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+            const int rr = 32 * n + (m & 7) + 8 * rb;
+            row_in[rb] = aj_ok && rr < RR;
+            rowoff[rb] = (int64_t)min(rr, RR - 1) * rstride + (4 * ((m >> 3) & 1) + 2 * ((m >> 4) & 1) + hf) * 8;
+        }
 #pragma unroll
         for (int which = 0; which < 2; ++which) {
             const char* src = which == 0 ? dos : qs;
-            uint16_t* const orow = (which == 0 ? dyb : dkb) + (int64_t)min(r, RR - 1) * rstride;
+            uint16_t* const obase = which == 0 ? dyb : dkb;
             const float osc = which == 0 ? 1.f : p.scale;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                f32x16 o;
+            for (int dp = 0; dp < DT / 2; ++dp) {
+                uint32_t w[2][2][4];                     // [block in pair][gp][dword]
 #pragma unroll
-                for (int v = 0; v < 16; ++v) o[v] = 0.f;
+                for (int dl = 0; dl < 2; ++dl) {
+                    const int dt = 2 * dp + dl;
+                    f32x16 o;
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const u32x2 lo = bl_read_tr(src, tr0 + ks * 16 * kPitch + dt * 64);
-                    const u32x2 hi = bl_read_tr(src, tr1 + ks * 16 * kPitch + dt * 64);
-                    const u32x4 aop = {lo.x, lo.y, hi.x, hi.y};
-                    o = E::mfma32(aop, which == 0 ? pl[ks] : pg[ks], o);
+                    for (int v = 0; v < 16; ++v) o[v] = 0.f;
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const u32x2 lo = bl_read_tr(src, tr0 + ks * 16 * kPitch + dt * 64);
+                        const u32x2 hi = bl_read_tr(src, tr1 + ks * 16 * kPitch + dt * 64);
+                        const u32x4 aop = {lo.x, lo.y, hi.x, hi.y};
+                        o = E::mfma32(aop, which == 0 ? pl[ks] : pg[ks], o);
+                    }
+#pragma unroll
+                    for (int gp = 0; gp < 2; ++gp) {
+                        const int g0 = 2 * gp, g1 = 2 * gp + 1;
+                        auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(o[4 * g0 + 0] * osc, o[4 * g0 + 1] * osc),
+                                                                   pack2<E>(o[4 * g1 + 0] * osc, o[4 * g1 + 1] * osc), false, false);
+                        auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(o[4 * g0 + 2] * osc, o[4 * g0 + 3] * osc),
+                                                                   pack2<E>(o[4 * g1 + 2] * osc, o[4 * g1 + 3] * osc), false, false);
+                        w[dl][gp][0] = rx[0]; w[dl][gp][1] = ry[0]; w[dl][gp][2] = rx[1]; w[dl][gp][3] = ry[1];
+                    }
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        auto x = __builtin_amdgcn_permlane16_swap(w[dl][0][q], w[dl][1][q], false, false);
+                        w[dl][0][q] = x[0]; w[dl][1][q] = x[1];
+                    }
                 }
-                // lane (r, hf) holds head-dim 32 dt + 8 g + 4 hf + 0..3; the half-swap leaves 8 consecutive ones per lane
 #pragma unroll
-                for (int gp = 0; gp < 2; ++gp) {
-                    const int g0 = 2 * gp, g1 = 2 * gp + 1;
-                    auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(o[4 * g0 + 0] * osc, o[4 * g0 + 1] * osc),
-                                                               pack2<E>(o[4 * g1 + 0] * osc, o[4 * g1 + 1] * osc), false, false);
-                    auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(o[4 * g0 + 2] * osc, o[4 * g0 + 3] * osc),
-                                                               pack2<E>(o[4 * g1 + 2] * osc, o[4 * g1 + 3] * osc), false, false);
-                    const u32x4 w = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
-                    if (aj_ok && r_in) *(u32x4*)(orow + 32 * dt + 16 * gp + 8 * hf) = w;
+                for (int r4 = 0; r4 < 2; ++r4) {
+                    u32x4 lo, hi;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t x0 = w[0][r4][q], x1 = w[1][r4][q];
+                        // row_ror:8 within 16 lanes; bank mask 0xc writes lanes 8..15 of a row, 0x3 lanes 0..7
+                        lo[q] = (uint32_t)__builtin_amdgcn_update_dpp((int)x0, (int)x1, 0x128, 0xf, 0xc, false);
+                        hi[q] = (uint32_t)__builtin_amdgcn_update_dpp((int)x1, (int)x0, 0x128, 0xf, 0x3, false);
+                    }
+                    // non-temporal: the rows are read once, by the right factor's kernel, after this grid has finished
+                    if (row_in[2 * r4 + 0]) __builtin_nontemporal_store(lo, (u32x4*)(obase + rowoff[2 * r4 + 0] + 64 * dp));
+                    if (row_in[2 * r4 + 1]) __builtin_nontemporal_store(hi, (u32x4*)(obase + rowoff[2 * r4 + 1] + 64 * dp));
                 }
             }
         }
