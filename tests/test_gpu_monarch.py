@@ -43,6 +43,10 @@ def test_c1_plumbing_fp32():
     (1, 1, 128, 2, 3, 40, 33),        # more than 32 block rows: two query-row tiles in step 2
     (1, 3, 64, 5, 2, 3, 64),          # full 64-wide key tile
     (1, 1, 128, 9, 2, 4, 32),         # 9 x 32 = 288 columns: query block-frames split across workgroups
+    (1, 2, 64, 3, 4, 7, 52),          # head_dim 64 with two 32-row key tiles, five waves per group
+    (1, 1, 128, 4, 3, 5, 40),         # 160 columns exactly; the second key tile is ragged (rows 40..63 masked)
+    (1, 1, 64, 7, 2, 3, 24),          # one key tile, 168 columns: six waves in a single group
+    (1, 1, 128, 2, 11, 3, 36),        # 33 scratch rows per (a, j): the last 32-row chunk of step 2 holds one valid row
 ])
 def test_mfma_path_small_shapes(dtype, B, H, D, a, f, b1, b2):
     q, k, v = (randn((B, n * b1 * b2, H, D), 10 + i, dtype) for i, n in enumerate((a, f, f)))
