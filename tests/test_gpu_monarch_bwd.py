@@ -149,6 +149,9 @@ def test_480p_block_shape_bf16_one_head(bwd_path):
     (4, 52, 4, 4, 64, True, torch.bfloat16),       # 208 columns: two passes of the right-factor kernel over each tile
     (4, 52, 7, 7, 128, False, torch.float16),      # 364 columns: three passes
     (5, 6, 2, 3, 64, False, torch.bfloat16),       # b2 = 6, not a multiple of 4: likewise
+    (4, 20, 3, 9, 128, False, torch.bfloat16),     # 36 rows (f, k) per column: two chunks of the left factor, the second with 4 rows
+    (8, 12, 2, 8, 64, False, torch.float16),       # 64 rows: two full chunks
+    (6, 10, 6, 6, 128, True, torch.bfloat16),      # block-causal with two chunks: the visible rows end inside a chunk
 ])
 def test_16bit_gradients_across_the_fused_kernels_limits(h, w, Fq, Fk, D, causal, dtype):
     H = 2
