@@ -177,6 +177,10 @@ def op_level(torch, sfa, args):
     ws.zero_()
     floor_us = C.c_float(0)
     L.check(lib.sfm_probe_tile_traffic(tiles, rows_in, rows_out, row_bytes, 1, ws.data_ptr(), ws.numel(), stream, C.byref(floor_us)))
+    # step 2's: one wave per (unit, a, j) reading its Kbar rows and its Y rows
+    s2_waves, s2_kb = B * H * A * B2, (F * B1 * 2 * D + 1023) // 1024
+    read_us = C.c_float(0)
+    L.check(lib.sfm_probe_row_stream(s2_waves, s2_kb, ws.data_ptr(), ws.numel(), stream, C.byref(read_us)))
     del ws
 
     s1_gbs = STEP1_BYTES / (s1_ms * 1e-3) / 1e9
@@ -200,7 +204,8 @@ def op_level(torch, sfa, args):
         "roofline_step2": {"kernel": "monarch_step2_kernel (configs[1] shape)", "bound": "hbm", "achieved": s2_gbs,
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s2_gbs / HBM_PEAK_GBS,
                            "algorithmic_bytes": STEP2_BYTES, "traffic": MEASURED_TRAFFIC["monarch_step2_kernel"],
-                           "copy_probe_gbs": copy_gbs, "frac_of_copy_probe": s2_gbs / copy_gbs},
+                           "copy_probe_gbs": copy_gbs, "frac_of_copy_probe": s2_gbs / copy_gbs,
+                           "traffic_only_us": read_us.value, "frac_of_traffic_only": read_us.value / (s2_ms * 1e3)},
     }
 
 

@@ -278,6 +278,14 @@ int sfm_probe_mfma_bf16(int32_t iters, void* stream, float* tflops);
 int sfm_probe_tile_traffic(int32_t tiles, int32_t rows_in, int32_t rows_out, int32_t row_bytes, int32_t nontemporal,
                            void* workspace, size_t workspace_bytes, void* stream, float* us);
 
+/* Measurement aid with no counterpart in the reference: the memory traffic of the Monarch forward's step 2 and nothing
+ * else.  `waves` waves (four per workgroup), each reading two contiguous blocks of kb_per_block KB of `workspace`
+ * (device memory, 16-byte aligned, >= 2 * waves * kb_per_block KB; only read), 16 bytes per lane, 8 KB of each block
+ * per batch and the next batch requested as soon as the current one is consumed.  Runs on `stream`, waits, and returns
+ * the mean duration of one pass in microseconds, which bench.py reports beside step 2's own duration. */
+int sfm_probe_row_stream(int32_t waves, int32_t kb_per_block, const void* workspace, size_t workspace_bytes, void* stream,
+                         float* us);
+
 /* Thread-local description of the last error returned on this thread ("" if none). */
 const char* sfm_last_error(void);
 

@@ -77,6 +77,38 @@ __global__ __launch_bounds__(320) void tile_traffic_kernel(const u32x4* in, u32x
     }
 }
 
+// Memory traffic of the Monarch forward's step 2 with nothing else: wave w reads two blocks of `kb_per_block` KB (its
+// Kbar rows and its Y rows), 16 bytes per lane and 8 KB of each block per batch, the next batch requested as soon as
+// the current one has been consumed.
+__global__ __launch_bounds__(256) void row_stream_kernel(const u32x4* in, int nwaves, int kb_per_block) {
+    const int w = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (w >= nwaves) return;
+    const size_t block = (size_t)kb_per_block * 64;                      // 16-byte pieces per block
+    const u32x4* k = in + (size_t)w * block;
+    const u32x4* y = in + ((size_t)nwaves + w) * block;
+    const int last = kb_per_block * 64 - 1;
+    u32x4 buf[16];
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    auto load = [&](int batch) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int idx = min(batch * 512 + i * 64 + lane, last);
+            buf[i] = k[idx];
+            buf[8 + i] = y[idx];
+        }
+    };
+    const int nb = (kb_per_block + 7) / 8;
+    load(0);
+    for (int b = 0; b < nb; ++b) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            acc.x ^= buf[i].x; acc.y += buf[i].y; acc.z ^= buf[i].z; acc.w += buf[i].w;
+        }
+        load(min(b + 1, nb - 1));
+    }
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sfm_probe_sink[0] = (float)acc.x;    // keeps the loads alive
+}
+
 }  // namespace
 }  // namespace sfm
 
@@ -149,6 +181,43 @@ extern "C" int sfm_probe_tile_traffic(int32_t tiles, int32_t rows_in, int32_t ro
     (void)hipEventDestroy(e1);
     if (e != hipSuccess || ms <= 0.f) {
         set_error("sfm_probe_tile_traffic: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    *us = ms * 1e3f / reps;
+    return SFM_OK;
+}
+
+extern "C" int sfm_probe_row_stream(int32_t waves, int32_t kb_per_block, const void* workspace, size_t workspace_bytes, void* stream,
+                                    float* us) {
+    using namespace sfm;
+    if (waves < 1 || kb_per_block < 1 || workspace == nullptr || us == nullptr) {
+        set_error("sfm_probe_row_stream: waves, kb_per_block >= 1, workspace and us non-null");
+        return SFM_ERR_RANGE;
+    }
+    const size_t need = (size_t)2 * waves * kb_per_block * 1024;
+    if (need > workspace_bytes || ((uintptr_t)workspace & 15)) {
+        set_error("sfm_probe_row_stream: workspace of %zu bytes, 16-byte aligned, needed", need);
+        return SFM_ERR_WORKSPACE;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        set_error("sfm_probe_row_stream: hipEventCreate failed");
+        return SFM_ERR_HIP;
+    }
+    const int wgs = (waves + 3) / 4, reps = 5;
+    auto launch = [&] { hipLaunchKernelGGL(row_stream_kernel, dim3(wgs), dim3(256), 0, st, (const u32x4*)workspace, waves, kb_per_block); };
+    launch();                                                // warm-up
+    (void)hipEventRecord(e0, st);
+    for (int i = 0; i < reps; ++i) launch();
+    (void)hipEventRecord(e1, st);
+    hipError_t e = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (e != hipSuccess || ms <= 0.f) {
+        set_error("sfm_probe_row_stream: %s", hipGetErrorString(e));
         return SFM_ERR_HIP;
     }
     *us = ms * 1e3f / reps;

@@ -21,7 +21,7 @@ SYMBOLS = [
     "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
     "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm",
-    "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_dense_bwd_workspace_bytes", "sfm_dense_bwd", "sfm_probe_mfma_bf16", "sfm_probe_tile_traffic", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_last_error", "sfm_version",
+    "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_dense_bwd_workspace_bytes", "sfm_dense_bwd", "sfm_probe_mfma_bf16", "sfm_probe_tile_traffic", "sfm_probe_row_stream", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_last_error", "sfm_version",
 ]
 
 
@@ -116,6 +116,7 @@ def load():
     lib.sfm_vae_norm_act.argtypes = [C.c_int32] * 6 + [P, S3, P, P, S3, P]
     lib.sfm_probe_mfma_bf16.argtypes = [C.c_int32, P, C.POINTER(C.c_float)]
     lib.sfm_probe_tile_traffic.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, P, C.c_size_t, P, C.POINTER(C.c_float)]
+    lib.sfm_probe_row_stream.argtypes = [C.c_int32, C.c_int32, P, C.c_size_t, P, C.POINTER(C.c_float)]
     for name in SYMBOLS:
         if name not in ("sfm_version", "sfm_last_error"):
             getattr(lib, name).restype = C.c_int

@@ -246,3 +246,17 @@ def test_traffic_probe_rejects_bad_arguments_before_any_launch():
     assert lib.sfm_probe_tile_traffic(10, 52, 156, 256, 1, fake, need - 1, None, C.byref(out)) == -6
     assert str(need).encode() in lib.sfm_last_error()
     assert lib.sfm_probe_tile_traffic(10, 52, 156, 256, 1, C.c_void_p(4100), need, None, C.byref(out)) == -6
+
+
+def test_row_stream_probe_rejects_bad_arguments_before_any_launch():
+    lib = L.load()
+    out = C.c_float(0)
+    fake = C.c_void_p(4096)                                   # never dereferenced: every call below fails the checks
+    assert lib.sfm_probe_row_stream(0, 8, fake, 1 << 30, None, C.byref(out)) == -4
+    assert lib.sfm_probe_row_stream(4, 0, fake, 1 << 30, None, C.byref(out)) == -4
+    assert lib.sfm_probe_row_stream(4, 8, None, 1 << 30, None, C.byref(out)) == -4
+    assert lib.sfm_probe_row_stream(4, 8, fake, 1 << 30, None, None) == -4
+    need = 2 * 4 * 8 * 1024
+    assert lib.sfm_probe_row_stream(4, 8, fake, need - 1, None, C.byref(out)) == -6
+    assert str(need).encode() in lib.sfm_last_error()
+    assert lib.sfm_probe_row_stream(4, 8, C.c_void_p(4100), need, None, C.byref(out)) == -6

@@ -136,6 +136,21 @@ def test_mfma_probe_reports_a_rate():
 
 
 @pytest.mark.gpu
+def test_row_stream_probe_reports_a_duration_and_leaves_the_rows_alone():
+    import ctypes as C
+    from self_forcing_amd import lib as L
+    lib = L.load()
+    waves, kb = 37, 19                                         # a workgroup with one wave, a last batch of 3 KB
+    ws = torch.randint(0, 256, (2 * waves * kb * 1024,), dtype=torch.uint8, device="cuda")
+    before = ws.clone()
+    out = C.c_float(0)
+    L.check(lib.sfm_probe_row_stream(waves, kb, ws.data_ptr(), ws.numel(), None, C.byref(out)))
+    torch.cuda.synchronize()
+    assert 0.1 < out.value < 1e5               # microseconds per pass
+    assert torch.equal(ws, before)
+
+
+@pytest.mark.gpu
 def test_traffic_probe_moves_the_bytes_and_reports_a_duration():
     import ctypes as C
     from self_forcing_amd import lib as L
