@@ -157,6 +157,20 @@ class CausalInferencePipeline(nn.Module):
             self._reset_caches(noise.device)
         self.last_chunk_ms = []
         start_frame = 0
+        # The noise re-injected between denoising steps is drawn on the host, so that the same seeds give the same
+        # video on any device.  All of a video's draws are made up front, in the order the steps consume the seeds,
+        # into one pinned buffer that is uploaded once: a pageable upload inside the loop would wait for the GPU at
+        # every step.
+        n_draws = num_blocks * (len(self.denoising_step_list) - 1)
+        eps_all = None
+        if n_draws > 0:
+            nf = self.num_frame_per_block
+            host = torch.empty((n_draws, B * nf, C, H, W), dtype=noise.dtype, pin_memory=noise.is_cuda)
+            for i in range(n_draws):
+                g = torch.Generator().manual_seed(self._next_seed())
+                host[i] = torch.randn((B * nf, C, H, W), generator=g, dtype=torch.float32)
+            eps_all = host.to(noise.device, non_blocking=True)
+        draw = 0
         decode_state = vae.new_state() if vae is not None else None
         pixels = []
         for block in range(num_blocks):
@@ -171,10 +185,9 @@ class CausalInferencePipeline(nn.Module):
                 _, denoised = self.generator(noisy, cond, timestep, self.kv_cache1, self.crossattn_cache, cur)
                 if index < len(self.denoising_step_list) - 1:
                     next_t = self.denoising_step_list[index + 1]
-                    # drawn on the host so that the same seeds give the same video on any device
-                    g = torch.Generator().manual_seed(self._next_seed())
                     flat = denoised.flatten(0, 1)
-                    eps = torch.randn(flat.shape, generator=g, dtype=torch.float32).to(flat.device, flat.dtype)
+                    eps = eps_all[draw]
+                    draw += 1
                     noisy = self.scheduler.add_noise(
                         flat, eps, next_t * torch.ones([B * nf], device=noise.device, dtype=torch.long)
                     ).unflatten(0, denoised.shape[:2])
