@@ -100,7 +100,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const uint32_t fstep = p.ws_f ? p.ws_f : (uint32_t)p.b1 * p.ws_row;     // scratch rows between consecutive f
 
     struct Tile {
-        int f, k, ul, a0, ncols;
+        int f, k, ul, ac, a0, ncols;
     };
     auto decode = [&](int t) {
         Tile x;
@@ -110,6 +110,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         r /= p.n_achunks;
         x.k = r % p.b1;
         x.ul = r / p.b1;
+        x.ac = ac;
         x.a0 = ac * p.a_chunk;
         x.ncols = min(p.a_chunk, p.na - x.a0) * b2;
         return x;
@@ -176,7 +177,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         if (fresh) cur = nxt;
         const char* kt = lds + (r & 1) * 2 * L::kTile;
         const char* vt = kt + L::kTile;
-        const int key = (cur.ul * p.b1 + cur.k) * p.n_achunks + cur.a0;
+        const int key = (cur.ul * p.b1 + cur.k) * p.n_achunks + cur.ac;       // one value per (unit, k, query chunk)
         if (key != qkey) {
             qkey = key;
             const int unit = p.unit0 + cur.ul;

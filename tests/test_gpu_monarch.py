@@ -47,6 +47,8 @@ def test_c1_plumbing_fp32():
     (1, 1, 128, 4, 3, 5, 40),         # 160 columns exactly; the second key tile is ragged (rows 40..63 masked)
     (1, 1, 64, 7, 2, 3, 24),          # one key tile, 168 columns: six waves in a single group
     (1, 1, 128, 2, 11, 3, 36),        # 33 scratch rows per (a, j): the last 32-row chunk of step 2 holds one valid row
+    (1, 1, 128, 9, 1, 3, 52),         # one kv block-frame, three query chunks: consecutive tiles differ in (k, chunk) only
+    (1, 2, 128, 9, 1, 2, 53),         # same with an odd column count
 ])
 def test_mfma_path_small_shapes(dtype, B, H, D, a, f, b1, b2):
     q, k, v = (randn((B, n * b1 * b2, H, D), 10 + i, dtype) for i, n in enumerate((a, f, f)))
