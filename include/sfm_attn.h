@@ -144,6 +144,19 @@ int sfm_monarch_attn_with_kv_cache(const sfm_monarch_desc* desc, const void* q, 
                                    int64_t start_idx, int64_t end_idx, void* out,
                                    void* workspace, size_t workspace_bytes, void* stream);
 
+/* sfm_monarch_attn_with_kv_cache for callers that cannot allocate or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The scratch is a
+ * file-scope device array of SFM_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process
+ * ends; the (batch x head) units are processed in as many passes as that size requires.  Returns SFM_ERR_WORKSPACE
+ * when a single unit needs more than the array holds (the size sfm_monarch_workspace_bytes reports for
+ * heads_per_pass = 1).  The call allocates nothing and never synchronises; its first call on a device looks up the
+ * array's address (make that call outside a graph capture).  All calls on one GPU share the array: calls that may
+ * overlap on one GPU (different streams, different threads) race on it and must be serialised by the caller. */
+#define SFM_STATIC_SCRATCH_BYTES (128u << 20)
+int sfm_monarch_attn_with_kv_cache_static(const sfm_monarch_desc* desc, const void* q, void* k_cache, void* v_cache,
+                                          const void* new_k, const void* new_v, const int64_t new_stride[3],
+                                          int64_t start_idx, int64_t end_idx, void* out, void* stream);
+
 typedef struct sfm_dense_desc {
     int32_t dtype;            /* SFM_BF16 | SFM_F16 (attn_patch.py:317) | SFM_F32 */
     int32_t B, H, D;

@@ -1,4 +1,5 @@
 // extern "C" entry points: argument validation, workspace accounting, pass scheduling.
+#include <pthread.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -654,6 +655,67 @@ int sfm_monarch_attn_with_kv_cache(const sfm_monarch_desc* desc, const void* q, 
                             v_cache, desc->k_stride, desc->kv_tokens, start_idx, end_idx, stream);
     if (rc) return rc;
     return sfm_monarch_fwd(desc, q, k_cache, v_cache, out, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"
+
+// Scratch of sfm_monarch_attn_with_kv_cache_static: one array per GPU, allocated with the code object and held until
+// the process ends.  In host code the array's name only stands for the symbol; the device address is looked up once per
+// device and that pointer is what the kernels, and every other use on the host, get.
+static __device__ __align__(256) unsigned char scratch[SFM_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];
+bool g_scratch_ok[kMaxDevices];
+pthread_mutex_t g_scratch_mutex = PTHREAD_MUTEX_INITIALIZER;
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch_ptr(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("static scratch: no current device (%s)", e == hipSuccess ? "device index out of range" : hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    pthread_mutex_lock(&g_scratch_mutex);
+    if (!g_scratch_ok[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            pthread_mutex_unlock(&g_scratch_mutex);
+            set_error("hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+            return SFM_ERR_HIP;
+        }
+        g_scratch_ptr[dev] = ptr;
+        g_scratch_ok[dev] = true;
+    }
+    *out = g_scratch_ptr[dev];
+    pthread_mutex_unlock(&g_scratch_mutex);
+    return SFM_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int sfm_monarch_attn_with_kv_cache_static(const sfm_monarch_desc* desc, const void* q, void* k_cache, void* v_cache,
+                                          const void* new_k, const void* new_v, const int64_t new_stride[3],
+                                          int64_t start_idx, int64_t end_idx, void* out, void* stream) {
+    MonarchPlan pl;
+    int rc = plan_monarch(desc, &pl);
+    if (rc) return rc;
+    if (pl.per_unit > (size_t)SFM_STATIC_SCRATCH_BYTES) {
+        set_error("one (batch, head) unit needs %zu bytes of scratch, more than the %zu-byte static scratch of this entry "
+                  "point; use sfm_monarch_attn_with_kv_cache with a caller-owned workspace",
+                  pl.per_unit, (size_t)SFM_STATIC_SCRATCH_BYTES);
+        return SFM_ERR_WORKSPACE;
+    }
+    void* ws = nullptr;
+    if ((rc = static_scratch_ptr(&ws))) return rc;
+    // Every pass overwrites the rows of the scratch that it reads (step 1 writes each Kbar / Y / cl row that step 2
+    // loads), so nothing of an earlier call's contents has to be cleared.
+    return sfm_monarch_attn_with_kv_cache(desc, q, k_cache, v_cache, new_k, new_v, new_stride, start_idx, end_idx, out, ws,
+                                          (size_t)SFM_STATIC_SCRATCH_BYTES, stream);
 }
 
 static int check_dense(const sfm_dense_desc* d) {

@@ -10,6 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libsfm_attn.so")
 
 SFM_BF16, SFM_F16, SFM_F32 = 0, 1, 2
+STATIC_SCRATCH_BYTES = 128 << 20      # SFM_STATIC_SCRATCH_BYTES of include/sfm_attn.h
 
 ERR_NAMES = {
     -1: "SFM_ERR_NULL", -2: "SFM_ERR_DTYPE", -3: "SFM_ERR_SHAPE", -4: "SFM_ERR_RANGE", -5: "SFM_ERR_STRIDE",
@@ -19,6 +20,7 @@ ERR_NAMES = {
 # every symbol include/sfm_attn.h declares
 SYMBOLS = [
     "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
+    "sfm_monarch_attn_with_kv_cache_static",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
     "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm",
     "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_dense_bwd_workspace_bytes", "sfm_dense_bwd", "sfm_probe_mfma_bf16", "sfm_probe_tile_traffic", "sfm_probe_row_stream", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_last_error", "sfm_version",
@@ -104,6 +106,7 @@ def load():
                                        S3, I64, I64, I64, P]
     lib.sfm_monarch_attn_with_kv_cache.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, S3, I64, I64, P, P,
                                                    C.c_size_t, P]
+    lib.sfm_monarch_attn_with_kv_cache_static.argtypes = [C.POINTER(MonarchDesc), P, P, P, P, P, S3, I64, I64, P, P]
     lib.sfm_dense_fwd.argtypes = [C.POINTER(DenseDesc), P, P, P, P, P, P]
     lib.sfm_full_attention_with_kv_cache.argtypes = [C.POINTER(DenseDesc), P, P, P, P, P, S3, I64, I64, P, P, P]
     lib.sfm_qk_prologue.argtypes = [C.POINTER(PrologueDesc), P, P, P, P, P, P, C.c_int32, P, P, P, P]

@@ -270,6 +270,34 @@ def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end
     return out
 
 
+def monarch_attn_with_kv_cache_static(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, f_tied, h_reduce, w_reduce, h, w,
+                                      sm_scale=None, num_iters=1, out=None):
+    """monarch_attn_with_kv_cache for callers that cannot allocate (HIP graph capture, serving loops): the scratch
+    is the library's own per-GPU array (lib.STATIC_SCRATCH_BYTES) instead of a fresh tensor, and with `out` given
+    nothing is allocated at all.  No autograd.  Calls on one GPU share the scratch and must not overlap."""
+    _check4("q", q)
+    for name, t in (("k_cache", k_cache), ("v_cache", v_cache), ("new_k", new_k), ("new_v", new_v)):
+        _check4(name, t, q.dtype, q.device)
+    if k_cache.shape != v_cache.shape or new_k.shape != new_v.shape or new_k.stride() != new_v.stride():
+        raise ValueError("k/v shapes or strides differ")
+    if new_k.shape[1] != end_idx - start_idx:
+        raise ValueError(f"new_k holds {new_k.shape[1]} tokens but end_idx - start_idx = {end_idx - start_idx}")
+    if sm_scale is None:
+        sm_scale = q.shape[-1] ** -0.5
+    if out is None:
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    else:
+        _check4("out", out, q.dtype, q.device)
+        if out.shape != q.shape:
+            raise ValueError("out must have q's shape")
+    d = _desc(q, k_cache, v_cache, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1, 0, num_iters)
+    with torch.cuda.device(q.device):
+        _l.check(_l.load().sfm_monarch_attn_with_kv_cache_static(
+            C.byref(d), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), new_k.data_ptr(), new_v.data_ptr(),
+            _l.strides3(new_k), start_idx, end_idx, out.data_ptr(), _stream(q)))
+    return out
+
+
 def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block_causal_size=None, num_iters=1,
                  heads_per_pass=0, kv_block_order=False):
     """One-iteration Monarch attention without a cache write; `block_causal_size` (tokens) masks

@@ -260,3 +260,19 @@ def test_row_stream_probe_rejects_bad_arguments_before_any_launch():
     assert lib.sfm_probe_row_stream(4, 8, fake, need - 1, None, C.byref(out)) == -6
     assert str(need).encode() in lib.sfm_last_error()
     assert lib.sfm_probe_row_stream(4, 8, C.c_void_p(4100), need, None, C.byref(out)) == -6
+
+
+def test_static_scratch_entry_point_rejects_a_unit_beyond_its_size():
+    """sfm_monarch_attn_with_kv_cache_static: one (batch, head) unit of a 63-frame cache at the 480p block shape needs
+    155 MB of scratch, more than the library's 128 MiB array: SFM_ERR_WORKSPACE before any device is touched."""
+    h, w, H, D = 30, 52, 1, 128
+    d = _desc(H=H, kv_tokens=63 * h * w)
+    d.k_stride = d.v_stride = (C.c_int64 * 3)(63 * h * w * H * D, H * D, D)
+    d.q_stride = d.o_stride = (C.c_int64 * 3)(3 * h * w * H * D, H * D, D)
+    rc, one = _ws(d, 1)
+    assert rc == 0 and one > L.STATIC_SCRATCH_BYTES
+    rc = L.load().sfm_monarch_attn_with_kv_cache_static(C.byref(d), 16, 16, 16, 16, 16, (C.c_int64 * 3)(3 * h * w * H * D, H * D, D),
+                                                        60 * h * w, 63 * h * w, 16, None)
+    assert rc == -6 and b"static scratch" in L.load().sfm_last_error()
+    text = open(os.path.join(ROOT, "include", "sfm_attn.h")).read()
+    assert re.search(r"#define\s+SFM_STATIC_SCRATCH_BYTES\s+\(128u\s*<<\s*20\)", text)
