@@ -86,7 +86,7 @@ def op_level(torch, sfa, args):
 
     def step():
         return sfa.monarch_attn.monarch_attn_with_kv_cache(q, kc, vc, nk, nv, start, end, 1, 1, 1, B1, B2,
-                                                           heads_per_pass=args.heads_per_pass)
+                                                           heads_per_pass=args.heads_per_pass, one_kernel=args.one_kernel)
 
     for _ in range(10):
         out = step()
@@ -100,7 +100,7 @@ def op_level(torch, sfa, args):
 
     # per-kernel durations, HIP events on the launch stream (inside the library)
     lib = L.load()
-    d = _desc(q, kc, vc, out, 1, 1, 1, B1, B2, D ** -0.5, 1, 0)
+    d = _desc(q, kc, vc, out, 1, 1, 1, B1, B2, D ** -0.5, 1, 0, 1, args.one_kernel)
     nbytes = sfa.monarch_attn.monarch_workspace_bytes(d, args.heads_per_pass)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -237,6 +237,9 @@ def main():
     ap.add_argument("--heads-per-pass", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--op-only", action="store_true", help="skip the model; time the attention op only")
+    ap.add_argument("--one-kernel", action="store_true",
+                    help="op-level figures of the opt-in one-kernel Monarch forward (Kbar / Y kept in LDS) instead of the default "
+                         "two kernels; kernel_ms then holds the fused kernel and its merge kernel")
     ap.add_argument("--copy-probe", action="store_true",
                     help="accepted for the profile commands; the 1 GiB device copies (known HBM traffic, for scaling rocprof "
                          "counters) always run")

@@ -42,6 +42,12 @@ typedef struct sfm_tiling {
     int32_t f_tied, h_reduce, w_reduce, h, w;
 } sfm_tiling;
 
+/* sfm_monarch_desc.flags: run the forward as ONE kernel that keeps Kbar / Y / cl in LDS instead of the workspace, where
+ * that kernel applies (16-bit tensors, head_dim 128, b1 <= 32, b2 <= 64, no causal mask, num_iters 1; elsewhere the
+ * flag is ignored).  Its workspace is a few MB per unit instead of tens; at the 480p shapes it is slower than the two
+ * kernels (it re-reads every K/V tile once per group of 12 (a, j) columns), so it is opt-in.  Results agree to rounding. */
+#define SFM_MONARCH_ONE_KERNEL 1
+
 typedef struct sfm_monarch_desc {
     int32_t dtype;            /* SFM_BF16 | SFM_F16 | SFM_F32 : type of q, k, v, out */
     int32_t B, H, D;          /* batch, heads, head_dim */
@@ -55,7 +61,7 @@ typedef struct sfm_monarch_desc {
     float   sm_scale;         /* logit scale; the reference default is D^-0.5 (monarch_attn.py:1780-1781) */
     int32_t num_iters;        /* 1: the two-kernel fast path; > 1: alternating refinement of the two factors
                                  (monarch_attn_slow, monarch_attn.py:1705-1751), fp32 kernels, no causal mask */
-    int32_t reserved;         /* 0 */
+    int32_t flags;            /* 0, or SFM_MONARCH_ONE_KERNEL */
     int64_t q_stride[3];      /* batch, token, head */
     int64_t k_stride[3];
     int64_t v_stride[3];      /* must equal k_stride (monarch_attn.py:1261) */
@@ -64,13 +70,13 @@ typedef struct sfm_monarch_desc {
 
 /* Bytes of device scratch sfm_monarch_fwd needs when it processes `heads_per_pass`
  * (batch x head) units at a time (0 = library default).  Replaces the per-call torch.empty
- * scratch of monarch_attn.py:1246-1259. */
+ * scratch of monarch_attn.py:1246-1259.  The size is not proportional to heads_per_pass. */
 int sfm_monarch_workspace_bytes(const sfm_monarch_desc* desc, int32_t heads_per_pass, size_t* bytes);
 
 /* One-iteration Monarch attention forward.  Replaces _attention_with_cache.forward /
  * _attention_no_cache.forward and their two Triton kernels: monarch_attn.py:1225-1323,
  * 1472-1563, 109-253 (_al_cl_y_fwd), 698-842 (_z_fwd).  q and out are in token order.
- * The number of (batch x head) units per pass is derived from workspace_bytes. */
+ * The number of (batch x head) units per pass is derived from workspace_bytes (as many as it holds). */
 int sfm_monarch_fwd(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
                     void* workspace, size_t workspace_bytes, void* stream);
 

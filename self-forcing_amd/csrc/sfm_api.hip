@@ -109,8 +109,14 @@ static int check_strides(const char* name, const int64_t s[3], int64_t tokens, i
 struct MonarchPlan {
     int na, nf, b1, b2, r_pad, units;
     bool mfma, iter;
-    size_t per_unit;   // workspace bytes per (batch x head) unit
+    bool fused;        // the one-kernel forward (monarch_fused.hip) runs: its scratch is sized per pass, not per unit
+    size_t per_unit;   // workspace bytes of a pass over one (batch x head) unit: the least a call needs
 };
+
+// Workspace of a pass over n units.
+static size_t pass_bytes(const MonarchPlan& pl, int n) {
+    return pl.fused ? monarch_fused_bytes(pl.na, pl.nf, pl.b1, pl.b2, n) : pl.per_unit * (size_t)n;
+}
 
 static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
     if (!d) {
@@ -181,12 +187,19 @@ static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
     const size_t rows = (size_t)pl->na * pl->b2 * pl->r_pad;
     pl->per_unit = rows * d->D * (pl->mfma ? 2 : 4) * (pl->iter ? 3 : 2) + rows * sizeof(float) * (pl->iter ? 2 : 1);
     pl->per_unit = (pl->per_unit + 255) / 256 * 256;
+    if (d->flags & ~SFM_MONARCH_ONE_KERNEL) {
+        set_error("unknown bits in flags (0x%x)", (unsigned)d->flags);
+        return SFM_ERR_SHAPE;
+    }
+    pl->fused = pl->mfma && (d->flags & SFM_MONARCH_ONE_KERNEL) && monarch_fused_supported(d->dtype, d->D, pl->b1, pl->b2, d->causal_block_frames);
+    if (pl->fused) pl->per_unit = monarch_fused_bytes(pl->na, pl->nf, pl->b1, pl->b2, 1);
     return SFM_OK;
 }
 
 // Default number of units per pass: all of them while the scratch stays under 4 GiB (one launch pair
 // fills the chip best; smaller passes only pay when the scratch would not fit).
 static int default_units_per_pass(const MonarchPlan& pl) {
+    if (pl.fused) return pl.units;                // a few MB per unit
     const size_t budget = (size_t)3 << 30;        // keeps 32-bit element offsets into each scratch matrix
     size_t n = budget / pl.per_unit;
     if (n < 1) n = 1;
@@ -200,7 +213,7 @@ using namespace sfm;
 
 extern "C" {
 
-int sfm_version(void) { return 5; }
+int sfm_version(void) { return 6; }
 
 const char* sfm_last_error(void) { return g_err; }
 
@@ -217,7 +230,7 @@ int sfm_monarch_workspace_bytes(const sfm_monarch_desc* desc, int32_t heads_per_
         return SFM_ERR_SHAPE;
     }
     int upp = heads_per_pass == 0 ? default_units_per_pass(pl) : (heads_per_pass > pl.units ? pl.units : heads_per_pass);
-    *bytes = pl.per_unit * (size_t)upp;
+    *bytes = pass_bytes(pl, upp);
     return SFM_OK;
 }
 
@@ -276,6 +289,43 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
         set_error("workspace must be non-NULL, 256-byte aligned and hold at least %zu bytes (one unit)", pl.per_unit);
         return SFM_ERR_WORKSPACE;
     }
+    MonarchArgs a;
+    init_args(desc, pl, &a);
+    a.q = q; a.k = k; a.v = v; a.out = out;
+    a.stats = stats;
+    a.stats_ld = (uint32_t)((pl.b1 + 31) / 32 * 32);
+    if (pl.fused) {
+        // as many units per pass as the workspace holds (the scratch of a pass is not linear in its units)
+        int upp = pl.units;
+        while (upp > 1 && pass_bytes(pl, upp) > workspace_bytes) --upp;
+        for (int u0 = 0; u0 < pl.units; u0 += upp) {
+            const int n = pl.units - u0 < upp ? pl.units - u0 : upp;
+            a.unit0 = u0;
+            StepEvents se;
+            if (step_ms)
+                for (int i = 0; i < 3; ++i)
+                    if (hipEventCreate(&se.ev[i]) != hipSuccess) {
+                        set_error("hipEventCreate failed");
+                        return SFM_ERR_HIP;
+                    }
+            rc = launch_monarch_fused(a, desc->dtype, n, workspace, (hipStream_t)stream, step_ms ? &se : nullptr);
+            if (step_ms) {
+                float t1 = 0.f, t2 = 0.f;
+                hipError_t e = rc ? hipSuccess : hipEventSynchronize(se.ev[2]);
+                if (!rc && e == hipSuccess) e = hipEventElapsedTime(&t1, se.ev[0], se.ev[1]);
+                if (!rc && e == hipSuccess) e = hipEventElapsedTime(&t2, se.ev[1], se.ev[2]);
+                for (int i = 0; i < 3; ++i) (void)hipEventDestroy(se.ev[i]);
+                if (!rc && e != hipSuccess) {
+                    set_error("event timing failed: %s", hipGetErrorString(e));
+                    return SFM_ERR_HIP;
+                }
+                step_ms[0] += t1;
+                step_ms[1] += t2;
+            }
+            if (rc) return rc;
+        }
+        return SFM_OK;
+    }
     size_t upp_sz = workspace_bytes / pl.per_unit;
     if (upp_sz * pl.per_unit > ((size_t)3 << 30)) upp_sz = ((size_t)3 << 30) / pl.per_unit;   // 32-bit offsets
     if (upp_sz < 1) {
@@ -283,12 +333,6 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
         return SFM_ERR_UNSUPPORTED;
     }
     const int upp = upp_sz > (size_t)pl.units ? pl.units : (int)upp_sz;
-
-    MonarchArgs a;
-    init_args(desc, pl, &a);
-    a.q = q; a.k = k; a.v = v; a.out = out;
-    a.stats = stats;
-    a.stats_ld = (uint32_t)((pl.b1 + 31) / 32 * 32);
     const size_t rows = (size_t)pl.na * pl.b2 * pl.r_pad;
     const size_t mat_bytes = rows * desc->D * (pl.mfma ? 2 : 4);
     for (int u0 = 0; u0 < pl.units; u0 += upp) {

@@ -45,6 +45,10 @@ struct BF16 {
     static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
     }
+    // 16x16x32: A lane L supplies row L % 16, k = 8 (L / 16) + e; B column L % 16, same k; D column L % 16, rows 4 (L / 16) + v
+    static __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
 };
 
 struct F16 {
@@ -60,6 +64,9 @@ struct F16 {
     }
     static __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mfma16(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
     }
 };
 
@@ -175,6 +182,10 @@ struct StepEvents {
 int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev);
 int launch_monarch_generic(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev);
 bool monarch_mfma_supported(int dtype, int D, int b2);
+// one-kernel forward (monarch_fused.hip): Kbar / Y stay in LDS; `ws` holds monarch_fused_bytes for a pass of nunits units
+bool monarch_fused_supported(int dtype, int D, int b1, int b2, int causal);
+size_t monarch_fused_bytes(int na, int nf, int b1, int b2, int nunits);
+int launch_monarch_fused(const MonarchArgs& a, int dtype, int nunits, void* ws, hipStream_t stream, const StepEvents* ev);
 int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
 int launch_monarch_bwd(const MonarchBwdArgs& g, int dtype, int nunits, hipStream_t stream);
 bool monarch_bwd_gemm_available();

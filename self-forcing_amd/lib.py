@@ -10,6 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libsfm_attn.so")
 
 SFM_BF16, SFM_F16, SFM_F32 = 0, 1, 2
+SFM_MONARCH_ONE_KERNEL = 1
 STATIC_SCRATCH_BYTES = 128 << 20      # SFM_STATIC_SCRATCH_BYTES of include/sfm_attn.h
 
 ERR_NAMES = {
@@ -42,7 +43,7 @@ class MonarchDesc(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("B", C.c_int32), ("H", C.c_int32), ("D", C.c_int32),
                 ("q_tokens", C.c_int32), ("kv_tokens", C.c_int32), ("tiling", Tiling),
                 ("kv_block_order", C.c_int32), ("causal_block_frames", C.c_int32), ("sm_scale", C.c_float),
-                ("num_iters", C.c_int32), ("reserved", C.c_int32),
+                ("num_iters", C.c_int32), ("flags", C.c_int32),
                 ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
                 ("o_stride", C.c_int64 * 3)]
 

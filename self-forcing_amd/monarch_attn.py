@@ -31,7 +31,8 @@ def _check4(name, t, dtype=None, device=None):
         raise ValueError(f"{name}: device {t.device} differs from q's {device}")
 
 
-def _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, kv_block_order, causal_block_frames, num_iters=1):
+def _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, kv_block_order, causal_block_frames, num_iters=1,
+          one_kernel=False):
     if q.dtype not in _DT:
         raise ValueError(f"unsupported dtype {q.dtype}")
     d = _l.MonarchDesc()
@@ -43,6 +44,7 @@ def _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, kv_block_ord
     d.causal_block_frames = causal_block_frames
     d.sm_scale = float(sm_scale)
     d.num_iters = int(num_iters)
+    d.flags = _l.SFM_MONARCH_ONE_KERNEL if one_kernel else 0
     d.q_stride = _l.strides3(q)
     d.k_stride = _l.strides3(k)
     d.v_stride = _l.strides3(v)
@@ -237,9 +239,10 @@ def _needs_grad(*ts):
 
 
 def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, f_tied, h_reduce, w_reduce, h, w,
-                               sm_scale=None, num_iters=1, grad_only_new_kv=False, heads_per_pass=0):
+                               sm_scale=None, num_iters=1, grad_only_new_kv=False, heads_per_pass=0, one_kernel=False):
     """Writes new_k/new_v into k_cache/v_cache[:, start_idx:end_idx] (block order, in place) and
-    returns one-iteration Monarch attention of q against the whole cache view."""
+    returns one-iteration Monarch attention of q against the whole cache view.  `heads_per_pass` and `one_kernel`
+    (no counterparts in the reference) bound the scratch and select the forward that keeps its intermediates in LDS."""
     if _needs_grad(q, k_cache, v_cache, new_k, new_v):
         if num_iters != 1:
             raise NotImplementedError("num_iters > 1 has no backward")
@@ -260,7 +263,7 @@ def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end
     if sm_scale is None:
         sm_scale = q.shape[-1] ** -0.5
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    d = _desc(q, k_cache, v_cache, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1, 0, num_iters)
+    d = _desc(q, k_cache, v_cache, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1, 0, num_iters, one_kernel)
     nbytes = monarch_workspace_bytes(d, heads_per_pass)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):
@@ -299,7 +302,7 @@ def monarch_attn_with_kv_cache_static(q, k_cache, v_cache, new_k, new_v, start_i
 
 
 def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block_causal_size=None, num_iters=1,
-                 heads_per_pass=0, kv_block_order=False):
+                 heads_per_pass=0, kv_block_order=False, one_kernel=False):
     """One-iteration Monarch attention without a cache write; `block_causal_size` (tokens) masks
     block-frames of later causal blocks.  `kv_block_order=True` (no counterpart in the reference) says
     that k, v are a KV-cache view whose rows are already in Monarch block order, e.g. after
@@ -320,7 +323,7 @@ def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block
         sm_scale = q.shape[-1] ** -0.5
     cbf = _causal_block_frames(q, k, (f_tied, h_reduce, w_reduce, h, w), block_causal_size, num_iters)
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-    d = _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1 if kv_block_order else 0, cbf, num_iters)
+    d = _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1 if kv_block_order else 0, cbf, num_iters, one_kernel)
     nbytes = monarch_workspace_bytes(d, heads_per_pass)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 9 and set(names) == set(L.SYMBOLS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sfm_version() == 5
+    assert lib.sfm_version() == 6
 
 
 def test_struct_sizes_match_header_layout():
@@ -54,16 +54,43 @@ def _ws(d, hpp=0):
     return rc, n.value
 
 
+def _fused_bytes(na, nf, b1, b2, units, cus=256):
+    """Scratch of the one-kernel forward for a pass over `units` units: one output block [b1, 128] (16 bit) and 32
+    floats per (unit, stream slot, column); streams = compute units // column groups of (up to) 12."""
+    ncols, tpu = na * b2, nf * b1
+    nj = min(12, ncols)
+    ngroups = -(-ncols // nj)
+    total = tpu * units
+    ns = max(1, min(cus // ngroups, total))
+    tps = -(-total // ns)
+    nstreams = -(-total // tps)
+    nslots = min(nstreams, (tpu - 1) // tps + 2)
+    blocks = units * nslots * ncols
+    r256 = lambda n: (n + 255) // 256 * 256
+    return r256(r256(blocks * b1 * 256) + blocks * 32 * 4)
+
+
 def test_workspace_bytes_accounting():
+    # per unit: 2 matrices of a*b2*r_pad rows x D bf16 + one fp32 per row, r_pad = round_up(21*30, 32)
     rc, n1 = _ws(_desc(), 1)
     assert rc == 0
-    # per unit: 2 matrices of a*b2*r_pad rows x D bf16 + one fp32 per row, r_pad = round_up(21*30, 32)
     rows = 3 * 52 * 640
     assert n1 == rows * 128 * 2 * 2 + rows * 4
     rc, n2 = _ws(_desc(), 2)
     assert rc == 0 and n2 == 2 * n1
     rc, nall = _ws(_desc(), 99)
     assert rc == 0 and nall == 2 * n1          # clamped to B*H units
+    # the one-kernel forward (16-bit tensors, head_dim 128, b1 <= 32, b2 <= 64) and its per-pass scratch
+    one = dict(flags=L.SFM_MONARCH_ONE_KERNEL)
+    rc, f1 = _ws(_desc(**one), 1)
+    assert rc == 0 and f1 == _fused_bytes(3, 21, 30, 52, 1)
+    rc, f2 = _ws(_desc(**one), 0)
+    assert rc == 0 and f2 == _fused_bytes(3, 21, 30, 52, 2)
+    rc, f12 = _ws(_desc(H=12, **one), 0)
+    assert rc == 0 and f12 == _fused_bytes(3, 21, 30, 52, 12) and f12 < 48 << 20
+    assert _ws(_desc(flags=2), 1)[0] == -3
+    # where the one-kernel forward does not apply the flag changes nothing
+    assert _ws(_desc(tiling=L.Tiling(1, 1, 1, 60, 26), **one), 1) == _ws(_desc(tiling=L.Tiling(1, 1, 1, 60, 26)), 1)
     # fp32 tensors take the generic path, which keeps its scratch rows in float
     rc, nf32 = _ws(_desc(dtype=L.SFM_F32), 1)
     assert rc == 0 and nf32 == rows * 128 * 4 * 2 + rows * 4

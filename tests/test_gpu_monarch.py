@@ -59,10 +59,40 @@ def test_mfma_path_small_shapes(dtype, B, H, D, a, f, b1, b2):
 
 @pytest.mark.parametrize("heads_per_pass", [1, 2, 5])
 def test_head_passes_give_identical_results(heads_per_pass):
+    """Passes over fewer heads give the same bits.  The one-kernel forward is the exception: the tile ranges of its
+    workgroups, and with them the points where partial outputs are rounded and merged, depend on the units of a pass,
+    so its passes agree to a rounding step of the output (and each with the oracle)."""
     q, k, v = (randn((1, n * 6 * 20, 5, 128), 20 + i, torch.bfloat16).to(DEV) for i, n in enumerate((2, 3, 3)))
     full = mattn.monarch_attn(q, k, v, 1, 1, 1, 6, 20, heads_per_pass=5)
     part = mattn.monarch_attn(q, k, v, 1, 1, 1, 6, 20, heads_per_pass=heads_per_pass)
     assert torch.equal(full, part)
+    ref = monarch.monarch_attn(q.cpu(), k.cpu(), v.cpu(), 1, 1, 1, 6, 20, dtype=torch.float32)
+    one = mattn.monarch_attn(q, k, v, 1, 1, 1, 6, 20, heads_per_pass=heads_per_pass, one_kernel=True)
+    assert_close_16bit(one, ref, torch.bfloat16)
+    assert max_abs(one, mattn.monarch_attn(q, k, v, 1, 1, 1, 6, 20, heads_per_pass=5, one_kernel=True)) <= 2 ** -6
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,H,a,f,b1,b2", [
+    (1, 1, 1, 1, 2, 8),            # two tiles in all
+    (1, 2, 3, 4, 6, 52),           # the 52-column block of the 480p grid
+    (2, 3, 2, 3, 5, 20),           # ragged everything, batch 2
+    (1, 2, 6, 6, 15, 52),          # reduce2xh-like
+    (1, 1, 2, 3, 32, 33),          # 32 block rows, odd column count (rows padded to 36 in LDS)
+    (1, 3, 5, 2, 3, 64),           # full 64-wide key tile: 11 columns per workgroup
+    (1, 1, 9, 2, 4, 32),           # 288 columns in 24 groups
+    (1, 1, 2, 11, 3, 36),          # 33 tiles per unit: a left-factor pass over one parked row
+    (1, 2, 1, 40, 30, 8),          # 1200 tiles per unit, 8 columns: many streams per unit, many slots to merge
+    (1, 7, 3, 2, 17, 13),          # streams that cross unit boundaries
+])
+def test_two_kernel_and_one_kernel_forward_agree_with_the_oracle(dtype, B, H, a, f, b1, b2):
+    q, k, v = (randn((B, n * b1 * b2, H, 128), 70 + i, dtype) for i, n in enumerate((a, f, f)))
+    ref = monarch.monarch_attn(q, k, v, 1, 1, 1, b1, b2, dtype=torch.float32)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    one = mattn.monarch_attn(qd, kd, vd, 1, 1, 1, b1, b2, one_kernel=True)
+    two = mattn.monarch_attn(qd, kd, vd, 1, 1, 1, b1, b2)
+    assert_close_16bit(one, ref, dtype)
+    assert_close_16bit(two, ref, dtype)
 
 
 @pytest.mark.parametrize("f_tied,h_reduce,w_reduce", [(1, 1, 1), (1, 2, 1), (3, 1, 1), (1, 2, 2), (3, 3, 4), (1, 6, 13)])
