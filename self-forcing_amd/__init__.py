@@ -8,7 +8,7 @@ reference's module names:
     attention.attention / attention.full_attention_with_kv_cache
     prologue.qk_prologue / prologue.rope_table
     causal_model.CausalWanModel (+ self-attention, block, head), pipeline.CausalInferencePipeline
-    vae_decode.WanVAEDecoder (streaming latent -> pixel decode; torch convolutions only)
+    vae_decode.WanVAEDecoder (streaming latent -> pixel decode; channels-last HIP convolutions and norms, conv_ops)
 """
 from . import lib, monarch_attn, attention, prologue, causal_model, pipeline, vae_decode  # noqa: F401
 

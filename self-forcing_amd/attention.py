@@ -108,7 +108,9 @@ def _needs_grad(*ts):
 
 def attention(q, k, v, q_lens=None, k_lens=None, dropout_p=0., softmax_scale=None, q_scale=None, causal=False,
               window_size=(-1, -1), deterministic=False, dtype=torch.bfloat16, fa_version=None, return_lse=False):
-    """softmax(q k^T * scale) v on [B, L, H, D] tensors; inputs are cast to `dtype` like the reference does."""
+    """softmax(q k^T * scale) v on [B, L, H, D] tensors.  Dtypes as in the reference's flash path (attention.py:62-70,
+    135-138): float16 / bfloat16 inputs are used as they are, anything else is cast to `dtype`, and the result comes
+    back in q's original dtype."""
     if causal or dropout_p != 0. or window_size != (-1, -1):
         raise NotImplementedError("only non-causal, dropout-free, full-window attention is built")
     if q_lens is not None or k_lens is not None:
@@ -116,16 +118,22 @@ def attention(q, k, v, q_lens=None, k_lens=None, dropout_p=0., softmax_scale=Non
     _check4("q", q)
     _check4("k", k, None, q.device)
     _check4("v", v, None, q.device)
+    half_dtypes = (torch.float16, torch.bfloat16)
+    if dtype not in half_dtypes:
+        raise ValueError("dtype must be float16 or bfloat16")
+    out_dtype = q.dtype
     if q_scale is not None:
         q = q * q_scale
-    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    q = q if q.dtype in half_dtypes else q.to(dtype)
+    k, v = k.to(q.dtype), v.to(q.dtype)
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** -0.5
     if _needs_grad(q, k, v):
         if return_lse:
             raise NotImplementedError("return_lse is not differentiable")
-        return _DenseFn.apply(q, k, v, softmax_scale)
+        return _DenseFn.apply(q, k, v, softmax_scale).to(out_dtype)
     out, lse = _dense_fwd(q, k, v, softmax_scale, return_lse)
+    out = out.to(out_dtype)
     return (out, lse) if return_lse else out
 
 

@@ -8,14 +8,33 @@ from .monarch_attn import _DT, _stream
 
 
 def _rows(x):
+    if not x.is_cuda:
+        raise ValueError("the block operators run on the GPU")
+    if x.dtype not in _DT:
+        raise ValueError(f"unsupported dtype {x.dtype}")
     if x.dim() != 3 or x.stride(2) != 1 or x.stride(0) != x.shape[1] * x.stride(1):
         raise ValueError("expected a [B, L, C] tensor with contiguous channels and evenly strided rows")
     return x.shape[0] * x.shape[1], x.shape[2], x.stride(1)
 
 
+def _like(name, t, x):
+    """The kernels read every operand in x's dtype: another dtype (or device) would be misread, not converted."""
+    if t.dtype != x.dtype or t.device != x.device:
+        raise ValueError(f"{name}: {t.dtype} on {t.device}, expected {x.dtype} on {x.device} like the activations")
+    return t
+
+
+def _vec(name, t, x):
+    _like(name, t, x)
+    if t.dim() != 1 or t.shape[0] != x.shape[2]:
+        raise ValueError(f"{name}: expected a [C] vector")
+    return t.contiguous()
+
+
 def _mod(e, x):
     """[B, F, 1, C] (or [B, F, C]) modulation tensor -> (tensor, frame stride, rows per frame)."""
     B, L, C = x.shape
+    _like("modulation", e, x)
     e = e.reshape(B, -1, C)
     if e.stride(2) != 1 or (B > 1 and e.stride(0) != e.shape[1] * e.stride(1)):
         e = e.contiguous()
@@ -41,6 +60,7 @@ def ln_modulate(x, scale, shift, eps=1e-6):
 
 def ln_affine(x, weight, bias, eps=1e-6):
     rows, C, xs = _rows(x)
+    weight, bias = _vec("weight", weight, x), _vec("bias", bias, x)
     y = torch.empty_like(x, memory_format=torch.contiguous_format)
     with torch.cuda.device(x.device):
         _l.check(_l.load().sfm_ln_modulate(_DT[x.dtype], rows, C, eps, x.data_ptr(), xs, y.data_ptr(), C, None, None, 0, 1,
@@ -51,7 +71,9 @@ def ln_affine(x, weight, bias, eps=1e-6):
 def gate_residual_(x, y, gate=None):
     """x += y * gate (per-frame gate) in place; gate=None: x += y."""
     rows, C, xs = _rows(x)
-    _, _, ys = _rows(y)
+    _, _, ys = _rows(_like("y", y, x))
+    if y.shape != x.shape:
+        raise ValueError("x and y must have the same shape")
     g, ms, rpf = (None, 0, 1) if gate is None else _mod(gate, x)
     with torch.cuda.device(x.device):
         _l.check(_l.load().sfm_gate_residual(_DT[x.dtype], rows, C, x.data_ptr(), xs, y.data_ptr(), ys,
@@ -63,7 +85,9 @@ def gate_residual_ln_(x, y, gate=None, scale=None, shift=None, weight=None, bias
     """x += y * gate in place (gate=None: x += y), then returns (x, LayerNorm(x) * (1 + scale) + shift), or the
     affine LayerNorm when weight / bias are given: one pass over the rows instead of two kernels."""
     rows, C, xs = _rows(x)
-    _, _, ys = _rows(y)
+    _, _, ys = _rows(_like("y", y, x))
+    if y.shape != x.shape:
+        raise ValueError("x and y must have the same shape")
     g, gms, grpf = (None, 0, 1) if gate is None else _mod(gate, x)
     out = torch.empty_like(x, memory_format=torch.contiguous_format)
     if weight is None:
@@ -74,6 +98,7 @@ def gate_residual_ln_(x, y, gate=None, scale=None, shift=None, weight=None, bias
             ms = sc.stride(1)
         mod = (sc.data_ptr(), sh.data_ptr(), ms, rpf, None, None)
     else:
+        weight, bias = _vec("weight", weight, x), _vec("bias", bias, x)
         mod = (None, None, 0, 1, weight.data_ptr(), bias.data_ptr())
     with torch.cuda.device(x.device):
         _l.check(_l.load().sfm_gate_residual_ln(_DT[x.dtype], rows, C, eps, x.data_ptr(), xs, y.data_ptr(), ys,
@@ -84,6 +109,7 @@ def gate_residual_ln_(x, y, gate=None, scale=None, shift=None, weight=None, bias
 
 def rms_norm(x, weight, eps=1e-6):
     rows, C, xs = _rows(x)
+    weight = _vec("weight", weight, x)
     y = torch.empty_like(x, memory_format=torch.contiguous_format)
     with torch.cuda.device(x.device):
         _l.check(_l.load().sfm_rms_norm(_DT[x.dtype], rows, C, eps, x.data_ptr(), xs, y.data_ptr(), C, weight.data_ptr(),

@@ -133,13 +133,37 @@ def sinusoidal_embedding_1d(dim, position):
     return torch.cat([torch.cos(sinusoid), torch.sin(sinusoid)], dim=1)
 
 
+def _sync_mirrors(kv_cache):
+    """The host-integer mirrors `_global_end` / `_local_end` follow the two int64 tensors of the reference's cache
+    dict: they are read back (one device sync) whenever a tensor is another object or has been written by anyone but
+    cache_commit since the mirrors were taken, e.g. after the reference's own reset, which replaces the tensors
+    (pipeline/causal_inference.py:134-138)."""
+    g, l = kv_cache["global_end_index"], kv_cache["local_end_index"]
+    src = kv_cache.get("_mirror_of")
+    if src is None or src[0] is not g or src[1] != g._version or src[2] is not l or src[3] != l._version:
+        kv_cache["_global_end"] = int(g.item())
+        kv_cache["_local_end"] = int(l.item())
+        kv_cache["_mirror_of"] = (g, g._version, l, l._version)
+        kv_cache.pop("_written", None)
+        kv_cache.pop("_ring", None)
+
+
+def reset_cache_counters(kv_cache, device):
+    """Start of a video (pipeline/causal_inference.py:134-138): fresh zero counters, K/V storage kept.  Sets the host
+    mirrors along with the tensors, so that no device sync is needed to learn that they are zero."""
+    g = kv_cache["global_end_index"] = torch.tensor([0], dtype=torch.long, device=device)
+    l = kv_cache["local_end_index"] = torch.tensor([0], dtype=torch.long, device=device)
+    kv_cache["_global_end"] = kv_cache["_local_end"] = 0
+    kv_cache["_mirror_of"] = (g, g._version, l, l._version)
+    kv_cache.pop("_written", None)
+    kv_cache.pop("_ring", None)
+
+
 def cache_step(kv_cache, current_start, num_new, frame_seqlen, local_attn_size, sink_size, max_attention_size):
     """Index arithmetic of one self-attention call (causal_model.py:907-938), on host integers.
     Returns (roll, cache_start, local_start, local_end) with local_* relative to cache_start and
     roll = (src, dst, len) of the window-eviction copy (len 0 = none)."""
-    if "_global_end" not in kv_cache:
-        kv_cache["_global_end"] = int(kv_cache["global_end_index"].item())
-        kv_cache["_local_end"] = int(kv_cache["local_end_index"].item())
+    _sync_mirrors(kv_cache)
     g_end, l_end = kv_cache["_global_end"], kv_cache["_local_end"]
     current_end = current_start + num_new
     cache_len = kv_cache["k"].shape[1]
@@ -179,9 +203,11 @@ def cache_commit(kv_cache, current_end, local_end):
     """causal_model.py:1102-1103 (the reference stores the view-relative local end)."""
     kv_cache["_global_end"], kv_cache["_local_end"] = current_end, local_end
     if kv_cache.get("_written") != (current_end, local_end):     # unchanged when a chunk is re-run at another timestep
-        kv_cache["global_end_index"].fill_(current_end)
-        kv_cache["local_end_index"].fill_(local_end)
+        g, l = kv_cache["global_end_index"], kv_cache["local_end_index"]
+        g.fill_(current_end)
+        l.fill_(local_end)
         kv_cache["_written"] = (current_end, local_end)
+        kv_cache["_mirror_of"] = (g, g._version, l, l._version)
 
 
 class CausalWanSelfAttention(nn.Module):

@@ -27,6 +27,7 @@ int launch_prologue(const sfm_prologue_desc& d, const TokMap& map, const void* x
                     const void* wq, const void* wk, const double* rope, void* q_out, void* kc, void* vc,
                     hipStream_t stream);
 bool monarch_generic_supported(const MonarchArgs& a);
+bool monarch_iter_supported(const MonarchArgs& a);
 int launch_ln_modulate(int dtype, int64_t rows, int C, float eps, const void* x, int64_t xs, void* y, int64_t ys,
                        const void* scale, const void* shift, int64_t ms, int rows_per_frame, const void* weight,
                        const void* bias, hipStream_t stream);
@@ -187,6 +188,18 @@ static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
     const size_t rows = (size_t)pl->na * pl->b2 * pl->r_pad;
     pl->per_unit = rows * d->D * (pl->mfma ? 2 : 4) * (pl->iter ? 3 : 2) + rows * sizeof(float) * (pl->iter ? 2 : 1);
     pl->per_unit = (pl->per_unit + 255) / 256 * 256;
+    // the fp32 kernels' own limits, checked here so that no entry point has written anything (the KV-cache entry points
+    // write the cache before the forward is launched) when they are exceeded
+    if (!pl->mfma) {
+        MonarchArgs lim;
+        memset(&lim, 0, sizeof(lim));
+        lim.D = d->D; lim.na = pl->na; lim.nf = pl->nf; lim.b1 = pl->b1; lim.b2 = pl->b2;
+        if (pl->iter ? !monarch_iter_supported(lim) : !monarch_generic_supported(lim)) {
+            set_error("block shape b1=%d, b2=%d, %d rows per column, head_dim %d exceeds the LDS budget of the fp32 kernels that "
+                      "this dtype / shape / num_iters runs on", pl->b1, pl->b2, pl->nf * pl->b1, d->D);
+            return SFM_ERR_UNSUPPORTED;
+        }
+    }
     if (d->flags & ~SFM_MONARCH_ONE_KERNEL) {
         set_error("unknown bits in flags (0x%x)", (unsigned)d->flags);
         return SFM_ERR_SHAPE;

@@ -11,7 +11,7 @@ import time
 import torch
 import torch.nn as nn
 
-from .causal_model import FRAME_HEIGHT, FRAME_WIDTH, CausalWanModel
+from .causal_model import FRAME_HEIGHT, FRAME_WIDTH, CausalWanModel, reset_cache_counters
 
 
 class FlowMatchScheduler:
@@ -110,10 +110,9 @@ class CausalInferencePipeline(nn.Module):
         self.kv_cache1 = [{
             "k": torch.zeros([batch_size, size, m.num_heads, m.dim // m.num_heads], dtype=dtype, device=device),
             "v": torch.zeros([batch_size, size, m.num_heads, m.dim // m.num_heads], dtype=dtype, device=device),
-            "global_end_index": torch.tensor([0], dtype=torch.long, device=device),
-            "local_end_index": torch.tensor([0], dtype=torch.long, device=device),
-            "_global_end": 0, "_local_end": 0,
         } for _ in range(m.num_layers)]
+        for c in self.kv_cache1:
+            reset_cache_counters(c, device)
 
     def _initialize_crossattn_cache(self):
         self.crossattn_cache = [{"k": None, "v": None, "is_init": False} for _ in range(self.generator.model.num_layers)]
@@ -122,11 +121,7 @@ class CausalInferencePipeline(nn.Module):
         for c in self.crossattn_cache:
             c["is_init"] = False
         for c in self.kv_cache1:       # only the counters are reset, not the K/V storage (`:129-138`)
-            c["global_end_index"] = torch.tensor([0], dtype=torch.long, device=device)
-            c["local_end_index"] = torch.tensor([0], dtype=torch.long, device=device)
-            c["_global_end"] = c["_local_end"] = 0
-            c.pop("_written", None)
-            c.pop("_ring", None)
+            reset_cache_counters(c, device)
 
     def _next_seed(self):
         if self.seeds is None:

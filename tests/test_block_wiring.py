@@ -1,0 +1,148 @@
+"""Wiring of CausalWanAttentionBlock / CausalHead (wan/modules/causal_model.py:1176-1205, 1229-1235), pinned on the
+CPU by invariants that a permuted modulation index, a missing `1 +` or a swapped residual would break, and by a
+statement of the block in plain tensor algebra that shares only the sub-modules (projections, attention) with it."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import self_forcing_amd as sfa
+from oracle.ops import OracleOps
+
+cm = sfa.causal_model
+DIM, HEADS, FR, HW = 64, 2, 3, (2, 3)
+S = FR * HW[0] * HW[1]
+
+
+class _Record(torch.nn.Module):
+    """Stands in for a sub-layer: keeps its input, returns a fixed tensor (zeros by default)."""
+
+    def __init__(self, out=None):
+        super().__init__()
+        self.seen, self.out = None, out
+
+    def forward(self, x, *a, **k):
+        self.seen = x.clone()
+        return torch.zeros_like(x) if self.out is None else self.out
+
+
+def _block(seed=0):
+    torch.manual_seed(seed)
+    b = cm.CausalWanAttentionBlock(DIM, 128, HEADS, block_num=0, frame_hw=HW, total_seq_len=2 * S, ops=OracleOps(),
+                                   flags=cm.AttentionFlags(0, use_framewise=True))
+    for m in b.modules():
+        if isinstance(m, torch.nn.Linear):
+            torch.nn.init.normal_(m.weight, std=0.2)
+            torch.nn.init.normal_(m.bias, std=0.1)
+    torch.nn.init.normal_(b.norm3.weight, mean=1.0, std=0.2)
+    torch.nn.init.normal_(b.norm3.bias, std=0.2)
+    return b.float().eval()
+
+
+def _inputs(seed=1):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(1, S, DIM, generator=g)
+    e = 0.5 * torch.randn(1, FR, 6, DIM, generator=g)
+    ctx = torch.randn(1, 5, DIM, generator=g)
+    return x, e, ctx
+
+
+def _cache():
+    return {"k": torch.zeros(1, 2 * S, HEADS, DIM // HEADS), "v": torch.zeros(1, 2 * S, HEADS, DIM // HEADS),
+            "global_end_index": torch.tensor([0]), "local_end_index": torch.tensor([0])}
+
+
+def _run(b, x, e, ctx):
+    with torch.no_grad():
+        return b(x, e, (FR,) + HW, ctx, _cache(), {"k": None, "v": None, "is_init": False}, 0)
+
+
+def _per_frame(t):           # [1, F, C] -> [1, S, C]
+    return t.repeat_interleave(S // FR, dim=1)
+
+
+def test_block_equals_the_reference_statement_in_tensor_algebra():
+    """e = (modulation + e_in) split into shift/scale/gate of the attention branch and of the FFN branch, in that order."""
+    b = _block()
+    x, e_in, ctx = _inputs()
+    got = _run(b, x, e_in, ctx)
+    with torch.no_grad():
+        e = [_per_frame(t.squeeze(2)) for t in (b.modulation.unsqueeze(1) + e_in).chunk(6, dim=2)]
+        ln = lambda t: F.layer_norm(t, (DIM,), None, None, b.eps)
+        y = b.self_attn(ln(x) * (1 + e[1]) + e[0], (FR,) + HW, _cache(), 0)
+        h = x + y * e[2]
+        h = h + b.cross_attn(F.layer_norm(h, (DIM,), b.norm3.weight, b.norm3.bias, b.eps), ctx, None)
+        y = b.ffn[2](F.gelu(b.ffn[0](ln(h) * (1 + e[4]) + e[3]), approximate="tanh"))
+        ref = h + y * e[5]
+    assert torch.allclose(got, ref, atol=2e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("zeroed,identity", [((2, 5), True), ((1, 4), False), ((0, 3), False), ((2, 4), False), ((1, 5), False)])
+def test_zero_gates_leave_only_the_cross_attention_residual(zeroed, identity):
+    """Chunks 2 and 5 are the gates: with both zero the block is x + cross_attn(norm3(x)); zeroing any other pair is not."""
+    b = _block()
+    x, e_in, ctx = _inputs()
+    e_in = e_in.clone()
+    for i in zeroed:
+        e_in[:, :, i] = -b.modulation.detach()[:, i]
+    got = _run(b, x, e_in, ctx)
+    with torch.no_grad():
+        ref = x + b.cross_attn(F.layer_norm(x, (DIM,), b.norm3.weight, b.norm3.bias, b.eps), ctx, None)
+    assert torch.allclose(got, ref, atol=1e-5) == identity
+
+
+def test_scale_minus_one_feeds_the_shift_alone():
+    """scale = -1 cancels the normalised input: the attention branch then sees exactly its shift (chunk 0 with scale chunk 1),
+    the FFN exactly its shift (chunk 3 with scale chunk 4)."""
+    b = _block()
+    x, e_in, ctx = _inputs()
+    e_in = e_in.clone()
+    e_in[:, :, 1] = -1 - b.modulation.detach()[:, 1]
+    e_in[:, :, 4] = -1 - b.modulation.detach()[:, 4]
+    b.self_attn = _Record()
+    rec_ffn = _Record(out=torch.zeros(1, S, 128))
+    b.ffn[0] = rec_ffn
+    _run(b, x, e_in, ctx)
+    mod = (b.modulation.unsqueeze(1) + e_in).detach()
+    # (1 + scale vanishes up to the rounding of modulation + e_in: the normalised rows survive with a factor ~1e-7)
+    assert torch.allclose(b.self_attn.seen, _per_frame(mod[:, :, 0]), atol=2e-6, rtol=0)
+    assert torch.allclose(rec_ffn.seen, _per_frame(mod[:, :, 3]), atol=2e-6, rtol=0)
+    # and scale 0 (not -1) feeds the plain normalised rows plus the shift: the `1 +` is there
+    e_in[:, :, 1] = -b.modulation.detach()[:, 1]
+    _run(b, x, e_in, ctx)
+    assert torch.allclose(b.self_attn.seen, F.layer_norm(x, (DIM,), None, None, b.eps) + _per_frame(mod[:, :, 0]), atol=1e-6)
+
+
+@pytest.mark.parametrize("chunk", range(6))
+def test_a_frames_modulation_touches_only_that_frames_tokens(chunk):
+    """With the (token-mixing) self-attention replaced by a per-token stand-in, changing frame 1's modulation row `chunk`
+    changes frame 1's tokens and no others: modulation is applied per frame, in token order."""
+    b = _block()
+    x, e_in, ctx = _inputs()
+    b.self_attn = torch.nn.Sequential(torch.nn.Linear(DIM, DIM))          # per-token
+    b.self_attn.forward = lambda t, *a, **k: torch.tanh(b.self_attn[0](t))
+    base = _run(b, x, e_in, ctx)
+    e2 = e_in.clone()
+    e2[:, 1, chunk] += 0.7
+    diff = (_run(b, x, e2, ctx) - base).abs().amax(-1)[0]
+    per = S // FR
+    assert diff[per:2 * per].min() > 1e-6
+    assert diff[:per].max() == 0 and diff[2 * per:].max() == 0
+
+
+def test_head_is_linear_of_the_modulated_norm():
+    """CausalHead: chunk 0 is the shift, chunk 1 the scale; e = -modulation leaves Linear(LayerNorm(x))."""
+    torch.manual_seed(3)
+    hd = cm.CausalHead(DIM, 16, (1, 2, 2)).float().eval()
+    torch.nn.init.normal_(hd.head.weight, std=0.2)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(1, S, DIM, generator=g)
+    e = torch.randn(1, FR, 1, DIM, generator=g)
+    ln = F.layer_norm(x, (DIM,), None, None, hd.norm.eps)
+    with torch.no_grad():
+        got = hd(x, e).flatten(1, 2)
+        mod = hd.modulation.unsqueeze(1) + e                                    # [1, F, 2, C]: shift, scale
+        ref = hd.head(ln * (1 + _per_frame(mod[:, :, 1])) + _per_frame(mod[:, :, 0]))
+        swapped = hd.head(ln * (1 + _per_frame(mod[:, :, 0])) + _per_frame(mod[:, :, 1]))
+        plain = hd(x, -hd.modulation.unsqueeze(1).expand(1, FR, 2, DIM)).flatten(1, 2)
+    assert torch.allclose(got, ref, atol=1e-5) and not torch.allclose(got, swapped, atol=1e-3)
+    assert torch.allclose(plain, hd.head(ln), atol=1e-5)

@@ -303,3 +303,23 @@ def test_static_scratch_entry_point_rejects_a_unit_beyond_its_size():
     assert rc == -6 and b"static scratch" in L.load().sfm_last_error()
     text = open(os.path.join(ROOT, "include", "sfm_attn.h")).read()
     assert re.search(r"#define\s+SFM_STATIC_SCRATCH_BYTES\s+\(128u\s*<<\s*20\)", text)
+
+
+def test_fp32_kernel_limits_are_reported_before_anything_is_written():
+    """Blocks 208 columns wide do not fit the LDS of the fp32 kernels that take them (b2 > 64 is beyond the MFMA kernels):
+    every entry point, the workspace query included, answers SFM_ERR_UNSUPPORTED from the descriptor alone, i.e. before
+    the KV-cache entry point could have written the new rows."""
+    h, w = 30, 208
+    for kw in (dict(), dict(num_iters=2), dict(dtype=L.SFM_F32)):
+        d = _desc(q_tokens=3 * h * w, kv_tokens=6 * h * w, tiling=L.Tiling(1, 1, 1, h, w), **kw)
+        d.q_stride = d.o_stride = (C.c_int64 * 3)(3 * h * w * 256, 256, 128)
+        d.k_stride = d.v_stride = (C.c_int64 * 3)(6 * h * w * 256, 256, 128)
+        assert _ws(d, 1)[0] == -9 and b"LDS budget" in L.load().sfm_last_error()
+        rc = L.load().sfm_monarch_attn_with_kv_cache(C.byref(d), 16, 16, 16, 16, 16, (C.c_int64 * 3)(3 * h * w * 256, 256, 128),
+                                                     3 * h * w, 6 * h * w, 16, 256, 1 << 40, None)
+        assert rc == -9
+    # 104 columns (the 720p grid halved) still run
+    d = _desc(q_tokens=3 * 30 * 104, kv_tokens=6 * 30 * 104, tiling=L.Tiling(1, 1, 1, 30, 104))
+    d.q_stride = d.o_stride = (C.c_int64 * 3)(3 * 30 * 104 * 256, 256, 128)
+    d.k_stride = d.v_stride = (C.c_int64 * 3)(6 * 30 * 104 * 256, 256, 128)
+    assert _ws(d, 1)[0] == 0

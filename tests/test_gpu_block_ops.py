@@ -60,3 +60,21 @@ def test_block_ops_reject_bad_layouts():
                         torch.zeros(1, 3, 1, 64, dtype=torch.bfloat16, device=DEV))
     with pytest.raises(ValueError):        # C not a multiple of 8
         blk.rms_norm(randn((1, 8, 12), 1, torch.bfloat16).to(DEV), torch.ones(12, dtype=torch.bfloat16, device=DEV))
+
+
+def test_block_ops_reject_operands_of_another_dtype_or_device():
+    """The kernels read every operand in the activations' dtype: fp32 modulation or norm weights next to bf16
+    activations would be misread, so the wrappers refuse them (and host tensors)."""
+    x = randn((1, 12, 64), 2, torch.bfloat16).to(DEV)
+    m16 = torch.zeros(1, 3, 1, 64, dtype=torch.bfloat16, device=DEV)
+    m32, w32 = m16.float(), torch.ones(64, device=DEV)
+    w16 = w32.bfloat16()
+    for call in (lambda: blk.ln_modulate(x, m32, m16), lambda: blk.ln_modulate(x, m16, m32),
+                 lambda: blk.ln_affine(x, w32, w16), lambda: blk.ln_affine(x, w16, w32), lambda: blk.rms_norm(x, w32),
+                 lambda: blk.rms_norm(x, w16.cpu()), lambda: blk.rms_norm(x.cpu(), w16.cpu()),
+                 lambda: blk.gate_residual_(x.clone(), x.float()), lambda: blk.gate_residual_(x.clone(), x, m32),
+                 lambda: blk.gate_residual_ln_(x.clone(), x, m16, weight=w32, bias=w16),
+                 lambda: blk.gate_residual_ln_(x.clone(), x, m16, scale=m32, shift=m16),
+                 lambda: blk.rms_norm(x, torch.ones(32, dtype=torch.bfloat16, device=DEV))):
+        with pytest.raises(ValueError):
+            call()

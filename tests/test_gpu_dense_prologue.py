@@ -25,6 +25,20 @@ def test_dense_reference_shapes(dtype, B, Lq, Lk, H, D):
     assert max_abs(lse, lse_ref) < 1e-3
 
 
+def test_attention_keeps_half_dtypes_and_returns_qs_dtype():
+    """attention.py:62-70, 135-138: float16 / bfloat16 inputs are used as they are (not recast to the default
+    bfloat16), anything else is computed in `dtype`; the result has q's original dtype."""
+    q, k, v = (randn((1, n, 2, 64), 90 + i, torch.float32) for i, n in enumerate((33, 70, 70)))
+    ref = dense.attention(q, k, v, dtype=torch.float64)
+    o16 = sfa.attention.attention(q.half().to(DEV), k.half().to(DEV), v.half().to(DEV))
+    assert o16.dtype == torch.float16
+    assert max_abs(o16, dense.attention(q.half(), k.half(), v.half(), dtype=torch.float64)) < 2e-3       # fp16 bar, not bf16's
+    o32 = sfa.attention.attention(q.to(DEV), k.to(DEV), v.to(DEV))
+    assert o32.dtype == torch.float32 and max_abs(o32, ref) < 2e-2
+    o32h = sfa.attention.attention(q.to(DEV), k.to(DEV), v.to(DEV), dtype=torch.float16)
+    assert o32h.dtype == torch.float32 and max_abs(o32h, ref) < 2e-3
+
+
 def test_dense_with_kv_cache_writes_in_token_order():
     dtype = torch.bfloat16
     q = randn((2, 40, 3, 64), 4, dtype)

@@ -28,7 +28,9 @@ def _cos(a, b):
 
 
 @pytest.mark.parametrize("flags", [dict(use_framewise=True), dict(use_framewise=True, h_reduce=2, use_dense_init=True),
-                                   dict(disable_monarch=True), dict(use_framewise=True, num_iters=2)])
+                                   dict(disable_monarch=True), dict(use_framewise=True, num_iters=2),
+                                   dict(),                                  # the reference's default tiling: f_tied = 3
+                                   dict(w_reduce=2)])
 def test_rollout_latents_match_oracle_model(flags):
     """2 chunks x (4 + 1) passes of a 2-layer model at the 52-column grid.  Tolerance: bf16 GEMMs differ in
     accumulation order between CPU and GPU, so latents are compared by cosine > 0.995 per chunk and
@@ -37,16 +39,21 @@ def test_rollout_latents_match_oracle_model(flags):
     noise = torch.randn(1, 6, 16, 12, 104, generator=g).to(torch.bfloat16)
     ctx = torch.randn(1, 16, 64, generator=g).to(torch.bfloat16)
     ref_gen, dev_gen = _pair(**flags)
-    ref = pl.CausalInferencePipeline(ref_gen, frame_hw=(6, 52), num_cache_frames=6).inference(noise, ctx)
+    pipe_ref = pl.CausalInferencePipeline(ref_gen, frame_hw=(6, 52), num_cache_frames=6)
+    ref = pipe_ref.inference(noise, ctx)
     pipe = pl.CausalInferencePipeline(dev_gen, frame_hw=(6, 52), num_cache_frames=6)
     out = pipe.inference(noise.to("cuda:0"), ctx.to("cuda:0"), profile=True)
     assert torch.isfinite(out).all() and len(pipe.last_chunk_ms) == 2
     for c in range(2):
         assert _cos(out[:, 3 * c:3 * c + 3], ref[:, 3 * c:3 * c + 3]) > 0.995
     assert max_abs(out, ref) < 0.05 * ref.float().abs().max().item()
-    # the caches end up holding the same clean-chunk K/V
-    kd, kr = pipe.kv_cache1[1]["k"], ref_gen.model.blocks[1].self_attn  # noqa: F841
-    assert pipe.kv_cache1[0]["_global_end"] == 6 * 312
+    # the caches end up holding the same clean-chunk K/V, row for row (same block order), and the same counters
+    for layer in range(2):
+        for key in ("k", "v"):
+            cd, cr = pipe.kv_cache1[layer][key], pipe_ref.kv_cache1[layer][key]
+            assert _cos(cd, cr) > 0.999 and max_abs(cd, cr) < 0.05 * cr.float().abs().max().item()
+        assert pipe.kv_cache1[layer]["_global_end"] == pipe_ref.kv_cache1[layer]["_global_end"] == 6 * 312
+        assert int(pipe.kv_cache1[layer]["local_end_index"]) == int(pipe_ref.kv_cache1[layer]["local_end_index"]) == 6 * 312
 
 
 def test_single_forward_matches_closely():

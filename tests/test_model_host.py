@@ -54,6 +54,38 @@ def test_cache_step_matches_oracle_state_machine():
             assert int(kv["global_end_index"]) == st.global_end and int(kv["local_end_index"]) == st.local_end
 
 
+@pytest.mark.parametrize("reset", ["replace", "in_place"])
+def test_reference_style_reset_of_a_rolled_window_cache(reset):
+    """The reference starts a new video by resetting only the two index tensors (pipeline/causal_inference.py:134-138).
+    A windowed cache that has rolled (local end = cache length, global end beyond it) must then start again at 0: the
+    host mirrors of the counters follow the tensors, whoever writes them."""
+    local_attn, sink, frame = 4, 0, 6
+    cache_len = local_attn * frame
+    kv = {"k": torch.zeros(1, cache_len, 1, 8), "global_end_index": torch.tensor([0]), "local_end_index": torch.tensor([0])}
+    for cur in (0, 12, 24, 36):
+        roll, cs, ls, le, ce = cm.cache_step(kv, cur, 12, frame, local_attn, sink, cache_len)
+        cm.cache_commit(kv, ce, le)
+    assert (le, ce) == (cache_len, 48) and roll[2] > 0
+    if reset == "replace":
+        kv["global_end_index"] = torch.tensor([0])
+        kv["local_end_index"] = torch.tensor([0])
+    else:
+        kv["global_end_index"].zero_()
+        kv["local_end_index"].fill_(0)
+    roll, cs, ls, le, ce = cm.cache_step(kv, 0, 12, frame, local_attn, sink, cache_len)
+    assert (roll[2], cs, ls, le, ce) == (0, 0, 0, 12, 12)
+    cm.cache_commit(kv, ce, le)
+    # ... and a run of steps after the reset follows the oracle's state machine from scratch
+    st = ocache.KVCacheState(cache_len, cache_len, frame, local_attn, sink)
+    st.step(0, 12)
+    for cur in (12, 12, 24):
+        roll, cs, ls, le, ce = cm.cache_step(kv, cur, 12, frame, local_attn, sink, cache_len)
+        cm.cache_commit(kv, ce, le)
+        o = st.step(cur, 12)
+        assert (cs, ls, le) == (o.cache_start, o.write_start, o.write_end)
+    assert int(kv["global_end_index"]) == st.global_end and int(kv["local_end_index"]) == st.local_end
+
+
 def test_pipeline_rollout_dispatch_and_cache_trace():
     ops = OracleOps()
     gen = _tiny(ops, use_framewise=True)
