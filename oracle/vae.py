@@ -13,8 +13,9 @@ brute-force triple loop and, frame by frame with its cache, against one convolut
 zero-front-padded clip; the norm against its closed form; the attention block against an explicit softmax;
 causality of the whole decoder (pixels of frames <= 1 + 4 (t - 1) do not depend on latent frames > t); the
 frame count 1 + 4 (T - 1).  The composition of these pieces into the full decoder (channel counts, order of
-blocks) follows the cited lines and is otherwise parity unpinned: no reference output exists offline (the VAE
-checkpoint is not available and nothing of the reference is imported).
+blocks, the chunked stream) is pinned by tests/golden/vae_reference_vectors.npz: the output of the reference's
+own `decode` and `cached_decode` on seeded weights at dim=32 (tests/golden/make_vae_reference_vectors.py wrote
+it in the authoring container), which decode_frames reproduces to 1e-6 (the reference rounds to fp32 at every upsampling, vae.py:57-63).
 """
 import numpy as np
 import torch
@@ -142,9 +143,9 @@ def decode_frame(x, W, st):
     return _cached_conv(x, W, "decoder.head.2", st)
 
 
-def decode_to_pixel(latent, W, st=None):
-    """latent [B,T,C,h,w] -> pixels [B,T',3,8h,8w] (float64, clamped), one latent frame per decoder call;
-    pass the Stream of earlier chunks to continue it (vae.py:574-596)."""
+def decode_frames(latent, W, st=None):
+    """latent [B,T,C,h,w] -> decoder output [B,T',3,8h,8w] (float64, before the wrapper's clamp), one latent
+    frame per decoder call; pass the Stream of earlier chunks to continue it (vae.py:574-596)."""
     W = {k: torch.as_tensor(np.asarray(v.detach().cpu().double()) if isinstance(v, torch.Tensor) else v, dtype=F64) for k, v in W.items()}
     st = Stream() if st is None else st
     z = torch.as_tensor(latent, dtype=F64).permute(0, 2, 1, 3, 4)
@@ -153,4 +154,9 @@ def decode_to_pixel(latent, W, st=None):
     x = causal_conv3d(z, W["conv2.weight"], W["conv2.bias"])
     outs = [decode_frame(x[:, :, i:i + 1], W, st) for i in range(x.shape[2])]
     st.frames += x.shape[2]
-    return torch.cat(outs, dim=2).clamp(-1, 1).permute(0, 2, 1, 3, 4)
+    return torch.cat(outs, dim=2).permute(0, 2, 1, 3, 4)
+
+
+def decode_to_pixel(latent, W, st=None):
+    """decode_frames followed by the clamp to [-1, 1] of utils/wan_wrapper.py:109."""
+    return decode_frames(latent, W, st).clamp(-1, 1)

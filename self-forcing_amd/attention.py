@@ -110,7 +110,8 @@ def attention(q, k, v, q_lens=None, k_lens=None, dropout_p=0., softmax_scale=Non
               window_size=(-1, -1), deterministic=False, dtype=torch.bfloat16, fa_version=None, return_lse=False):
     """softmax(q k^T * scale) v on [B, L, H, D] tensors.  Dtypes as in the reference's flash path (attention.py:62-70,
     135-138): float16 / bfloat16 inputs are used as they are, anything else is cast to `dtype`, and the result comes
-    back in q's original dtype."""
+    back in q's original dtype.  dtype=torch.float32 (which the reference does not accept) keeps fp32 inputs on the
+    fp32 kernel."""
     if causal or dropout_p != 0. or window_size != (-1, -1):
         raise NotImplementedError("only non-causal, dropout-free, full-window attention is built")
     if q_lens is not None or k_lens is not None:
@@ -119,8 +120,8 @@ def attention(q, k, v, q_lens=None, k_lens=None, dropout_p=0., softmax_scale=Non
     _check4("k", k, None, q.device)
     _check4("v", v, None, q.device)
     half_dtypes = (torch.float16, torch.bfloat16)
-    if dtype not in half_dtypes:
-        raise ValueError("dtype must be float16 or bfloat16")
+    if dtype not in half_dtypes + (torch.float32,):
+        raise ValueError("dtype must be float16, bfloat16 or float32")
     out_dtype = q.dtype
     if q_scale is not None:
         q = q * q_scale

@@ -92,3 +92,32 @@ def test_fp16_decode_streams_on_the_hip_path():
     err = (got - want).abs()
     assert err.max() < 1.5e-2 and err.mean() < 2e-3, (err.max().item(), err.mean().item())
 
+
+
+def _reference_fixture(dtype):
+    """The decoder at dim=32 with the fixture's seeded weights, the latent, and the output of the reference's own
+    `decode` (clamped as its wrapper does): tests/golden/vae_reference_vectors.npz."""
+    from test_vae_reference_vectors import reference_decoder
+    m, lat, want = reference_decoder()
+    return m.to("cuda", dtype), lat, want
+
+
+def test_fp32_decode_reproduces_the_reference_output():
+    m, lat, want = _reference_fixture(torch.float32)
+    got = m.decode_to_pixel(lat.float().cuda()).cpu().double()
+    torch.testing.assert_close(got, want, atol=2e-4, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("split", [(5,), (2, 3)])
+def test_hip_convolution_path_reproduces_the_reference_output(dtype, split):
+    """The channels-last 16-bit path (own convolution kernels) whole and as the reference's `cached_decode` chunks."""
+    m, lat, want = _reference_fixture(dtype)
+    st, outs, t0 = m.new_state(), [], 0
+    for n in split:
+        outs.append(m.decode_to_pixel(lat[:, t0:t0 + n].to(dtype).cuda(), use_cache=True, state=st))
+        t0 += n
+    assert st.layout == "cl"
+    err = (torch.cat(outs, 1).cpu().double() - want).abs()
+    bar = (6e-2, 8e-3) if dtype == torch.bfloat16 else (1e-2, 1.5e-3)
+    assert err.max() < bar[0] and err.mean() < bar[1], (err.max().item(), err.mean().item())
