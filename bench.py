@@ -30,11 +30,84 @@ ROWS = B * H * A * B2 * F * B1                        # rows of Kbar / Y
 STEP1_BYTES = (2 * SKV + SQ) * H * D * 2 + 2 * ROWS * D * 2 + ROWS * 4      # read K,V,Q; write Kbar,Y,cl
 STEP2_BYTES = 2 * ROWS * D * 2 + ROWS * 4 + 2 * SQ * H * D * 2              # read Kbar,Y,cl,Q; write O
 
-# HBM bytes per launch measured with rocprofv3 (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 1 GiB
-# device copy in the same run); the runs and raw counters are in profiles/monarch_step{1,2}_c2.md.
-MEASURED_TRAFFIC = {"monarch_step1_kernel": 881.0e6, "monarch_step2_kernel": 637.6e6}
-
 LAYERS, CHUNKS, PASSES = 30, 7, 5
+
+# the rollouts --config selects: (BASELINE.json entry, model size, attention flags, description)
+ROLLOUTS = {
+    "c3": ("configs[2]", "1.3B", dict(use_framewise=True),
+           "random-init causal Wan-1.3B (30 layers, dim 1536, 12x128 heads, FFN 8960), Monarch framewise attention"),
+    "c4": ("configs[3]", "1.3B", dict(use_framewise=True, h_reduce=2, use_dense_init=True),
+           "random-init causal Wan-1.3B, Monarch framewise attention on the reduce2xh tiling (h_reduce=2: a=6, f=42, "
+           "b1=15, b2=52) with dense attention on the first chunk (USE_DENSE_INIT)"),
+    "c5": ("configs[4]", "14B", dict(use_framewise=True),
+           "random-init causal Wan-14B (40 layers, dim 5120, 40x128 heads, FFN 13824), Monarch framewise attention"),
+    "dense": ("configs[2] with DISABLE_MONARCH_ATTN=1", "1.3B", dict(disable_monarch=True),
+              "random-init causal Wan-1.3B, every layer on the dense chunk-vs-cache fallback"),
+}
+
+
+def measured_traffic():
+    """HBM bytes per launch of the two forward kernels from rocprofv3 counters (FETCH_SIZE, WRITE_SIZE scaled by what
+    the same counters read for a 1 GiB device copy), with the commit they were measured at: profiles/traffic.json,
+    rewritten whenever the counters are collected again.  Missing file or kernel: traffic is reported as null."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {"commit": None, "kernels": {}}
+
+
+def write_traffic(fetch_csv, write_csv):
+    """Turns the counter_collection CSVs of two rocprofv3 runs of `bench.py --op-only --no-cpu-baseline --copy-probe`
+    (`--pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`; KiB per dispatch) into profiles/traffic.json.  Each counter is scaled
+    by what it reads for the run's own 1 GiB device-to-device copies, whose traffic is known (1 GiB read, 1 GiB written)."""
+    import collections
+    import csv
+    import subprocess
+
+    def read(path, counter):
+        """kernel name -> list of per-dispatch values"""
+        per = collections.defaultdict(lambda: collections.defaultdict(float))
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] == counter:
+                    per[row["Kernel_Name"]][row["Dispatch_Id"]] += float(row["Counter_Value"])
+        return {k: list(v.values()) for k, v in per.items()}
+
+    fetch, write = read(fetch_csv, "FETCH_SIZE"), read(write_csv, "WRITE_SIZE")
+    mean = lambda v: sum(v) / len(v)
+
+    def pick(table, key):
+        """(name, mean) of the instantiation of `key` with the most dispatches (the forward's own: the backward leg
+        launches a statistics-keeping instantiation a few times)."""
+        name = max((k for k in table if key + "<" in k), key=lambda k: len(table[k]))
+        return name, mean(table[name])
+
+    def copy_factor(table):
+        """The run's 1 GiB device copies are the largest dispatches of the runtime's buffer-copy kernel."""
+        v = table["__amd_rocclr_copyBuffer"]
+        big = [x for x in v if x > 0.5 * max(v)]
+        return float(1 << 20) / mean(big), len(big)
+
+    (f_fac, n_f), (w_fac, n_w) = copy_factor(fetch), copy_factor(write)
+    kernels = {}
+    for key in ("monarch_step1_kernel", "monarch_step2_kernel", "monarch_fused_kernel", "monarch_fused_merge_kernel"):
+        if any(key + "<" in k for k in fetch):
+            (name, fk), (_, wk) = pick(fetch, key), pick(write, key)
+            kernels[key] = {"instantiation": name.split("(")[0], "dispatches": len(fetch[name]), "fetch_size_kib": fk,
+                            "write_size_kib": wk, "traffic_bytes": round((fk * f_fac + wk * w_fac) * 1024)}
+    commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    dirty = subprocess.run(["git", "-C", ROOT, "status", "--porcelain", "--", "self-forcing_amd/csrc"], capture_output=True,
+                           text=True).stdout.strip()
+    rec = {"commit": (commit + ("+uncommitted kernel changes" if dirty else "")) or None,
+           "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -- python3 bench.py --op-only "
+                      "--no-cpu-baseline --copy-probe, then python bench.py --write-traffic FETCH.csv WRITE.csv",
+           "copy_kernel": "__amd_rocclr_copyBuffer", "copy_dispatches": [n_f, n_w], "fetch_factor": f_fac,
+           "write_factor": w_fac, "kernels": kernels}
+    with open(os.path.join(ROOT, "profiles", "traffic.json"), "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    print(json.dumps(rec, indent=1))
 
 
 def cpu_baseline(torch):
@@ -183,6 +256,8 @@ def op_level(torch, sfa, args):
     L.check(lib.sfm_probe_row_stream(s2_waves, s2_kb, ws.data_ptr(), ws.numel(), stream, C.byref(read_us)))
     del ws
 
+    traffic = measured_traffic()
+    t_of = lambda k: traffic["kernels"].get(k, {}).get("traffic_bytes")
     s1_gbs = STEP1_BYTES / (s1_ms * 1e-3) / 1e9
     s2_gbs = STEP2_BYTES / (s2_ms * 1e-3) / 1e9
     tfl = MONARCH_FLOPS / (ms_call * 1e-3) / 1e12
@@ -198,12 +273,14 @@ def op_level(torch, sfa, args):
                            "bwd_ms_per_call": dense_bwd["all_keys"], "bwd_ms_per_call_new_chunk_keys": dense_bwd["new_chunk_keys"]},
         "roofline": {"kernel": "monarch_step1_kernel (configs[1] shape)", "bound": "hbm", "achieved": s1_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s1_gbs / HBM_PEAK_GBS,
-                     "algorithmic_bytes": STEP1_BYTES, "traffic": MEASURED_TRAFFIC["monarch_step1_kernel"],
+                     "algorithmic_bytes": STEP1_BYTES, "traffic": t_of("monarch_step1_kernel"),
+                     "traffic_measured_at_commit": traffic["commit"],
                      "copy_probe_gbs": copy_gbs, "frac_of_copy_probe": s1_gbs / copy_gbs,
                      "traffic_only_us": floor_us.value, "frac_of_traffic_only": floor_us.value / (s1_ms * 1e3)},
         "roofline_step2": {"kernel": "monarch_step2_kernel (configs[1] shape)", "bound": "hbm", "achieved": s2_gbs,
                            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": s2_gbs / HBM_PEAK_GBS,
-                           "algorithmic_bytes": STEP2_BYTES, "traffic": MEASURED_TRAFFIC["monarch_step2_kernel"],
+                           "algorithmic_bytes": STEP2_BYTES, "traffic": t_of("monarch_step2_kernel"),
+                           "traffic_measured_at_commit": traffic["commit"],
                            "copy_probe_gbs": copy_gbs, "frac_of_copy_probe": s2_gbs / copy_gbs,
                            "traffic_only_us": read_us.value, "frac_of_traffic_only": read_us.value / (s2_ms * 1e3)},
     }
@@ -234,16 +311,28 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3, help="timed videos (21 latent frames each)")
     ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--config", choices=sorted(ROLLOUTS), default="c3",
+                    help="the rollout that `value` measures: c3 = BASELINE.json configs[2] (the headline), c4 = configs[3] "
+                         "(reduce2xh + dense first chunk), c5 = configs[4] (14B), dense = the 1.3B model with Monarch "
+                         "disabled.  The op-level legs are the same for all; the VAE leg and the CPU baseline belong to c3")
     ap.add_argument("--heads-per-pass", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--op-only", action="store_true", help="skip the model; time the attention op only")
+    ap.add_argument("--rollout-only", action="store_true",
+                    help="for kernel traces: the rollout alone, without the op-level legs, the VAE leg and the CPU baseline "
+                         "(the line then carries no roofline)")
     ap.add_argument("--one-kernel", action="store_true",
                     help="op-level figures of the opt-in one-kernel Monarch forward (Kbar / Y kept in LDS) instead of the default "
                          "two kernels; kernel_ms then holds the fused kernel and its merge kernel")
     ap.add_argument("--copy-probe", action="store_true",
                     help="accepted for the profile commands; the 1 GiB device copies (known HBM traffic, for scaling rocprof "
                          "counters) always run")
+    ap.add_argument("--write-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: rewrite profiles/traffic.json from two rocprofv3 counter_collection CSVs")
     args = ap.parse_args()
+    if args.write_traffic:
+        write_traffic(*args.write_traffic)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
@@ -252,18 +341,18 @@ def main():
     import self_forcing_amd as sfa
 
     torch.cuda.set_device(0)
-    rec = {"metric": "latent frames/s, causal Wan-1.3B 480x832 bf16 (+ Monarch attn ms/call, MFMA %)",
+    entry, size, flags, what = ROLLOUTS[args.config]
+    rec = {"metric": f"latent frames/s, causal Wan-{size} 480x832 bf16 (+ Monarch attn ms/call, MFMA %)",
            "unit": "latent frames/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-           "config": {"workload": "configs[2]: random-init causal Wan-1.3B (30 layers, dim 1536, 12x128 heads, FFN 8960), "
-                                  "latents 21x16x60x104 in 7 chunks of 3 frames, 4 denoising steps + 1 cache-refresh "
-                                  "pass per chunk, Monarch framewise attention, per-layer KV cache, text context "
-                                  "[1,512,4096] ~ N(0,1); VAE and text encoder excluded",
-                      "heads_per_pass": args.heads_per_pass}}
+           "config": {"workload": f"{entry}: {what}, latents 21x16x60x104 in 7 chunks of 3 frames, 4 denoising steps + 1 "
+                                  "cache-refresh pass per chunk, per-layer KV cache, text context [1,512,4096] ~ N(0,1); "
+                                  "VAE and text encoder excluded",
+                      "name": args.config, "heads_per_pass": args.heads_per_pass}}
     if not args.op_only:
         pl = sfa.pipeline
         pl.use_tuned_gemms()          # hipBLASLt solution per GEMM shape (shipped selections; unknown shapes tuned in warm-up)
-        gen = pl.build_generator("1.3B", attention_flags=dict(use_framewise=True))
+        gen = pl.build_generator(size, attention_flags=flags)
         pipe = pl.CausalInferencePipeline(gen)
         g = torch.Generator().manual_seed(0)
         noise = torch.randn(1, 21, 16, 60, 104, generator=g).to(torch.bfloat16).cuda()
@@ -282,13 +371,17 @@ def main():
         del pipe, gen
         torch.cuda.empty_cache()
         torch.cuda.tunable.tuning_enable(False)       # the legs below keep the selections made so far and tune nothing new
+    if args.rollout_only:
+        print(json.dumps(rec))
+        return
     rec.update(op_level(torch, sfa, args))
-    rec["vae_decode"] = vae_decode_leg(torch, sfa)
+    if args.config == "c3":
+        rec["vae_decode"] = vae_decode_leg(torch, sfa)
     if args.op_only:
         rec["metric"] = "Monarch attn ms/call, causal Wan-1.3B 480x832 chunk shape, bf16"
         rec["unit"], rec["higher_is_better"] = "ms/call", False
         rec["value"] = rec["ms_per_step"] = rec["monarch_attn"]["ms_per_call"]
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.config == "c3":
         rec["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(rec))
 
