@@ -116,7 +116,7 @@ typedef struct sfm_monarch_bwd_desc {
 } sfm_monarch_bwd_desc;
 
 int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t heads_per_pass, size_t* bytes);
-/* 1 when rocBLAS was found at run time and SFM_BWD_SIMT is unset.  The backward is a chain of parts, each a fused
+/* 1 when rocBLAS was found at run time and the SFM_SW_BWD_SIMT switch is off.  The backward is a chain of parts, each a fused
  * MFMA kernel where the problem allows (16-bit tensors, head_dim 64 / 128, b1 <= 32, b2 <= 64 a multiple of 4, at
  * most 480 (a, j) columns) and batched rocBLAS GEMMs + row kernels otherwise; when every part is fused the chain
  * runs with or without rocBLAS, else without rocBLAS the fp32 SIMT kernels run.  The first GEMM call on a device
@@ -304,6 +304,23 @@ int sfm_probe_tile_traffic(int32_t tiles, int32_t rows_in, int32_t rows_out, int
  * the mean duration of one pass in microseconds, which bench.py reports beside step 2's own duration. */
 int sfm_probe_row_stream(int32_t waves, int32_t kb_per_block, const void* workspace, size_t workspace_bytes, void* stream,
                          float* us);
+
+/* Implementation switches for measurements and tests; no counterpart in the reference.  The environment is read
+ * ONCE, when the library is loaded: a variable of the same name as a bit below that is set to anything but "0" turns
+ * the bit on (SFM_BWD_SIMT=1 ...), SFM_NO_ROCBLAS makes the library behave as where rocBLAS is absent, and SFM_S1_WGS=n
+ * overrides the step-1 workgroup count.  No entry point reads the environment afterwards; sfm_set_switches replaces the
+ * mask for the whole process (returns the previous one; unknown bits are rejected with (unsigned)-1 and leave it
+ * unchanged), which is how the tests reach every path from one process.  Workspace queries follow the mask, so change it
+ * only between a query and the call it sizes, never in between. */
+#define SFM_SW_BWD_SIMT        0x01u  /* backward on the fp32 SIMT kernels */
+#define SFM_SW_BWD_LEFT_GEMM   0x02u  /* backward parts on the batched library GEMMs instead of their fused kernels: */
+#define SFM_SW_BWD_FWD_GEMM    0x04u
+#define SFM_SW_BWD_DQA_GEMM    0x08u
+#define SFM_SW_BWD_RIGHT_GEMM  0x10u
+#define SFM_SW_BWD_DQK_GEMM    0x20u
+#define SFM_SW_ALL             0x3fu
+unsigned sfm_set_switches(unsigned mask);
+unsigned sfm_get_switches(void);
 
 /* Thread-local description of the last error returned on this thread ("" if none). */
 const char* sfm_last_error(void);

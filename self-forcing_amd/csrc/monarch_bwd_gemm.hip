@@ -49,7 +49,7 @@ bool blas_load() {
     std::lock_guard<std::mutex> lock(g_blas_mutex);
     if (g_blas.tried) return g_blas.ok;
     g_blas.tried = true;
-    if (getenv("SFM_NO_ROCBLAS") != nullptr) return false;             // for tests: behave as where the library is absent
+    if (rocblas_disabled()) return false;                              // for tests: behave as where the library is absent
     void* lib = dlopen("librocblas.so.5", RTLD_NOW | RTLD_GLOBAL);
     if (!lib) lib = dlopen("/opt/rocm/lib/librocblas.so.5", RTLD_NOW | RTLD_GLOBAL);
     if (!lib) lib = dlopen("librocblas.so", RTLD_NOW | RTLD_GLOBAL);
@@ -404,7 +404,7 @@ template <typename E> constexpr int left_dtype() { return -1; }
 template <> constexpr int left_dtype<BF16>() { return SFM_BF16; }
 template <> constexpr int left_dtype<F16>() { return SFM_F16; }
 
-// Which parts of the chain run as fused kernels: decided by shapes, strides and (for measurements) the environment,
+// Which parts of the chain run as fused kernels: decided by shapes, strides and (for measurements) the process-wide switches,
 // so that the workspace query and the run agree.
 struct Parts {
     bool left;     // 4-7: statistics and gradients of the left factor without the [i x r] matrices in memory
@@ -416,17 +416,18 @@ struct Parts {
 
 Parts make_parts(const MonarchArgs& p, int dtype, const int64_t* dks) {
     Parts f;
+    const unsigned sw = switches();
     const bool h16 = dtype == SFM_BF16 || dtype == SFM_F16;
     const bool q_rows_ok = (p.qs[0] | p.qs[1] | p.qs[2] | p.os[0] | p.os[1] | p.os[2]) % 8 == 0 &&       // 16-byte rows of q, dout, out
                            (int64_t)p.na * p.b1 * p.b2 * p.qs[1] * 2 < ((int64_t)1 << 32);
-    f.left = h16 && q_rows_ok && monarch_bwd_left_supported(dtype, p.D, p.b1) && getenv("SFM_BWD_LEFT_GEMM") == nullptr;
-    f.fwd = f.left && monarch_mfma_supported(dtype, p.D, p.b2) && getenv("SFM_BWD_FWD_GEMM") == nullptr;
-    f.dqa = f.left && getenv("SFM_BWD_DQA_GEMM") == nullptr;
+    f.left = h16 && q_rows_ok && monarch_bwd_left_supported(dtype, p.D, p.b1) && !(sw & SFM_SW_BWD_LEFT_GEMM);
+    f.fwd = f.left && monarch_mfma_supported(dtype, p.D, p.b2) && !(sw & SFM_SW_BWD_FWD_GEMM);
+    f.dqa = f.left && !(sw & SFM_SW_BWD_DQA_GEMM);
     const bool direct_ok = (dks[0] | dks[1] | dks[2] | p.vs[0] | p.vs[1] | p.vs[2] | p.ks[0] | p.ks[1] | p.ks[2]) % 8 == 0 &&      // 16-byte rows of k, v, dk, dv
                            (int64_t)p.nf * p.b1 * p.b2 * p.ks[1] * 2 < ((int64_t)1 << 32);
     f.right = f.fwd && direct_ok && monarch_bwd_right_supported(dtype, p.D, p.b2, p.na * p.b2) &&
-              getenv("SFM_BWD_RIGHT_GEMM") == nullptr;
-    f.dqk = f.right && monarch_bwd_dqk_supported(dtype, p.D, p.b2, p.na * p.b2) && getenv("SFM_BWD_DQK_GEMM") == nullptr;
+              !(sw & SFM_SW_BWD_RIGHT_GEMM);
+    f.dqk = f.right && monarch_bwd_dqk_supported(dtype, p.D, p.b2, p.na * p.b2) && !(sw & SFM_SW_BWD_DQK_GEMM);
     return f;
 }
 

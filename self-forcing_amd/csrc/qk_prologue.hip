@@ -53,15 +53,21 @@ template <class E> struct Row8_16 {
 template <> struct Row8<BF16> : Row8_16<BF16> {};
 template <> struct Row8<F16> : Row8_16<F16> {};
 
-constexpr int kMaxChunksPerThread = 4;   // 256 threads x 4 chunks x 8 elements = model dim <= 8192
+constexpr int kMaxThreads = 512;
 
-template <typename T>
-__global__ __launch_bounds__(256) void qk_prologue_kernel(sfm_prologue_desc p, TokMap map, const void* xq, const void* xk,
-                                                          const void* xv, const void* wq, const void* wk,
-                                                          const double* __restrict__ rope, void* q_out, void* kc, void* vc) {
+// One workgroup per token, CPT chunks of 8 elements per thread, blockDim = the chunk count of a row divided by CPT and
+// rounded up to whole waves (192 threads at model dim 1536, 320 x 2 chunks at 5120), so that no lane idles.  Every load
+// a thread needs (its q, k, v chunks, the two norm weights, its four rotation pairs) is issued before the row's sum of
+// squares is reduced; the reduction is the only point where the waves of a token meet.  The sums of squares are
+// accumulated in float64 (per thread over its chunks, then a butterfly over the wave, then the waves in order).
+template <typename T, int CPT>
+__global__ __launch_bounds__(kMaxThreads) void qk_prologue_kernel(sfm_prologue_desc p, TokMap map, const void* xq,
+                                                                  const void* xk, const void* xv, const void* wq,
+                                                                  const void* wk, const double* __restrict__ rope,
+                                                                  void* q_out, void* kc, void* vc) {
     using R8 = Row8<T>;
-    __shared__ double red[2][4];
-    const int tid = threadIdx.x;
+    __shared__ double red[2][kMaxThreads / 64];
+    const int tid = threadIdx.x, nt = blockDim.x;
     const int b = blockIdx.x / p.S;
     const int s = blockIdx.x % p.S;
     const int D = p.D, C = p.H * p.D;
@@ -76,26 +82,53 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(sfm_prologue_desc p, T
     const int e = col / map.ww, j = col - e * map.ww;
     const int bf = (A * map.h_reduce + c) * map.w_reduce + e;
     const int64_t crow = p.start_idx + ((int64_t)bf * map.b1 + (ft * map.hh + ii)) * map.b2 + j;
+    const int64_t cbase = (int64_t)b * p.cache_stride[0] + crow * p.cache_stride[1];
 
     const int64_t xoff = (int64_t)b * p.x_stride[0] + (int64_t)s * p.x_stride[1];
-    float q[kMaxChunksPerThread][8], k[kMaxChunksPerThread][8];
+    float q[CPT][8], k[CPT][8], wqv[CPT][8], wkv[CPT][8];
     double sq = 0.0, sk = 0.0;
 #pragma unroll
-    for (int t = 0; t < kMaxChunksPerThread; ++t) {
-        const int ch = tid + t * 256;
+    for (int t = 0; t < CPT; ++t) {
+        const int ch = tid + t * nt;
         if (ch < nchunk) {
             R8::load(xq, xoff + ch * 8, q[t]);
             R8::load(xk, xoff + ch * 8, k[t]);
+            float v[8];
+            R8::load(xv, xoff + ch * 8, v);
+            R8::load(wq, ch * 8, wqv[t]);
+            R8::load(wk, ch * 8, wkv[t]);
+            // V is copied as is
+            const int hd = (ch * 8) / D, d0 = (ch * 8) % D;
+            R8::store(vc, cbase + (int64_t)hd * p.cache_stride[2] + d0, v);
+        }
+    }
+    // the rotation pairs of a thread's chunks: the same for every chunk when the block's stride is a multiple of the
+    // head dim (always so for power-of-two head dims up to 512), fetched per chunk otherwise
+    const int half = D / 2;
+    const int n0 = half - 2 * (half / 3), n1 = half / 3;
+    const int pos0 = frame + p.start_frame;
+    const bool same_pairs = (nt * 8) % D == 0;
+    double cs[4], sn[4];
+    auto load_pairs = [&](int d0) {
+#pragma unroll
+        for (int pr = 0; pr < 4; ++pr) {
+            const int mpair = d0 / 2 + pr;
+            const int pos = mpair < n0 ? pos0 : (mpair < n0 + n1 ? row : col);
+            const double2 v = *(const double2*)(rope + ((int64_t)pos * half + mpair) * 2);
+            cs[pr] = v.x;
+            sn[pr] = v.y;
+        }
+    };
+    if (same_pairs) load_pairs((tid * 8) % D);
+
+#pragma unroll
+    for (int t = 0; t < CPT; ++t) {
+        if (tid + t * nt < nchunk) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 sq += (double)q[t][i] * q[t][i];
                 sk += (double)k[t][i] * k[t][i];
             }
-            // V is copied as is
-            float v[8];
-            R8::load(xv, xoff + ch * 8, v);
-            const int hd = (ch * 8) / D, d0 = (ch * 8) % D;
-            R8::store(vc, (int64_t)b * p.cache_stride[0] + crow * p.cache_stride[1] + (int64_t)hd * p.cache_stride[2] + d0, v);
         }
     }
 #pragma unroll
@@ -108,54 +141,62 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(sfm_prologue_desc p, T
         red[1][tid >> 6] = sk;
     }
     __syncthreads();
-    sq = red[0][0] + red[0][1] + red[0][2] + red[0][3];
-    sk = red[1][0] + red[1][1] + red[1][2] + red[1][3];
+    sq = sk = 0.0;
+    for (int w = 0; w < nt / 64; ++w) {
+        sq += red[0][w];
+        sk += red[1][w];
+    }
     const float rq = 1.0f / sqrtf((float)(sq / C) + p.eps);
     const float rk = 1.0f / sqrtf((float)(sk / C) + p.eps);
 
-    const int half = D / 2;
-    const int n0 = half - 2 * (half / 3), n1 = half / 3;
-    const int pos0 = frame + p.start_frame;
 #pragma unroll
-    for (int t = 0; t < kMaxChunksPerThread; ++t) {
-        const int ch = tid + t * 256;
+    for (int t = 0; t < CPT; ++t) {
+        const int ch = tid + t * nt;
         if (ch < nchunk) {
-            float wqv[8], wkv[8];
-            R8::load(wq, ch * 8, wqv);
-            R8::load(wk, ch * 8, wkv);
             const int hd = (ch * 8) / D, d0 = (ch * 8) % D;
+            if (!same_pairs) load_pairs(d0);
             float oq[8], ok[8];
 #pragma unroll
             for (int pr = 0; pr < 4; ++pr) {
-                const int mpair = d0 / 2 + pr;
-                const int pos = mpair < n0 ? pos0 : (mpair < n0 + n1 ? row : col);
-                const double cs = rope[((int64_t)pos * half + mpair) * 2];
-                const double sn = rope[((int64_t)pos * half + mpair) * 2 + 1];
-                const double q0 = R8::rnd(R8::rnd(q[t][2 * pr] * rq) * wqv[2 * pr]);
-                const double q1 = R8::rnd(R8::rnd(q[t][2 * pr + 1] * rq) * wqv[2 * pr + 1]);
-                const double k0 = R8::rnd(R8::rnd(k[t][2 * pr] * rk) * wkv[2 * pr]);
-                const double k1 = R8::rnd(R8::rnd(k[t][2 * pr + 1] * rk) * wkv[2 * pr + 1]);
-                oq[2 * pr] = (float)(q0 * cs - q1 * sn);
-                oq[2 * pr + 1] = (float)(q0 * sn + q1 * cs);
-                ok[2 * pr] = (float)(k0 * cs - k1 * sn);
-                ok[2 * pr + 1] = (float)(k0 * sn + k1 * cs);
+                const double q0 = R8::rnd(R8::rnd(q[t][2 * pr] * rq) * wqv[t][2 * pr]);
+                const double q1 = R8::rnd(R8::rnd(q[t][2 * pr + 1] * rq) * wqv[t][2 * pr + 1]);
+                const double k0 = R8::rnd(R8::rnd(k[t][2 * pr] * rk) * wkv[t][2 * pr]);
+                const double k1 = R8::rnd(R8::rnd(k[t][2 * pr + 1] * rk) * wkv[t][2 * pr + 1]);
+                oq[2 * pr] = (float)(q0 * cs[pr] - q1 * sn[pr]);
+                oq[2 * pr + 1] = (float)(q0 * sn[pr] + q1 * cs[pr]);
+                ok[2 * pr] = (float)(k0 * cs[pr] - k1 * sn[pr]);
+                ok[2 * pr + 1] = (float)(k0 * sn[pr] + k1 * cs[pr]);
             }
             R8::store(q_out, (int64_t)b * p.q_stride[0] + (int64_t)s * p.q_stride[1] + (int64_t)hd * p.q_stride[2] + d0, oq);
-            R8::store(kc, (int64_t)b * p.cache_stride[0] + crow * p.cache_stride[1] + (int64_t)hd * p.cache_stride[2] + d0, ok);
+            R8::store(kc, cbase + (int64_t)hd * p.cache_stride[2] + d0, ok);
         }
     }
 }
 
+template <typename T>
+static void launch_t(int cpt, dim3 grid, dim3 block, hipStream_t stream, const sfm_prologue_desc& d, const TokMap& map,
+                     const void* xq, const void* xk, const void* xv, const void* wq, const void* wk, const double* rope,
+                     void* q_out, void* kc, void* vc) {
+    if (cpt == 1)
+        hipLaunchKernelGGL((qk_prologue_kernel<T, 1>), grid, block, 0, stream, d, map, xq, xk, xv, wq, wk, rope, q_out, kc, vc);
+    else
+        hipLaunchKernelGGL((qk_prologue_kernel<T, 2>), grid, block, 0, stream, d, map, xq, xk, xv, wq, wk, rope, q_out, kc, vc);
+}
+
+// Model dims up to kMaxThreads x 2 chunks x 8 elements = 8192 (the entry point checks it).
 int launch_prologue(const sfm_prologue_desc& d, const TokMap& map, const void* xq, const void* xk, const void* xv,
                     const void* wq, const void* wk, const double* rope, void* q_out, void* kc, void* vc,
                     hipStream_t stream) {
-    dim3 grid((unsigned)((int64_t)d.B * d.S));
+    const int nchunk = d.H * d.D / 8;
+    const int cpt = nchunk > kMaxThreads ? 2 : 1;
+    const int nt = (((nchunk + cpt - 1) / cpt) + 63) / 64 * 64;
+    dim3 grid((unsigned)((int64_t)d.B * d.S)), block(nt);
     if (d.dtype == SFM_BF16)
-        hipLaunchKernelGGL((qk_prologue_kernel<BF16>), grid, dim3(256), 0, stream, d, map, xq, xk, xv, wq, wk, rope, q_out, kc, vc);
+        launch_t<BF16>(cpt, grid, block, stream, d, map, xq, xk, xv, wq, wk, rope, q_out, kc, vc);
     else if (d.dtype == SFM_F16)
-        hipLaunchKernelGGL((qk_prologue_kernel<F16>), grid, dim3(256), 0, stream, d, map, xq, xk, xv, wq, wk, rope, q_out, kc, vc);
+        launch_t<F16>(cpt, grid, block, stream, d, map, xq, xk, xv, wq, wk, rope, q_out, kc, vc);
     else
-        hipLaunchKernelGGL((qk_prologue_kernel<float>), grid, dim3(256), 0, stream, d, map, xq, xk, xv, wq, wk, rope, q_out, kc, vc);
+        launch_t<float>(cpt, grid, block, stream, d, map, xq, xk, xv, wq, wk, rope, q_out, kc, vc);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) {
         set_error("hip launch failed: %s", hipGetErrorString(err));

@@ -1,5 +1,6 @@
 // extern "C" entry points: argument validation, workspace accounting, pass scheduling.
 #include <pthread.h>
+#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -10,6 +11,37 @@
 namespace sfm {
 
 static thread_local char g_err[512] = "";
+
+namespace {
+// The environment is read here, once, when the library is loaded; nothing reads it afterwards.
+struct Switches {
+    std::atomic<unsigned> mask{0};
+    bool no_rocblas = false;
+    int s1_wgs = 0;
+    Switches() {
+        static const struct { const char* name; unsigned bit; } names[] = {
+            {"SFM_BWD_SIMT", SFM_SW_BWD_SIMT},           {"SFM_BWD_LEFT_GEMM", SFM_SW_BWD_LEFT_GEMM},
+            {"SFM_BWD_FWD_GEMM", SFM_SW_BWD_FWD_GEMM},   {"SFM_BWD_DQA_GEMM", SFM_SW_BWD_DQA_GEMM},
+            {"SFM_BWD_RIGHT_GEMM", SFM_SW_BWD_RIGHT_GEMM}, {"SFM_BWD_DQK_GEMM", SFM_SW_BWD_DQK_GEMM}};
+        unsigned m = 0;
+        for (const auto& n : names) {
+            const char* e = getenv(n.name);
+            if (e && strcmp(e, "0") != 0) m |= n.bit;
+        }
+        mask.store(m);
+        no_rocblas = getenv("SFM_NO_ROCBLAS") != nullptr;
+        if (const char* e = getenv("SFM_S1_WGS")) {
+            const int v = atoi(e);
+            if (v >= 1 && v <= 65535) s1_wgs = v;
+        }
+    }
+};
+Switches g_sw;
+}  // namespace
+
+unsigned switches() { return g_sw.mask.load(std::memory_order_relaxed); }
+bool rocblas_disabled() { return g_sw.no_rocblas; }
+int step1_wgs_override() { return g_sw.s1_wgs; }
 
 void set_error(const char* fmt, ...) {
     va_list ap;
@@ -226,7 +258,17 @@ using namespace sfm;
 
 extern "C" {
 
-int sfm_version(void) { return 6; }
+int sfm_version(void) { return 7; }
+
+unsigned sfm_set_switches(unsigned mask) {
+    if (mask & ~SFM_SW_ALL) {
+        set_error("unknown switch bits 0x%x", mask & ~SFM_SW_ALL);
+        return (unsigned)-1;
+    }
+    return g_sw.mask.exchange(mask);
+}
+
+unsigned sfm_get_switches(void) { return switches(); }
 
 const char* sfm_last_error(void) { return g_err; }
 
@@ -274,11 +316,7 @@ static void init_args(const sfm_monarch_desc* desc, const MonarchPlan& pl, Monar
     a.n_achunks = (pl.na + a_max - 1) / a_max;
     a.a_chunk = (pl.na + a.n_achunks - 1) / a.n_achunks;
     a.n_achunks = (pl.na + a.a_chunk - 1) / a.a_chunk;
-    a.s1_wgs = 0;
-    if (const char* e = getenv("SFM_S1_WGS")) {            // tuning override: step-1 workgroups (default one per CU)
-        int v = atoi(e);
-        if (v >= 1 && v <= 65535) a.s1_wgs = v;
-    }
+    a.s1_wgs = step1_wgs_override();            // tuning override: step-1 workgroups (default 0: one per CU)
 }
 
 static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const void* k, const void* v, void* out,
@@ -461,10 +499,9 @@ static int plan_bwd(const sfm_monarch_bwd_desc* bd, MonarchPlan* pl, size_t* per
     return SFM_OK;
 }
 
-// The batched-GEMM backward is used whenever rocBLAS can be loaded; SFM_BWD_SIMT=1 selects the fp32 SIMT kernels.
+// The batched-GEMM backward is used whenever rocBLAS can be loaded; the SFM_SW_BWD_SIMT switch selects the fp32 SIMT kernels.
 static bool bwd_uses_gemm() {
-    const char* e = getenv("SFM_BWD_SIMT");
-    if (e && atoi(e) != 0) return false;
+    if (switches() & SFM_SW_BWD_SIMT) return false;
     return monarch_bwd_gemm_available();
 }
 
@@ -473,8 +510,7 @@ int sfm_monarch_bwd_uses_gemm(void) { return bwd_uses_gemm() ? 1 : 0; }
 // The chain of fused kernels and library products runs when rocBLAS is there, and also without it when every part of
 // the chain has a fused kernel for this problem.
 static bool bwd_uses_chain(const sfm_monarch_bwd_desc* desc, const MonarchPlan& pl) {
-    const char* e = getenv("SFM_BWD_SIMT");
-    if (e && atoi(e) != 0) return false;
+    if (switches() & SFM_SW_BWD_SIMT) return false;
     if (monarch_bwd_gemm_available()) return true;
     MonarchArgs a;
     init_args(&desc->fwd, pl, &a);

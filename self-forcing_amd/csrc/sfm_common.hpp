@@ -189,6 +189,10 @@ int launch_monarch_fused(const MonarchArgs& a, int dtype, int nunits, void* ws, 
 int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
 int launch_monarch_bwd(const MonarchBwdArgs& g, int dtype, int nunits, hipStream_t stream);
 bool monarch_bwd_gemm_available();
+// process-wide implementation switches (SFM_SW_* of the header), read from the environment once at load
+unsigned switches();
+bool rocblas_disabled();           // SFM_NO_ROCBLAS was set at load
+int step1_wgs_override();          // SFM_S1_WGS at load, 0 = none
 // every part of the chain runs as a fused kernel for this problem: no library GEMM is called
 bool monarch_bwd_all_fused(const MonarchArgs& p, int dtype, const int64_t* dkv_stride);
 size_t monarch_bwd_gemm_bytes(const MonarchArgs& p, int dtype, int nunits, const int64_t* dkv_stride);

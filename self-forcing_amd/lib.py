@@ -12,6 +12,8 @@ LIB_PATH = os.path.join(HERE, "libsfm_attn.so")
 SFM_BF16, SFM_F16, SFM_F32 = 0, 1, 2
 SFM_MONARCH_ONE_KERNEL = 1
 STATIC_SCRATCH_BYTES = 128 << 20      # SFM_STATIC_SCRATCH_BYTES of include/sfm_attn.h
+# SFM_SW_* of include/sfm_attn.h: process-wide implementation switches (sfm_set_switches)
+SW_BWD_SIMT, SW_BWD_LEFT_GEMM, SW_BWD_FWD_GEMM, SW_BWD_DQA_GEMM, SW_BWD_RIGHT_GEMM, SW_BWD_DQK_GEMM = (1 << i for i in range(6))
 
 ERR_NAMES = {
     -1: "SFM_ERR_NULL", -2: "SFM_ERR_DTYPE", -3: "SFM_ERR_SHAPE", -4: "SFM_ERR_RANGE", -5: "SFM_ERR_STRIDE",
@@ -24,7 +26,7 @@ SYMBOLS = [
     "sfm_monarch_attn_with_kv_cache_static",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
     "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm",
-    "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_dense_bwd_workspace_bytes", "sfm_dense_bwd", "sfm_probe_mfma_bf16", "sfm_probe_tile_traffic", "sfm_probe_row_stream", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_last_error", "sfm_version",
+    "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_dense_bwd_workspace_bytes", "sfm_dense_bwd", "sfm_probe_mfma_bf16", "sfm_probe_tile_traffic", "sfm_probe_row_stream", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_set_switches", "sfm_get_switches", "sfm_last_error", "sfm_version",
 ]
 
 
@@ -121,8 +123,10 @@ def load():
     lib.sfm_probe_mfma_bf16.argtypes = [C.c_int32, P, C.POINTER(C.c_float)]
     lib.sfm_probe_tile_traffic.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, P, C.c_size_t, P, C.POINTER(C.c_float)]
     lib.sfm_probe_row_stream.argtypes = [C.c_int32, C.c_int32, P, C.c_size_t, P, C.POINTER(C.c_float)]
+    lib.sfm_set_switches.argtypes = [C.c_uint]
+    lib.sfm_set_switches.restype = lib.sfm_get_switches.restype = C.c_uint
     for name in SYMBOLS:
-        if name not in ("sfm_version", "sfm_last_error"):
+        if name not in ("sfm_version", "sfm_last_error", "sfm_set_switches", "sfm_get_switches"):
             getattr(lib, name).restype = C.c_int
     _lib = lib
     return lib

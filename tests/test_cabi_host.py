@@ -23,7 +23,40 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 9 and set(names) == set(L.SYMBOLS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sfm_version() == 6
+    assert lib.sfm_version() == 7
+
+
+def test_switches_are_a_process_wide_mask_set_through_the_abi():
+    """The implementation switches: header constants == binding constants, set returns the previous mask, unknown bits
+    are refused and leave the mask alone, and the workspace query of the backward follows the mask."""
+    lib = L.load()
+    text = open(os.path.join(ROOT, "include", "sfm_attn.h")).read()
+    for i, name in enumerate(("BWD_SIMT", "BWD_LEFT_GEMM", "BWD_FWD_GEMM", "BWD_DQA_GEMM", "BWD_RIGHT_GEMM", "BWD_DQK_GEMM")):
+        assert re.search(rf"#define\s+SFM_SW_{name}\s+0x{1 << i:02x}u", text), name
+        assert getattr(L, "SW_" + name) == 1 << i
+    old = lib.sfm_get_switches()
+    try:
+        assert lib.sfm_set_switches(L.SW_BWD_SIMT) == old
+        assert lib.sfm_get_switches() == L.SW_BWD_SIMT and lib.sfm_monarch_bwd_uses_gemm() == 0
+        assert lib.sfm_set_switches(0x40) == 0xFFFFFFFF and b"unknown switch" in lib.sfm_last_error()
+        assert lib.sfm_get_switches() == L.SW_BWD_SIMT
+    finally:
+        lib.sfm_set_switches(old)
+    assert lib.sfm_get_switches() == old
+
+
+def test_environment_is_read_once_at_load():
+    """A process started with SFM_BWD_SIMT=1 has the bit set from the start; changing the variable afterwards does
+    nothing (no entry point reads the environment)."""
+    import subprocess
+    import sys
+    code = ("import os, sys; sys.path.insert(0, %r); import importlib; L = importlib.import_module('self_forcing_amd').lib; "
+            "lib = L.load(); a = lib.sfm_get_switches(); os.environ['SFM_BWD_SIMT'] = '0'; os.environ['SFM_BWD_DQK_GEMM'] = '1'; "
+            "print('MASK', a, lib.sfm_get_switches(), lib.sfm_monarch_bwd_uses_gemm())") % ROOT
+    env = dict(os.environ, SFM_BWD_SIMT="1")
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-1500:]
+    assert [ln for ln in r.stdout.splitlines() if ln.startswith("MASK")][0] == "MASK 1 1 0"
 
 
 def test_struct_sizes_match_header_layout():
