@@ -321,6 +321,9 @@ def main():
     ap.add_argument("--rollout-only", action="store_true",
                     help="for kernel traces: the rollout alone, without the op-level legs, the VAE leg and the CPU baseline "
                          "(the line then carries no roofline)")
+    ap.add_argument("--own-gemm", action="store_true",
+                    help="rollout with the FFN's linear layers on the library's own fused-epilogue kernel (sfm_linear) instead of "
+                         "hipBLASLt + element-wise kernels")
     ap.add_argument("--one-kernel", action="store_true",
                     help="op-level figures of the opt-in one-kernel Monarch forward (Kbar / Y kept in LDS) instead of the default "
                          "two kernels; kernel_ms then holds the fused kernel and its merge kernel")
@@ -352,7 +355,9 @@ def main():
     if not args.op_only:
         pl = sfa.pipeline
         pl.use_tuned_gemms()          # hipBLASLt solution per GEMM shape (shipped selections; unknown shapes tuned in warm-up)
-        gen = pl.build_generator(size, attention_flags=flags)
+        gen = pl.build_generator(size, attention_flags=flags,
+                                 ops=sfa.causal_model.HipAttentionOps(own_gemm=True) if args.own_gemm else None)
+        rec["config"]["own_gemm"] = bool(args.own_gemm)
         pipe = pl.CausalInferencePipeline(gen)
         g = torch.Generator().manual_seed(0)
         noise = torch.randn(1, 21, 16, 60, 104, generator=g).to(torch.bfloat16).cuda()

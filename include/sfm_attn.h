@@ -253,6 +253,32 @@ int sfm_gate_residual_ln(int32_t dtype, int64_t rows, int32_t C, float eps, void
                          int64_t out_stride, const void* scale, const void* shift, int64_t mod_stride, int32_t rows_per_frame,
                          const void* weight, const void* bias, void* stream);
 
+/* The block's linear layers with their element-wise tails in the matrix product's epilogue (16-bit tensors, fp32
+ * accumulation on MFMA).  x: [M, K] activations, rows x_stride elements apart; w: [N, K] contiguous (nn.Linear.weight);
+ * bias: [N] or NULL; out: [M, N], rows out_stride apart.
+ *   SFM_EPI_NONE           out = x w^T + bias                        nn.Linear (wan/modules/model.py:592-596, 632-650)
+ *   SFM_EPI_GELU_TANH      out = gelu_tanh(x w^T + bias)             the FFN's first half (model.py:648-650)
+ *   SFM_EPI_GATE_RESIDUAL  out = res + (x w^T + bias) * gate[m / rows_per_frame]   the output projections with the adaLN
+ *                          gates and the residual update (wan/modules/causal_model.py:1189, 1196, 1203-1204);
+ *                          gate = NULL: out = res + (x w^T + bias); res ([M, N], rows res_stride apart) may be `out`.
+ * Rounding points are the eager chain's: the product plus bias is rounded to the tensor dtype, the GELU of that value
+ * is rounded, the gated product is rounded, the residual sum is rounded.  K a multiple of 64, N a multiple of 8, all
+ * strides multiples of 8 elements, pointers 16-byte aligned, operands below 4 GiB each. */
+#define SFM_EPI_NONE          0
+#define SFM_EPI_GELU_TANH     1
+#define SFM_EPI_GATE_RESIDUAL 2
+typedef struct sfm_linear_desc {
+    int32_t dtype;            /* SFM_BF16 | SFM_F16 */
+    int32_t epilogue;         /* SFM_EPI_* */
+    int64_t M;
+    int32_t N, K;
+    int64_t x_stride, out_stride, res_stride, gate_stride;   /* elements */
+    int32_t rows_per_frame;   /* rows sharing one gate row (GATE_RESIDUAL with a gate) */
+    int32_t reserved;
+} sfm_linear_desc;
+int sfm_linear(const sfm_linear_desc* desc, const void* x, const void* w, const void* bias, const void* res, const void* gate,
+               void* out, void* stream);
+
 typedef struct sfm_conv_desc {
     int32_t dtype;            /* SFM_BF16 | SFM_F16 */
     int32_t T, H, W;          /* output frames, rows, columns */

@@ -63,6 +63,9 @@ class OracleOps:
     def linear_gelu(self, x, linear):
         return torch.nn.functional.gelu(linear(x), approximate='tanh')
 
+    def linear_gate_residual(self, x, h, linear, gate):
+        return self.gate_residual(x, linear(h), gate)
+
     def rms_norm(self, x, weight, eps):
         xf = x.float()
         return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)).type_as(x) * weight

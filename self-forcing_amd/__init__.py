@@ -10,6 +10,6 @@ reference's module names:
     causal_model.CausalWanModel (+ self-attention, block, head), pipeline.CausalInferencePipeline
     vae_decode.WanVAEDecoder (streaming latent -> pixel decode; channels-last HIP convolutions and norms, conv_ops)
 """
-from . import lib, monarch_attn, attention, prologue, causal_model, pipeline, vae_decode  # noqa: F401
+from . import lib, monarch_attn, attention, prologue, causal_model, pipeline, vae_decode, linear, block_ops  # noqa: F401
 
-__all__ = ["lib", "monarch_attn", "attention", "prologue", "causal_model", "pipeline", "vae_decode"]
+__all__ = ["lib", "monarch_attn", "attention", "prologue", "causal_model", "pipeline", "vae_decode", "linear"]

@@ -12,7 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsfm_attn.so")
-SOURCES = ["sfm_api.hip", "monarch_mfma.hip", "monarch_fused.hip", "monarch_generic.hip", "dense_attn.hip", "dense_attn_bwd.hip", "qk_prologue.hip", "block_fused.hip",
+SOURCES = ["sfm_api.hip", "monarch_mfma.hip", "monarch_fused.hip", "monarch_generic.hip", "dense_attn.hip", "dense_attn_bwd.hip", "qk_prologue.hip", "block_fused.hip", "block_gemm.hip",
            "monarch_bwd_gemm.hip", "monarch_bwd_left.hip", "monarch_bwd_right.hip", "probe.hip", "conv3d_cl.hip"]
 
 FLAGS = [

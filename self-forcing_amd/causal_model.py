@@ -25,6 +25,7 @@ import torch.nn.functional as F
 
 from . import attention as _attn
 from . import block_ops as _blk
+from . import linear as _lin
 from . import monarch_attn as _mon
 from . import prologue as _pro
 
@@ -36,7 +37,14 @@ TOTAL_SEQ_LEN = 21 * 30 * 52
 class HipAttentionOps:
     """The HIP operators the model calls (attention, fused prologue, fused block element-wise ops).  Tests
     may pass another object with the same methods (e.g. one built on the CPU oracle and eager torch ops) to
-    obtain a reference run of the same module code."""
+    obtain a reference run of the same module code.
+
+    own_gemm=True runs the FFN's two linear layers on the library's own matrix-product kernel with the GELU and the
+    gated residual update in its epilogue (`linear.linear`) instead of hipBLASLt + a separate element-wise kernel; it is
+    off by default because hipBLASLt's kernels are faster on MI355X at these shapes."""
+
+    def __init__(self, own_gemm=False):
+        self.own_gemm = bool(own_gemm)
 
     def rope_table(self, head_dim, device):
         return _pro.rope_table(head_dim, device=device)
@@ -72,8 +80,17 @@ class HipAttentionOps:
         """GELU(tanh)(x W^T + b) with the activation applied in the GEMM's epilogue (hipBLASLt through
         torch's addmm-with-activation); the reference runs Linear and nn.GELU(approximate='tanh') apart
         (model.py:648-650)."""
+        if self.own_gemm and _lin.supported(x, linear.weight):
+            return _lin.linear(x, linear.weight, linear.bias, epilogue="gelu_tanh")
         out = torch._addmm_activation(linear.bias, x.reshape(-1, x.shape[-1]), linear.weight.t(), use_gelu=True)
         return out.view(*x.shape[:-1], out.shape[-1])
+
+    def linear_gate_residual(self, x, h, linear, gate):
+        """x + linear(h) * gate, in place into x (the FFN's second half and the block's last residual update,
+        causal_model.py:1203-1204)."""
+        if self.own_gemm and _lin.supported(h, linear.weight):
+            return _lin.linear(h, linear.weight, linear.bias, epilogue="gate_residual", res=x, gate=gate)
+        return self.gate_residual(x, linear(h), gate)
 
 
 def _env_int(name, default):
@@ -352,8 +369,7 @@ class CausalWanAttentionBlock(nn.Module):
         else:
             x, xn = ops.gate_residual_ln(x, y, e[2], self.eps, weight=self.norm3.weight, bias=self.norm3.bias)
         x, xn = ops.gate_residual_ln(x, self.cross_attn(xn, context, crossattn_cache), None, self.eps, scale=e[4], shift=e[3])
-        y = self.ffn[2](ops.linear_gelu(xn, self.ffn[0]))
-        return ops.gate_residual(x, y, e[5])
+        return ops.linear_gate_residual(x, ops.linear_gelu(xn, self.ffn[0]), self.ffn[2], e[5])
 
 
 class CausalHead(nn.Module):

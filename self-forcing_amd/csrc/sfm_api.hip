@@ -58,6 +58,8 @@ int launch_dense(const sfm_dense_desc& d, const void* q, const void* k, const vo
 int launch_prologue(const sfm_prologue_desc& d, const TokMap& map, const void* xq, const void* xk, const void* xv,
                     const void* wq, const void* wk, const double* rope, void* q_out, void* kc, void* vc,
                     hipStream_t stream);
+int launch_linear(const sfm_linear_desc& d, const void* x, const void* w, const void* bias, const void* res, const void* gate,
+                  void* out, hipStream_t stream);
 bool monarch_generic_supported(const MonarchArgs& a);
 bool monarch_iter_supported(const MonarchArgs& a);
 int launch_ln_modulate(int dtype, int64_t rows, int C, float eps, const void* x, int64_t xs, void* y, int64_t ys,
@@ -258,7 +260,7 @@ using namespace sfm;
 
 extern "C" {
 
-int sfm_version(void) { return 7; }
+int sfm_version(void) { return 8; }
 
 unsigned sfm_set_switches(unsigned mask) {
     if (mask & ~SFM_SW_ALL) {
@@ -1065,6 +1067,46 @@ int sfm_gate_residual(int32_t dtype, int64_t rows, int32_t C, void* x, int64_t x
     }
     return launch_gate_residual(dtype, rows, C, x, x_stride, y, y_stride, gate, mod_stride, gate ? rows_per_frame : 1,
                                 (hipStream_t)stream);
+}
+
+int sfm_linear(const sfm_linear_desc* d, const void* x, const void* w, const void* bias, const void* res, const void* gate,
+               void* out, void* stream) {
+    if (!d || !x || !w || !out) {
+        set_error("desc, x, w and out must be non-NULL");
+        return SFM_ERR_NULL;
+    }
+    if (d->dtype != SFM_BF16 && d->dtype != SFM_F16) {
+        set_error("sfm_linear takes 16-bit tensors (dtype %d)", d->dtype);
+        return SFM_ERR_DTYPE;
+    }
+    if (d->epilogue < SFM_EPI_NONE || d->epilogue > SFM_EPI_GATE_RESIDUAL) {
+        set_error("unknown epilogue %d", d->epilogue);
+        return SFM_ERR_SHAPE;
+    }
+    if (d->M < 1 || d->N < 8 || d->N % 8 || d->K < 64 || d->K % 64) {
+        set_error("M=%lld, N=%d, K=%d: need M >= 1, N a multiple of 8 and K a multiple of 64", (long long)d->M, d->N, d->K);
+        return SFM_ERR_SHAPE;
+    }
+    const bool gr = d->epilogue == SFM_EPI_GATE_RESIDUAL;
+    if (gr && !res) {
+        set_error("the gated-residual epilogue needs res");
+        return SFM_ERR_NULL;
+    }
+    if (d->x_stride < d->K || d->x_stride % 8 || d->out_stride < d->N || d->out_stride % 8 ||
+        (gr && (d->res_stride < d->N || d->res_stride % 8)) ||
+        (gr && gate && (d->rows_per_frame < 1 || d->gate_stride < 0 || d->gate_stride % 8))) {
+        set_error("row strides must cover a row and be multiples of 8 elements; rows_per_frame >= 1");
+        return SFM_ERR_STRIDE;
+    }
+    if ((uint64_t)d->M * (uint64_t)d->x_stride * 2 >= ((uint64_t)1 << 32) || (uint64_t)d->N * (uint64_t)d->K * 2 >= ((uint64_t)1 << 32)) {
+        set_error("x and w must span less than 4 GiB each");
+        return SFM_ERR_SHAPE;
+    }
+    if (!aligned16(x) || !aligned16(w) || !aligned16(bias) || !aligned16(res) || !aligned16(gate) || !aligned16(out)) {
+        set_error("tensors must be 16-byte aligned");
+        return SFM_ERR_ALIGN;
+    }
+    return launch_linear(*d, x, w, bias, gr ? res : nullptr, gr ? gate : nullptr, out, (hipStream_t)stream);
 }
 
 int sfm_rms_norm(int32_t dtype, int64_t rows, int32_t C, float eps, const void* x, int64_t x_stride, void* y,

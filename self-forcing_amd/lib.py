@@ -25,7 +25,7 @@ SYMBOLS = [
     "sfm_monarch_workspace_bytes", "sfm_monarch_fwd", "sfm_monarch_fwd_timed", "sfm_kv_cache_write", "sfm_monarch_attn_with_kv_cache",
     "sfm_monarch_attn_with_kv_cache_static",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
-    "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm",
+    "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_linear", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm",
     "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_dense_bwd_workspace_bytes", "sfm_dense_bwd", "sfm_probe_mfma_bf16", "sfm_probe_tile_traffic", "sfm_probe_row_stream", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_set_switches", "sfm_get_switches", "sfm_last_error", "sfm_version",
 ]
 
@@ -34,6 +34,15 @@ class ConvDesc(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("T", C.c_int32), ("H", C.c_int32), ("W", C.c_int32), ("Cin", C.c_int32),
                 ("Cout", C.c_int32), ("Cout_pad", C.c_int32), ("kt", C.c_int32), ("kh", C.c_int32), ("kw", C.c_int32),
                 ("up2x", C.c_int32), ("reserved", C.c_int32), ("x_stride", C.c_int64 * 3), ("y_stride", C.c_int64 * 3)]
+
+
+class LinearDesc(C.Structure):
+    _fields_ = [("dtype", C.c_int32), ("epilogue", C.c_int32), ("M", C.c_int64), ("N", C.c_int32), ("K", C.c_int32),
+                ("x_stride", C.c_int64), ("out_stride", C.c_int64), ("res_stride", C.c_int64), ("gate_stride", C.c_int64),
+                ("rows_per_frame", C.c_int32), ("reserved", C.c_int32)]
+
+
+EPI_NONE, EPI_GELU_TANH, EPI_GATE_RESIDUAL = 0, 1, 2
 
 
 class Tiling(C.Structure):
@@ -117,6 +126,7 @@ def load():
     lib.sfm_gate_residual.argtypes = [C.c_int32, I64, C.c_int32, P, I64, P, I64, P, I64, C.c_int32, P]
     lib.sfm_gate_residual_ln.argtypes = [C.c_int32, I64, C.c_int32, C.c_float, P, I64, P, I64, P, I64, C.c_int32, P, I64, P, P, I64,
                                          C.c_int32, P, P, P]
+    lib.sfm_linear.argtypes = [C.POINTER(LinearDesc), P, P, P, P, P, P, P]
     lib.sfm_rms_norm.argtypes = [C.c_int32, I64, C.c_int32, C.c_float, P, I64, P, I64, P, P]
     lib.sfm_conv3d_cl.argtypes = [C.POINTER(ConvDesc), P, P, P, P, P, P]
     lib.sfm_vae_norm_act.argtypes = [C.c_int32] * 6 + [P, S3, P, P, S3, P]

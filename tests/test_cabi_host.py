@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 9 and set(names) == set(L.SYMBOLS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sfm_version() == 7
+    assert lib.sfm_version() == 8
 
 
 def test_switches_are_a_process_wide_mask_set_through_the_abi():
