@@ -286,6 +286,53 @@ def op_level(torch, sfa, args):
     }
 
 
+def gemm_legs(torch, sfa):
+    """The block's four GEMM shapes at M = 4680 (1.3B and 14B widths), each with its element-wise tail: hipBLASLt
+    (TunableOp's pick) alone and followed by the separate tail kernel, against `linear.linear` with the tail in the
+    epilogue.  HIP-event means of 30 calls after 5 warm-up calls."""
+    dev, bf = "cuda:0", torch.bfloat16
+    sfa.pipeline.use_tuned_gemms()
+    shapes = [("qkv", 4680, 4608, 1536, "none"), ("o_proj", 4680, 1536, 1536, "gate_residual"),
+              ("ffn_up", 4680, 8960, 1536, "gelu_tanh"), ("ffn_down", 4680, 1536, 8960, "gate_residual"),
+              ("14b_qkv", 4680, 15360, 5120, "none"), ("14b_ffn_up", 4680, 13824, 5120, "gelu_tanh"),
+              ("14b_ffn_down", 4680, 5120, 13824, "gate_residual")]
+
+    def timeit(f, n=30):
+        for _ in range(5):
+            f()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            f()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / n
+
+    out = {}
+    g = torch.Generator().manual_seed(0)
+    with torch.no_grad():
+        for name, M, N, K, epi in shapes:
+            x = torch.randn(1, M, K, generator=g).to(bf).to(dev)
+            lin = torch.nn.Linear(K, N, device=dev, dtype=bf)
+            w, b = lin.weight.detach(), lin.bias.detach()
+            res = torch.randn(1, M, N, generator=g).to(bf).to(dev)
+            gate = torch.randn(1, 3, 1, N, generator=g).to(bf).to(dev)
+            rec = {"M": M, "N": N, "K": K, "epilogue": epi, "library_gemm_us": timeit(lambda: lin(x))}
+            if epi == "gelu_tanh":
+                rec["library_plus_tail_us"] = timeit(lambda: torch.nn.functional.gelu(lin(x), approximate="tanh"))
+                rec["library_fused_gelu_us"] = timeit(lambda: torch._addmm_activation(b, x[0], w.t(), use_gelu=True))
+                rec["own_us"] = timeit(lambda: sfa.linear.linear(x, w, b, epilogue="gelu_tanh"))
+            elif epi == "gate_residual":
+                rec["library_plus_tail_us"] = timeit(lambda: sfa.block_ops.gate_residual_(res, lin(x), gate))
+                rec["own_us"] = timeit(lambda: sfa.linear.linear(x, w, b, epilogue="gate_residual", res=res, gate=gate))
+            else:
+                rec["own_us"] = timeit(lambda: sfa.linear.linear(x, w, b))
+            rec["own_tflops"] = 2.0 * M * N * K / rec["own_us"] / 1e6
+            out[name] = rec
+    return out
+
+
 def vae_decode_leg(torch, sfa):
     """Streaming decode of one video's latents (outside the headline metric, which excludes the VAE): random-init
     decoder of the Wan 2.1 VAE shape, bf16, 21 latent frames in 7 chunks of 3 -> 81 frames of 480x832."""
@@ -330,6 +377,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="accepted for the profile commands; the 1 GiB device copies (known HBM traffic, for scaling rocprof "
                          "counters) always run")
+    ap.add_argument("--gemm-legs", action="store_true",
+                    help="only the table of the block's GEMM shapes: hipBLASLt (+ tail kernel) against sfm_linear with the tail fused")
     ap.add_argument("--write-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
                     help="no GPU work: rewrite profiles/traffic.json from two rocprofv3 counter_collection CSVs")
     args = ap.parse_args()
@@ -344,6 +393,9 @@ def main():
     import self_forcing_amd as sfa
 
     torch.cuda.set_device(0)
+    if args.gemm_legs:
+        print(json.dumps({"metric": "block GEMM shapes, us per call", "gemm": gemm_legs(torch, sfa)}))
+        return
     entry, size, flags, what = ROLLOUTS[args.config]
     rec = {"metric": f"latent frames/s, causal Wan-{size} 480x832 bf16 (+ Monarch attn ms/call, MFMA %)",
            "unit": "latent frames/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
