@@ -195,6 +195,31 @@ def op_level(torch, sfa, args):
     torch.cuda.synchronize()
     dense_ms = (time.perf_counter() - t0) * 1e3 / 5
 
+    # iterated refinement (num_iters = 8, the reference's "slow" quality setting) at the same shape: on the MFMA kernels
+    # and, once, on the fp32 SIMT kernels the same call runs on where the MFMA kernels do not apply
+    def iter_call():
+        return sfa.monarch_attn.monarch_attn(q, kc, vc, 1, 1, 1, B1, B2, kv_block_order=True, num_iters=8)
+
+    iter_call()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        iter_call()
+    torch.cuda.synchronize()
+    iter_ms = (time.perf_counter() - t0) * 1e3 / 5
+    iter_simt_ms = None
+    if not args.skip_simt:
+        old_sw = lib.sfm_set_switches(L.SW_ITER_SIMT)
+        try:
+            iter_call()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            iter_call()
+            torch.cuda.synchronize()
+            iter_simt_ms = (time.perf_counter() - t0) * 1e3
+        finally:
+            lib.sfm_set_switches(old_sw)
+
     # backward of the same op: with the output and row statistics the forward keeps under autograd, and recomputing
     # them; three timed calls after one warm-up each
     from self_forcing_amd.monarch_attn import _monarch_bwd, _monarch_fwd_stats
@@ -266,6 +291,9 @@ def op_level(torch, sfa, args):
                                      "(4680 q x 32760 kv), new chunk written at tokens 28080..32760",
                          "ms_per_call": ms_call, "tflops": tfl, "mfma_frac": tfl / MFMA_BF16_PEAK_TFLOPS,
                          "kernel_ms": {"monarch_step1": s1_ms, "monarch_step2": s2_ms}},
+        "monarch_iter": {"workload": "monarch_attn, num_iters = 8 (monarch_attn_slow), same shape and cache",
+                         "ms_per_call": iter_ms, "ms_per_call_fp32_simt_kernels": iter_simt_ms,
+                         "tflops": 8 * MONARCH_FLOPS / (iter_ms * 1e-3) / 1e12},
         "monarch_bwd": {"workload": "gradients of q and of all 21 cached K/V frames at the same shape",
                         "ms_per_call": bwd_ms, "ms_per_call_recomputing_statistics": bwd["recompute"]},
         "dense_fallback": {"ms_per_call": dense_ms, "tflops": dense_tfl, "mfma_frac": dense_tfl / MFMA_BF16_PEAK_TFLOPS,
@@ -374,6 +402,7 @@ def main():
     ap.add_argument("--one-kernel", action="store_true",
                     help="op-level figures of the opt-in one-kernel Monarch forward (Kbar / Y kept in LDS) instead of the default "
                          "two kernels; kernel_ms then holds the fused kernel and its merge kernel")
+    ap.add_argument("--skip-simt", action="store_true", help="leave out the 0.7 s of fp32 SIMT refinement calls (profile runs)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="accepted for the profile commands; the 1 GiB device copies (known HBM traffic, for scaling rocprof "
                          "counters) always run")

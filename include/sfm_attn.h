@@ -344,7 +344,8 @@ int sfm_probe_row_stream(int32_t waves, int32_t kb_per_block, const void* worksp
 #define SFM_SW_BWD_DQA_GEMM    0x08u
 #define SFM_SW_BWD_RIGHT_GEMM  0x10u
 #define SFM_SW_BWD_DQK_GEMM    0x20u
-#define SFM_SW_ALL             0x3fu
+#define SFM_SW_ITER_SIMT       0x40u  /* num_iters > 1 on the fp32 SIMT kernels also where the MFMA kernels apply */
+#define SFM_SW_ALL             0x7fu
 unsigned sfm_set_switches(unsigned mask);
 unsigned sfm_get_switches(void);
 

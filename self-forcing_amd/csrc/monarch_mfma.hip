@@ -56,7 +56,10 @@ struct S1Lds {
 
 // NT: 32-row tiles of the key axis l (2 when b2 > 32).
 // WR: also write the right factor R (16 bit, 64 values per scratch row) to p.rb; the backward uses it.
-template <class E, int D, int NT, bool WR = false>
+// IT: a pass of the iterated refinement (wan/modules/monarch_attn.py:1716-1722): the logits are scaled per (a, f, k, j)
+//     column and, after the first pass, the query operand of tile (f, k) is the column's representative p.rep[a, j, (f, k)]
+//     instead of Q[a, k, j]; the operand is then fetched for every tile.
+template <class E, int D, int NT, bool WR = false, bool IT = false>
 __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) void monarch_step1_kernel(MonarchArgs p) {
     using L = S1Lds<D>;
     constexpr int CPR = D / 8;   // 16-byte chunks of a K/V row
@@ -163,6 +166,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     uint32_t crow[4] = {0, 0, 0, 0};                       // byte offsets in the (f, k) slab of the four scratch rows this lane stores to
     uint32_t cloff = 0;                                    // same for cl
     int qkey = -1;
+    float wsc = 1.f;                                       // IT: the column's logits factor
 
     Tile cur = decode(t0 + grp), nxt = cur;
     stage(cur, 0);
@@ -178,7 +182,8 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         const char* kt = lds + (r & 1) * 2 * L::kTile;
         const char* vt = kt + L::kTile;
         const int key = (cur.ul * p.b1 + cur.k) * p.n_achunks + cur.ac;       // one value per (unit, k, query chunk)
-        if (key != qkey) {
+        const uint32_t srow = (uint32_t)cur.ul * p.ws_unit + (uint32_t)cur.k * p.ws_row + (uint32_t)cur.f * fstep;
+        if ((IT && p.iter_mode == 2) || key != qkey) {
             qkey = key;
             const int unit = p.unit0 + cur.ul;
             const int b = unit / p.H, h = unit % p.H;
@@ -188,6 +193,14 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             const int cj = cg - cl_a * b2;
             const int ca = cur.a0 + cl_a;
             const uint16_t* qrow = qg + ((uint32_t)(p.qmap.row(ca, cur.k) + cj) * qs1 + 8 * hf);
+            if (IT) {
+                wsc = 1.0f / (1.0f + 1e-6f);
+                if (p.iter_mode == 2) {
+                    const size_t rrow = (size_t)srow + (size_t)(ca * b2 + cj) * p.ws_aj;
+                    qrow = (const uint16_t*)p.rep + rrow * D + 8 * hf;
+                    wsc = fminf(1.0f / (p.wgt[rrow] + 1e-6f), 1e4f);
+                }
+            }
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
 #pragma unroll
@@ -207,8 +220,6 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             stage(nxt, (r + 1) & 1);
         }
 
-        const uint32_t srow = (uint32_t)cur.ul * p.ws_unit + (uint32_t)cur.k * p.ws_row + (uint32_t)cur.f * fstep;
-
         u32x4 pb[2 * NT];                // R^T as B operands, 16 contraction rows per step
         {
             f32x16 s[NT];
@@ -226,7 +237,7 @@ __global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     int l = 32 * t + 8 * (v >> 2) + 4 * hf + (v & 3);
-                    float zz = l < b2 ? s[t][v] * sc2 : kMaskLogit;
+                    float zz = l < b2 ? (IT ? s[t][v] * sc2 * wsc : s[t][v] * sc2) : kMaskLogit;
                     s[t][v] = zz;
                     mx = fmaxf(mx, zz);
                 }
@@ -534,6 +545,178 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
 }
 
 // ------------------------------------------------------------------------------------------------
+// iterated refinement: the next pass's query representatives (wan/modules/monarch_attn.py:1741-1744)
+//   rep[a, j, r, :] = sum_i L[i, r] Q[a, i, j, :],   wgt[a, j, r] = sum_i L[i, r],   r = (f, k)
+// with L[i, r] = exp2(s log2e <Q_i, Kbar_r> - cl_r - stats_i), stats = the left factor's row statistics that step 2 wrote.
+// Step 2 with the operands' roles exchanged: one wave per (a, j) streams the column's Kbar rows 32 at a time through its
+// LDS; the logits come out as S[i, r] (A = the lane's query row, in registers; B = Kbar rows), so that a lane holds a
+// column r, and rep^T[d, r] = sum_i Q^T[d, i] L[i, r] takes Q^T from transposing reads of the column's query rows, which
+// sit in the (otherwise unused) Y slot of the wave's first buffer.  b1 <= 32.
+// ------------------------------------------------------------------------------------------------
+template <class E, int D>
+__global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
+    using L = S2Lds<D>;
+    constexpr int DS = D / 16, DT = D / 32, CPR = D / 8;
+    extern __shared__ __attribute__((aligned(256))) char lds_s2[];
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int m = lane & 31;
+    const int hf = lane >> 5;
+
+    const int b2 = p.b2;
+    const int njg = (b2 + 3) / 4;
+    const int a = blockIdx.x / njg;
+    const int jraw = (blockIdx.x % njg) * 4 + wave;
+    if (jraw >= b2) return;                               // the waves of a workgroup share nothing
+    const int j = jraw;
+    const int ul = blockIdx.y;
+    const int unit = p.unit0 + ul;
+    const int b = unit / p.H, h = unit % p.H;
+
+    const int r_lim = p.nf * p.b1;
+    const int nch = (r_lim + 31) / 32;
+    const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj;
+    const char* kb = (const char*)p.kbar + blk * (2 * D);
+    const char* clp = (const char*)(p.cl + blk);
+    char* repb = (char*)p.rep + blk * (2 * D);
+    float* wgt = p.wgt + blk;
+
+    char* const wl = lds_s2 + wave * L::kWave;
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)wl;
+    char* const qt = wl + L::kTile;                       // the column's query rows, laid out like a chunk of scratch rows
+
+    const uint16_t* qg = (const uint16_t*)p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[2];
+    // query rows into LDS (rows past b1 repeat the last one; their weights are zero)
+#pragma unroll
+    for (int g = 0; g < CPR / 2; ++g) {
+        const int P = g * 64 + lane;
+        const int r = P / CPR, c = (P % CPR) ^ s1_swz<CPR>(r);
+        const uint32_t off = (uint32_t)((p.qmap.row(a, min(r, p.b1 - 1)) + j) * p.qs[1] * 2) + (uint32_t)c * 16;
+        s1_load_lds16((const char*)qg, off, lds0 + L::kTile + (uint32_t)g * 1024);
+    }
+    // logits operand (A): this lane's query row Q[a, m, j, :] (zero past b1), and the statistics of the 16 rows whose
+    // logits this lane will hold
+    u32x4 qa[DS];
+    {
+        const uint16_t* qrow = qg + (p.qmap.row(a, min(m, p.b1 - 1)) + j) * p.qs[1] + 8 * hf;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) qa[ds] = *(const u32x4*)(qrow + 16 * ds);
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) asm volatile("" : "+v"(qa[ds]));
+        if (m >= p.b1) {
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds) qa[ds] = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+    float st[16];
+    {
+        const float* sp = p.stats + ((int64_t)unit * (p.na * b2) + a * b2 + j) * p.stats_ld;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
+            st[v] = i < p.b1 ? sp[i] : 0.f;
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) asm volatile("" : "+v"(st[v]));
+    }
+
+    // chunk n of the Kbar rows (and their cl values) into buffer `buf`
+    auto issue = [&](int n, int buf) {
+        const uint32_t dst = lds0 + (uint32_t)buf * L::kBuf;
+#pragma unroll
+        for (int g = 0; g < CPR / 2; ++g) {
+            const int P = g * 64 + lane;
+            const int r = P / CPR, c = (P % CPR) ^ s1_swz<CPR>(r);
+            const uint32_t off = (uint32_t)min(32 * n + r, r_lim - 1) * (2 * D) + (uint32_t)c * 16;
+            s1_load_lds16(kb, off, dst + (uint32_t)g * 1024);
+        }
+        s2_load_lds4(clp, (uint32_t)(32 * n + m) * 4, dst + 2 * L::kTile);
+    };
+    const uint32_t b_off = (uint32_t)m * L::kPitch + (uint32_t)((hf ^ s1_swz<CPR>(m)) << 4);   // Kbar row m as the logits' B operand
+    uint32_t tr[DT][2];            // Q^T as the representatives' A operand: transposing reads, as step 2 reads Y^T
+    {
+        const int s16 = lane & 15, g16 = lane >> 4;
+        const int rl = 4 * hf + (s16 >> 2);
+        const int cl = 2 * (g16 & 1) + ((s16 & 3) >> 1);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int r = rl + 8 * half;
+                tr[dt][half] = (uint32_t)(r * L::kPitch + (((4 * dt + cl) ^ s1_swz<CPR>(r)) << 4) + (s16 & 1) * 8);
+            }
+    }
+
+    const float sc2 = p.scale * kLog2e;
+    const f32x16 kZero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    issue(0, 0);
+    for (int n = 0; n < nch; ++n) {
+        // everything older than the chunk requested last (the stores of the chunk before included) is waited for
+        if (n + 1 < nch) {
+            issue(n + 1, (n + 1) & 1);
+            if (D == 128) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        const char* kt = wl + (n & 1) * L::kBuf;
+
+        f32x16 s;                  // S[i = 8 g + 4 hf + e, r = 32 n + m]
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            const u32x4 bk = *(const u32x4*)(kt + (b_off ^ (uint32_t)(ds << 5)));
+            s = E::mfma32(qa[ds], bk, ds ? s : kZero);
+        }
+        const float cc = *(const float*)(kt + 2 * L::kTile + m * 4);
+        const bool rok = 32 * n + m < r_lim;
+        float wsum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
+            const float e = (rok && i < p.b1) ? exp2f(s[v] * sc2 - cc - st[v]) : 0.f;
+            s[v] = e;
+            wsum += e;
+        }
+        wsum = xhalf_sum(wsum);
+        if (hf == 0) wgt[32 * n + m] = wsum;
+        u32x4 pb[2];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            pb[q].x = pack2<E>(s[8 * q + 0], s[8 * q + 1]);
+            pb[q].y = pack2<E>(s[8 * q + 2], s[8 * q + 3]);
+            pb[q].z = pack2<E>(s[8 * q + 4], s[8 * q + 5]);
+            pb[q].w = pack2<E>(s[8 * q + 6], s[8 * q + 7]);
+        }
+        char* rrow = repb + (size_t)(32 * n + m) * (2 * D);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            f32x16 acc;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const u32x2 lo = s1_read_tr(qt, tr[dt][0] + q * 16 * L::kPitch);
+                const u32x2 hi = s1_read_tr(qt, tr[dt][1] + q * 16 * L::kPitch);
+                const u32x4 aq = {lo.x, lo.y, hi.x, hi.y};
+                acc = E::mfma32(aq, pb[q], q ? acc : kZero);
+            }
+            // rep^T[d = 32 dt + 8 g + 4 hf + e, r]: the half-swap leaves 8 consecutive d per lane
+#pragma unroll
+            for (int gp = 0; gp < 2; ++gp) {
+                const int g0 = 2 * gp, g1 = 2 * gp + 1;
+                auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 0], acc[4 * g0 + 1]),
+                                                           pack2<E>(acc[4 * g1 + 0], acc[4 * g1 + 1]), false, false);
+                auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[4 * g0 + 2], acc[4 * g0 + 3]),
+                                                           pack2<E>(acc[4 * g1 + 2], acc[4 * g1 + 3]), false, false);
+                const u32x4 o = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+                *(u32x4*)(rrow + (32 * dt + 16 * gp + 8 * hf) * 2) = o;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // host launch
 // ------------------------------------------------------------------------------------------------
 bool monarch_mfma_supported(int dtype, int D, int b2) {
@@ -555,7 +738,7 @@ int cu_count() {
 
 // Enqueues step 1 (with the right factor written too when a.rb is set).
 template <class E, int D>
-static int enqueue_step1(const MonarchArgs& a, int nunits, hipStream_t stream) {
+static int enqueue_step1(const MonarchArgs& a, int nunits, hipStream_t stream, const void* fn_override = nullptr) {
     const int ncols = a.a_chunk * a.b2;
     const int ntiles = (ncols + 31) / 32;
     const int nwaves = ntiles < 4 ? 4 : ntiles;   // a wave per 32 (a, j) columns, at least 4 to share the tile loads
@@ -565,8 +748,9 @@ static int enqueue_step1(const MonarchArgs& a, int nunits, hipStream_t stream) {
     }
     const int groups = nwaves <= 5 ? 2 : 1;             // wave groups per workgroup (<= 10 waves in all)
     const size_t lds1 = S1Lds<D>::bytes() * groups;
-    const void* fn = a.b2 > 32 ? (a.rb ? (const void*)monarch_step1_kernel<E, D, 2, true> : (const void*)monarch_step1_kernel<E, D, 2, false>)
-                               : (a.rb ? (const void*)monarch_step1_kernel<E, D, 1, true> : (const void*)monarch_step1_kernel<E, D, 1, false>);
+    const void* fn = fn_override ? fn_override
+                     : a.b2 > 32 ? (a.rb ? (const void*)monarch_step1_kernel<E, D, 2, true> : (const void*)monarch_step1_kernel<E, D, 2, false>)
+                                 : (a.rb ? (const void*)monarch_step1_kernel<E, D, 1, true> : (const void*)monarch_step1_kernel<E, D, 1, false>);
     if (lds1 > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1);
         if (e != hipSuccess) {
@@ -625,6 +809,53 @@ int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_
     if (dtype == SFM_BF16)
         return a.D == 128 ? launch_step1_t<BF16, 128>(a, nunits, stream) : launch_step1_t<BF16, 64>(a, nunits, stream);
     return a.D == 128 ? launch_step1_t<F16, 128>(a, nunits, stream) : launch_step1_t<F16, 64>(a, nunits, stream);
+}
+
+bool monarch_iter_mfma_supported(int dtype, int D, int b1, int b2) {
+    return monarch_mfma_supported(dtype, D, b2) && b1 >= 1 && b1 <= 32;
+}
+
+// num_iters passes of [step 1 with the pass's query operands | step 2 | representatives for the next pass]; the last
+// pass's step 2 writes the output (the earlier ones write it too: it is overwritten).
+template <class E, int D>
+static int launch_iter_t(const MonarchArgs& a, int nunits, int num_iters, hipStream_t stream) {
+    const int njg = (a.b2 + 3) / 4;
+    const dim3 g2(a.na * njg, nunits, 1);
+    const void* fn1 = a.b2 > 32 ? (const void*)monarch_step1_kernel<E, D, 2, false, true> : (const void*)monarch_step1_kernel<E, D, 1, false, true>;
+    hipError_t e = hipFuncSetAttribute((const void*)monarch_step2_kernel<E, D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)S2Lds<D>::bytes());
+    if (e == hipSuccess)
+        e = hipFuncSetAttribute((const void*)monarch_rep_kernel<E, D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)S2Lds<D>::bytes());
+    if (e != hipSuccess) {
+        set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    for (int it = 0; it < num_iters; ++it) {
+        const bool last = it + 1 == num_iters;
+        MonarchArgs a1 = a;
+        a1.rb = nullptr;
+        a1.iter_mode = it == 0 ? 1 : 2;
+        if (int rc = enqueue_step1<E, D>(a1, nunits, stream, fn1)) return rc;
+        MonarchArgs a2 = a;
+        if (last) a2.stats = nullptr;
+        hipLaunchKernelGGL((monarch_step2_kernel<E, D>), g2, dim3(256), S2Lds<D>::bytes(), stream, a2);
+        if (!last) hipLaunchKernelGGL((monarch_rep_kernel<E, D>), dim3(g2.x, g2.y), dim3(256), S2Lds<D>::bytes(), stream, a);
+    }
+    e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("hip launch failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
+}
+
+int launch_monarch_iter_mfma(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream) {
+    if (!monarch_iter_mfma_supported(dtype, a.D, a.b1, a.b2) || a.causal || !a.rep || !a.wgt || !a.stats || a.stats_ld < 32) {
+        set_error("internal: iterated MFMA launch");
+        return SFM_ERR_UNSUPPORTED;
+    }
+    if (dtype == SFM_BF16)
+        return a.D == 128 ? launch_iter_t<BF16, 128>(a, nunits, num_iters, stream) : launch_iter_t<BF16, 64>(a, nunits, num_iters, stream);
+    return a.D == 128 ? launch_iter_t<F16, 128>(a, nunits, num_iters, stream) : launch_iter_t<F16, 64>(a, nunits, num_iters, stream);
 }
 
 int launch_monarch_mfma(const MonarchArgs& a, int dtype, int nunits, hipStream_t stream, const StepEvents* ev) {

@@ -22,7 +22,8 @@ struct Switches {
         static const struct { const char* name; unsigned bit; } names[] = {
             {"SFM_BWD_SIMT", SFM_SW_BWD_SIMT},           {"SFM_BWD_LEFT_GEMM", SFM_SW_BWD_LEFT_GEMM},
             {"SFM_BWD_FWD_GEMM", SFM_SW_BWD_FWD_GEMM},   {"SFM_BWD_DQA_GEMM", SFM_SW_BWD_DQA_GEMM},
-            {"SFM_BWD_RIGHT_GEMM", SFM_SW_BWD_RIGHT_GEMM}, {"SFM_BWD_DQK_GEMM", SFM_SW_BWD_DQK_GEMM}};
+            {"SFM_BWD_RIGHT_GEMM", SFM_SW_BWD_RIGHT_GEMM}, {"SFM_BWD_DQK_GEMM", SFM_SW_BWD_DQK_GEMM},
+            {"SFM_ITER_SIMT", SFM_SW_ITER_SIMT}};
         unsigned m = 0;
         for (const auto& n : names) {
             const char* e = getenv(n.name);
@@ -144,6 +145,7 @@ static int check_strides(const char* name, const int64_t s[3], int64_t tokens, i
 struct MonarchPlan {
     int na, nf, b1, b2, r_pad, units;
     bool mfma, iter;
+    bool iter_mfma;    // num_iters > 1 on the MFMA kernels (16-bit scratch + the left factor's row statistics)
     bool fused;        // the one-kernel forward (monarch_fused.hip) runs: its scratch is sized per pass, not per unit
     size_t per_unit;   // workspace bytes of a pass over one (batch x head) unit: the least a call needs
 };
@@ -219,12 +221,14 @@ static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
     }
     pl->iter = d->num_iters > 1;
     pl->mfma = !pl->iter && monarch_mfma_supported(d->dtype, d->D, pl->b2);
+    pl->iter_mfma = pl->iter && monarch_iter_mfma_supported(d->dtype, d->D, pl->b1, pl->b2) && !(switches() & SFM_SW_ITER_SIMT);
     const size_t rows = (size_t)pl->na * pl->b2 * pl->r_pad;
-    pl->per_unit = rows * d->D * (pl->mfma ? 2 : 4) * (pl->iter ? 3 : 2) + rows * sizeof(float) * (pl->iter ? 2 : 1);
+    pl->per_unit = rows * d->D * (pl->mfma || pl->iter_mfma ? 2 : 4) * (pl->iter ? 3 : 2) + rows * sizeof(float) * (pl->iter ? 2 : 1) +
+                   (pl->iter_mfma ? (size_t)pl->na * pl->b2 * 32 * sizeof(float) : 0);
     pl->per_unit = (pl->per_unit + 255) / 256 * 256;
     // the fp32 kernels' own limits, checked here so that no entry point has written anything (the KV-cache entry points
     // write the cache before the forward is launched) when they are exceeded
-    if (!pl->mfma) {
+    if (!pl->mfma && !pl->iter_mfma) {
         MonarchArgs lim;
         memset(&lim, 0, sizeof(lim));
         lim.D = d->D; lim.na = pl->na; lim.nf = pl->nf; lim.b1 = pl->b1; lim.b2 = pl->b2;
@@ -260,7 +264,7 @@ using namespace sfm;
 
 extern "C" {
 
-int sfm_version(void) { return 8; }
+int sfm_version(void) { return 9; }
 
 unsigned sfm_set_switches(unsigned mask) {
     if (mask & ~SFM_SW_ALL) {
@@ -387,7 +391,7 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
     }
     const int upp = upp_sz > (size_t)pl.units ? pl.units : (int)upp_sz;
     const size_t rows = (size_t)pl.na * pl.b2 * pl.r_pad;
-    const size_t mat_bytes = rows * desc->D * (pl.mfma ? 2 : 4);
+    const size_t mat_bytes = rows * desc->D * (pl.mfma || pl.iter_mfma ? 2 : 4);
     for (int u0 = 0; u0 < pl.units; u0 += upp) {
         const int n = pl.units - u0 < upp ? pl.units - u0 : upp;
         a.unit0 = u0;
@@ -402,7 +406,13 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
                 set_error("the timed variant covers num_iters == 1 only");
                 return SFM_ERR_UNSUPPORTED;
             }
-            rc = launch_monarch_iter(a, desc->dtype, n, desc->num_iters, (hipStream_t)stream);
+            if (pl.iter_mfma) {
+                a.stats = (float*)((char*)a.wgt + rows * sizeof(float) * upp);
+                a.stats_ld = 32;
+                rc = launch_monarch_iter_mfma(a, desc->dtype, n, desc->num_iters, (hipStream_t)stream);
+            } else {
+                rc = launch_monarch_iter(a, desc->dtype, n, desc->num_iters, (hipStream_t)stream);
+            }
             if (rc) return rc;
             continue;
         }

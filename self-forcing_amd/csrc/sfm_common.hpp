@@ -133,8 +133,10 @@ struct MonarchArgs {
     void* kbar;      // [units_per_pass][na][b2][r_pad][D]   16-bit (MFMA path) or float (generic path)
     void* y;         // same shape
     float* cl;       // [units_per_pass][na][b2][r_pad]      sum_l R log2 R  (log2 units)
-    void* rep;       // iterated refinement only: query representatives, float, same shape as kbar
+    void* rep;       // iterated refinement only: query representatives, same shape and element type as kbar
     float* wgt;      // iterated refinement only: their weights, same shape as cl
+    int iter_mode;   // MFMA step 1: 0 = queries from q; 1 = first refinement pass (q, logits / (1 + 1e-6));
+                     // 2 = later pass (queries from rep, logits * min(1 / (wgt + 1e-6), 1e4))
     int B, H, D, na, nf, b1, b2;
     int r_pad;       // rows per (a, j) block of the workspace: round_up(nf*b1, 32)
     // scratch row index of (unit ul, a, j, r) = ul*ws_unit + (a*b2 + j)*ws_aj + r*ws_row
@@ -187,6 +189,10 @@ bool monarch_fused_supported(int dtype, int D, int b1, int b2, int causal);
 size_t monarch_fused_bytes(int na, int nf, int b1, int b2, int nunits);
 int launch_monarch_fused(const MonarchArgs& a, int dtype, int nunits, void* ws, hipStream_t stream, const StepEvents* ev);
 int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
+// the refinement on the MFMA kernels (16-bit, head_dim 64 / 128, b1 <= 32, b2 <= 64): a.rep in the tensor dtype, a.stats
+// [units][na * b2][a.stats_ld] scratch for the left factor's row statistics
+bool monarch_iter_mfma_supported(int dtype, int D, int b1, int b2);
+int launch_monarch_iter_mfma(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
 int launch_monarch_bwd(const MonarchBwdArgs& g, int dtype, int nunits, hipStream_t stream);
 bool monarch_bwd_gemm_available();
 // process-wide implementation switches (SFM_SW_* of the header), read from the environment once at load

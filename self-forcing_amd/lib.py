@@ -13,7 +13,7 @@ SFM_BF16, SFM_F16, SFM_F32 = 0, 1, 2
 SFM_MONARCH_ONE_KERNEL = 1
 STATIC_SCRATCH_BYTES = 128 << 20      # SFM_STATIC_SCRATCH_BYTES of include/sfm_attn.h
 # SFM_SW_* of include/sfm_attn.h: process-wide implementation switches (sfm_set_switches)
-SW_BWD_SIMT, SW_BWD_LEFT_GEMM, SW_BWD_FWD_GEMM, SW_BWD_DQA_GEMM, SW_BWD_RIGHT_GEMM, SW_BWD_DQK_GEMM = (1 << i for i in range(6))
+SW_BWD_SIMT, SW_BWD_LEFT_GEMM, SW_BWD_FWD_GEMM, SW_BWD_DQA_GEMM, SW_BWD_RIGHT_GEMM, SW_BWD_DQK_GEMM, SW_ITER_SIMT = (1 << i for i in range(7))
 
 ERR_NAMES = {
     -1: "SFM_ERR_NULL", -2: "SFM_ERR_DTYPE", -3: "SFM_ERR_SHAPE", -4: "SFM_ERR_RANGE", -5: "SFM_ERR_STRIDE",

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     assert len(names) >= 9 and set(names) == set(L.SYMBOLS)
     for n in names:
         assert hasattr(lib, n), n
-    assert lib.sfm_version() == 8
+    assert lib.sfm_version() == 9
 
 
 def test_switches_are_a_process_wide_mask_set_through_the_abi():
@@ -31,14 +31,14 @@ def test_switches_are_a_process_wide_mask_set_through_the_abi():
     are refused and leave the mask alone, and the workspace query of the backward follows the mask."""
     lib = L.load()
     text = open(os.path.join(ROOT, "include", "sfm_attn.h")).read()
-    for i, name in enumerate(("BWD_SIMT", "BWD_LEFT_GEMM", "BWD_FWD_GEMM", "BWD_DQA_GEMM", "BWD_RIGHT_GEMM", "BWD_DQK_GEMM")):
+    for i, name in enumerate(("BWD_SIMT", "BWD_LEFT_GEMM", "BWD_FWD_GEMM", "BWD_DQA_GEMM", "BWD_RIGHT_GEMM", "BWD_DQK_GEMM", "ITER_SIMT")):
         assert re.search(rf"#define\s+SFM_SW_{name}\s+0x{1 << i:02x}u", text), name
         assert getattr(L, "SW_" + name) == 1 << i
     old = lib.sfm_get_switches()
     try:
         assert lib.sfm_set_switches(L.SW_BWD_SIMT) == old
         assert lib.sfm_get_switches() == L.SW_BWD_SIMT and lib.sfm_monarch_bwd_uses_gemm() == 0
-        assert lib.sfm_set_switches(0x40) == 0xFFFFFFFF and b"unknown switch" in lib.sfm_last_error()
+        assert lib.sfm_set_switches(0x80) == 0xFFFFFFFF and b"unknown switch" in lib.sfm_last_error()
         assert lib.sfm_get_switches() == L.SW_BWD_SIMT
     finally:
         lib.sfm_set_switches(old)
@@ -127,9 +127,22 @@ def test_workspace_bytes_accounting():
     # fp32 tensors take the generic path, which keeps its scratch rows in float
     rc, nf32 = _ws(_desc(dtype=L.SFM_F32), 1)
     assert rc == 0 and nf32 == rows * 128 * 4 * 2 + rows * 4
-    # iterated refinement: fp32 Kbar, Y and representatives plus two fp32 scalars per row
+    # iterated refinement on the MFMA kernels: 16-bit Kbar, Y and representatives, two fp32 scalars per row, and the left
+    # factor's statistics (32 floats per (a, j) column); on the fp32 kernels (switch, or shapes the MFMA kernels do not
+    # take: b1 = 90 here) everything in float and no statistics
     rc, nit = _ws(_desc(num_iters=3), 1)
-    assert rc == 0 and nit == rows * 128 * 4 * 3 + rows * 4 * 2
+    assert rc == 0 and nit == rows * 128 * 2 * 3 + rows * 4 * 2 + 3 * 52 * 32 * 4
+    lib = L.load()
+    old = lib.sfm_get_switches()
+    try:
+        lib.sfm_set_switches(L.SW_ITER_SIMT)
+        rc, nsimt = _ws(_desc(num_iters=3), 1)
+    finally:
+        lib.sfm_set_switches(old)
+    assert rc == 0 and nsimt == rows * 128 * 4 * 3 + rows * 4 * 2
+    rows3 = 1 * 52 * ((7 * 90 + 31) // 32 * 32)
+    rc, ntied = _ws(_desc(num_iters=3, tiling=L.Tiling(3, 1, 1, 30, 52)), 1)
+    assert rc == 0 and ntied == (rows3 * 128 * 4 * 3 + rows3 * 4 * 2 + 255) // 256 * 256
 
 
 @pytest.mark.parametrize("kw,code", [

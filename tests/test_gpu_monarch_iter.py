@@ -92,3 +92,46 @@ def test_c2_shape_two_iterations_bf16(f_tied):
     vc = torch.full_like(v, 0.75)
     outc = mattn.monarch_attn(q.to(DEV), k.to(DEV), vc.to(DEV), f_tied, 1, 1, b1, b2, num_iters=2)
     assert max_abs(outc, torch.full_like(q, 0.75)) < 4e-3
+
+
+@pytest.fixture
+def switches():
+    lib = sfa.lib.load()
+    old = lib.sfm_get_switches()
+    yield lib.sfm_set_switches
+    lib.sfm_set_switches(old)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("h,w,D,frames,n", [(6, 20, 128, (1, 3), 2), (8, 40, 64, (2, 3), 3), (30, 52, 128, (1, 2), 3),
+                                             (5, 33, 64, (2, 2), 8), (32, 64, 128, (1, 2), 2), (4, 8, 128, (3, 5), 8)])
+def test_mfma_refinement_against_the_oracle_and_the_fp32_kernels(dtype, h, w, D, frames, n, switches):
+    """16-bit tensors with b1 <= 32, b2 <= 64 run the refinement on the MFMA kernels (representatives kept in the
+    tensor dtype); the same call with SFM_SW_ITER_SIMT runs the fp32 kernels.  Both against the fp32 oracle at the
+    reference's 16-bit bar, and against each other."""
+    H = 2
+    fq, fk = frames
+    q = randn((1, fq * h * w, H, D), 300, dtype)
+    k, v = (randn((1, fk * h * w, H, D), 301 + i, dtype) for i in range(2))
+    ref = monarch.monarch_attn(q, k, v, 1, 1, 1, h, w, num_iters=n, dtype=torch.float32)
+    switches(0)
+    fast = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, h, w, num_iters=n)
+    switches(sfa.lib.SW_ITER_SIMT)
+    slow = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, h, w, num_iters=n)
+    assert_close_16bit(slow, ref, dtype)
+    assert_close_16bit(fast, ref, dtype)
+    assert_close_16bit(fast, slow.float(), dtype)
+
+
+def test_mfma_refinement_golden_vectors_in_bf16():
+    """The reference's own refinement outputs (float64 golden vectors), inputs rounded to bf16: D = 64 case of the
+    fixture, num_iters 2, 3 and 8, on the MFMA kernels."""
+    q, k, v, s, (B, a, f, b1, b2, H, D) = _golden_inputs(2)
+    tok = lambda t: t.reshape(B, -1, H, D).to(torch.bfloat16).to(DEV)
+    for n in (2, 3, 8):
+        gold = torch.from_numpy(GOLD[f"case2_slow{n}"]).reshape(B, -1, H, D)
+        out = mattn.monarch_attn(tok(q), tok(k), tok(v), 1, 1, 1, b1, b2, sm_scale=s, num_iters=n)
+        # the golden output is that of the unrounded inputs: the input rounding alone moves it by ~1e-2
+        assert max_abs(out, gold) < 4e-2
+        ref = monarch.monarch_attn(tok(q).cpu(), tok(k).cpu(), tok(v).cpu(), 1, 1, 1, b1, b2, sm_scale=s, num_iters=n, dtype=torch.float32)
+        assert_close_16bit(out, ref, torch.bfloat16)
