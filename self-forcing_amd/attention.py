@@ -9,7 +9,7 @@ import warnings
 import torch
 
 from . import lib as _l
-from .monarch_attn import _DT, _check4, _stream
+from .monarch_attn import _DT, _check4, _stream, scratch as _scratch
 
 
 def _dense_desc(q, k, v, out, sm_scale):
@@ -52,7 +52,7 @@ def _dense_bwd(q, k, v, out, lse, dout, sm_scale, kv0=0, kv1=None):
     bd.kv_grad_start, bd.kv_grad_end = kv0, kv1
     n = C.c_size_t(0)
     _l.check(_l.load().sfm_dense_bwd_workspace_bytes(C.byref(bd), C.byref(n)))
-    ws = torch.empty(n.value, dtype=torch.uint8, device=q.device)
+    ws = _scratch(n.value, q.device)
     with torch.cuda.device(q.device):
         _l.check(_l.load().sfm_dense_bwd(C.byref(bd), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
                                          dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), n.value,

@@ -52,6 +52,24 @@ def _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, kv_block_ord
     return d
 
 
+_SCRATCH = {}
+
+
+def scratch(nbytes, device):
+    """The library's workspace for a call on `device`'s current stream: one grow-only byte buffer per (device, stream),
+    so that steady-state calls allocate nothing (a caller recording a HIP graph warms the buffer up with one eager
+    call first).  Calls on one stream are ordered, so they can share it; `release_scratch()` gives the memory back."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(device).cuda_stream)
+    buf = _SCRATCH.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = _SCRATCH[key] = torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+    return buf
+
+
+def release_scratch():
+    _SCRATCH.clear()
+
+
 def monarch_workspace_bytes(desc, heads_per_pass=0):
     n = C.c_size_t(0)
     _l.check(_l.load().sfm_monarch_workspace_bytes(C.byref(desc), heads_per_pass, C.byref(n)))
@@ -112,7 +130,7 @@ def _monarch_fwd_stats(q, k, v, tiling, sm_scale, kv_block_order, cbf, heads_per
     n = C.c_size_t(0)
     _l.check(_l.load().sfm_monarch_stats_bytes(C.byref(d), C.byref(n)))
     nbytes = monarch_workspace_bytes(d, heads_per_pass)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    ws = scratch(nbytes, q.device)
     stats = torch.empty(n.value // 4, dtype=torch.float32, device=q.device) if n.value else None
     with torch.cuda.device(q.device):
         if stats is None:
@@ -147,7 +165,7 @@ def _monarch_bwd(q, k, v, dout, tiling, sm_scale, kv_block_order, cbf, kv_f0=0, 
     bd.kv_grad_frame_start, bd.kv_grad_frame_end = kv_f0, kv_f1
     n = C.c_size_t(0)
     _l.check(_l.load().sfm_monarch_bwd_workspace_bytes(C.byref(bd), heads_per_pass, C.byref(n)))
-    ws = torch.empty(n.value, dtype=torch.uint8, device=q.device)
+    ws = scratch(n.value, q.device)
     with torch.cuda.device(q.device):
         if out is None or stats is None:
             _l.check(_l.load().sfm_monarch_bwd(C.byref(bd), q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(),
@@ -265,7 +283,7 @@ def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     d = _desc(q, k_cache, v_cache, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1, 0, num_iters, one_kernel)
     nbytes = monarch_workspace_bytes(d, heads_per_pass)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    ws = scratch(nbytes, q.device)
     with torch.cuda.device(q.device):
         _l.check(_l.load().sfm_monarch_attn_with_kv_cache(
             C.byref(d), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), new_k.data_ptr(), new_v.data_ptr(),
@@ -325,7 +343,7 @@ def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block
     out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     d = _desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, sm_scale, 1 if kv_block_order else 0, cbf, num_iters, one_kernel)
     nbytes = monarch_workspace_bytes(d, heads_per_pass)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    ws = scratch(nbytes, q.device)
     with torch.cuda.device(q.device):
         _l.check(_l.load().sfm_monarch_fwd(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                            ws.data_ptr(), nbytes, _stream(q)))

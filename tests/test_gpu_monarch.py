@@ -221,3 +221,31 @@ def test_host_argument_errors():
         mattn.monarch_attn(q.cpu(), kc, kc, 1, 1, 1, 3, 20)
     with pytest.raises(ValueError):
         mattn.monarch_attn(q, kc, kc, 1, 1, 1, 3, 20, block_causal_size=60)                  # needs Skv == Sq
+
+
+def test_wrappers_reuse_one_scratch_buffer_per_stream():
+    """Steady-state calls allocate nothing: the workspace is a grow-only buffer per (device, stream); results do not
+    depend on what an earlier, larger call left in it."""
+    mattn = sfa.monarch_attn
+    mattn.release_scratch()
+    h, w, H, D = 6, 20, 2, 128
+    q1, k1, v1 = (randn((1, n * h * w, H, D), 400 + i, torch.bfloat16).to(DEV) for i, n in enumerate((1, 3, 3)))
+    q2, k2, v2 = (randn((1, n * h * w, H, D), 410 + i, torch.bfloat16).to(DEV) for i, n in enumerate((2, 5, 5)))
+    small_first = mattn.monarch_attn(q1, k1, v1, 1, 1, 1, h, w)
+    key = (0, torch.cuda.current_stream().cuda_stream)
+    n_small = mattn._SCRATCH[key].numel()
+    mattn.monarch_attn(q2, k2, v2, 1, 1, 1, h, w)
+    buf = mattn._SCRATCH[key]
+    assert buf.numel() > n_small
+    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    small_again = mattn.monarch_attn(q1, k1, v1, 1, 1, 1, h, w)
+    assert mattn._SCRATCH[key] is buf                                   # no new workspace
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] - before == 1      # the output tensor only
+    assert torch.equal(small_again, small_first)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        other = mattn.monarch_attn(q1, k1, v1, 1, 1, 1, h, w)
+    side.synchronize()
+    assert (0, side.cuda_stream) in mattn._SCRATCH and torch.equal(other, small_first)
+    mattn.release_scratch()
+    assert not mattn._SCRATCH
