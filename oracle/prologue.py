@@ -9,6 +9,10 @@ Follows
                                           float64 by the angle of (frame+start_frame | row | col), result
                                           cast back to x's dtype
   * wan/modules/causal_model.py:801-807, 899-905  order: Linear -> RMSNorm -> view heads -> RoPE
+
+Pinned by the reference's own outputs (tests/golden/block_reference_vectors.npz: causal_rope_apply on three grids in
+float64 and bfloat16, the complex table, WanRMSNorm in float32 and bfloat16) in tests/test_block_reference_vectors.py, and by
+the closed forms and invariants of tests/test_oracle_dense_prologue.py.
 """
 import math
 
