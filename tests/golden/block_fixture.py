@@ -1,0 +1,89 @@
+"""Seeded sub-layers and inputs shared by make_wiring_reference_vectors.py (which plugs them into the reference's own
+`CausalWanAttentionBlock.forward` / `CausalHead.forward`) and by tests/test_block_reference_wiring.py (which plugs
+the same ones into the product's block and head).  The attention sub-layers are stand-ins: any deterministic
+function of their inputs shows whether the wiring around them (which modulation row goes where, the `1 +`, the
+residual sums) is the reference's."""
+import torch
+import torch.nn as nn
+
+DIM, FFN, FRAMES, FRAME_TOKENS, CTX = 48, 112, 3, 10, 7
+EPS = 1e-6
+
+
+def randn(seed, *shape):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=torch.float64)
+
+
+class SelfAttnStandIn(nn.Module):
+    """y = x W + (token index) * u: depends on every input channel and on the token's position."""
+
+    def __init__(self):
+        super().__init__()
+        self.w = nn.Parameter(randn(11, DIM, DIM) / DIM ** 0.5)
+        self.u = nn.Parameter(randn(12, DIM) * 0.01)
+
+    def apply_to(self, x):
+        pos = torch.arange(x.shape[1], dtype=x.dtype).view(1, -1, 1)
+        return x @ self.w + pos * self.u
+
+
+class CrossAttnStandIn(nn.Module):
+    """y = tanh(x W) + mean over the context tokens of (context V)."""
+
+    def __init__(self):
+        super().__init__()
+        self.w = nn.Parameter(randn(13, DIM, DIM) / DIM ** 0.5)
+        self.v = nn.Parameter(randn(14, DIM, DIM) / DIM ** 0.5)
+
+    def apply_to(self, x, context):
+        return torch.tanh(x @ self.w) + (context @ self.v).mean(dim=1, keepdim=True)
+
+
+def parameters():
+    """name -> tensor for the block's and the head's own parameters."""
+    return {
+        "modulation": randn(21, 1, 6, DIM) / DIM ** 0.5,
+        "norm3.weight": 1 + 0.2 * randn(22, DIM), "norm3.bias": 0.1 * randn(23, DIM),
+        "ffn.0.weight": randn(24, FFN, DIM) / DIM ** 0.5, "ffn.0.bias": 0.1 * randn(25, FFN),
+        "ffn.2.weight": randn(26, DIM, FFN) / FFN ** 0.5, "ffn.2.bias": 0.1 * randn(27, DIM),
+        "head.modulation": randn(28, 1, 2, DIM) / DIM ** 0.5,
+        "head.head.weight": randn(29, 16, DIM) / DIM ** 0.5, "head.head.bias": 0.1 * randn(30, 16),
+    }
+
+
+def inputs():
+    L = FRAMES * FRAME_TOKENS
+    return {"x": randn(31, 2, L, DIM), "e": 0.5 * randn(32, 2, FRAMES, 6, DIM), "context": randn(33, 2, CTX, DIM),
+            "e_head": 0.5 * randn(34, 2, FRAMES, 1, DIM)}
+
+
+# ---- whole-model wiring (embeddings -> blocks -> head -> unpatchify) -----------------------------------------------
+M_DIM, M_IN, M_OUT, M_FREQ, M_TEXT, M_TEXT_LEN, M_LAYERS = 32, 4, 4, 16, 24, 6, 2
+M_PATCH = (1, 2, 2)
+M_LATENT = (2, M_IN, 3, 4, 6)            # [B, C, F, H, W] -> 3 frames of 2 x 3 tokens
+
+
+def model_parameter(name, shape):
+    import zlib
+    t = randn(zlib.crc32(name.encode()) & 0x7FFFFFFF, *shape)
+    if name.endswith(".bias"):
+        return 0.1 * t
+    fan_in = 1
+    for s in shape[1:]:
+        fan_in *= s
+    return t / max(fan_in, 1) ** 0.5
+
+
+def model_inputs():
+    return {"x": randn(51, *M_LATENT), "t": torch.tensor([[1000.0, 937.5, 833.0], [625.0, 625.0, 3.0]], dtype=torch.float64),
+            "context": randn(52, 2, 5, M_TEXT)}            # 5 text tokens: padded to M_TEXT_LEN by the model
+
+
+def block_stand_in(x, e, context, index):
+    """Stands in for a whole attention block: uses every one of the six modulation rows with its own weight, per frame,
+    and the embedded context."""
+    nf = e.shape[1]
+    fs = x.shape[1] // nf
+    coef = sum((r + 1) * e[:, :, r] for r in range(6))                        # [B, F, C]
+    y = x + 0.1 * (index + 1) * (torch.tanh(x).unflatten(1, (nf, fs)) * coef.unsqueeze(2)).flatten(1, 2)
+    return y + 0.01 * context.mean(dim=1, keepdim=True)
