@@ -87,3 +87,39 @@ def block_stand_in(x, e, context, index):
     coef = sum((r + 1) * e[:, :, r] for r in range(6))                        # [B, F, C]
     y = x + 0.1 * (index + 1) * (torch.tanh(x).unflatten(1, (nf, fs)) * coef.unsqueeze(2)).flatten(1, 2)
     return y + 0.01 * context.mean(dim=1, keepdim=True)
+
+
+# ---- self-attention with the KV cache (cache state machine, RoPE start frame, dispatch) ---------------------------------
+A_DIM, A_HEADS, A_H, A_W = 32, 2, 4, 6
+A_FRAME = A_H * A_W
+
+# name -> (local_attn_size, sink_size, cache frames, flags, [(current_start in frames, chunk frames), ...])
+A_SCENARIOS = {
+    # whole-history cache, framewise Monarch; every chunk is run twice (a denoising pass, then the clean re-run)
+    "full_framewise": (-1, 0, 7, dict(use_framewise=True), [(0, 2), (0, 2), (2, 2), (2, 2), (4, 3), (4, 3)]),
+    # three frames tied per block, h_reduce = 2, dense attention on the first chunk (USE_DENSE_INIT)
+    "tied_reduce_init": (-1, 0, 6, dict(h_reduce=2, use_dense_init=True), [(0, 3), (0, 3), (3, 3), (3, 3)]),
+    # window of 4 frames with one sink frame: evictions from the fifth frame on, re-runs after an eviction
+    "window_sink": (4, 1, 4, dict(use_framewise=True), [(0, 1), (1, 1), (2, 1), (3, 1), (4, 1), (4, 1), (5, 1), (6, 2), (6, 2)]),
+    # Monarch disabled: dense attention, cache in token order, window without sink
+    "dense_window": (3, 0, 3, dict(disable_monarch=True), [(0, 1), (1, 2), (3, 1), (3, 1), (4, 2)]),
+    # refinement passes
+    "iters": (-1, 0, 4, dict(use_framewise=True, num_iters=3), [(0, 2), (2, 2), (2, 2)]),
+}
+
+
+def attn_parameter(name, shape):
+    import zlib
+    t = randn((zlib.crc32(("attn." + name).encode()) & 0x7FFFFFFF), *shape)
+    if name.endswith(".bias"):
+        return 0.1 * t
+    if name.startswith("norm_"):
+        return 1 + 0.2 * t
+    return t / shape[-1] ** 0.5
+
+
+def attn_input(scenario, call):
+    import zlib
+    _, _, _, _, calls = A_SCENARIOS[scenario]
+    frames = calls[call][1]
+    return randn(zlib.crc32(f"{scenario}.{call}".encode()) & 0x7FFFFFFF, 1, frames * A_FRAME, A_DIM)

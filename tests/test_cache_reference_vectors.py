@@ -1,0 +1,69 @@
+"""The product's `CausalWanSelfAttention` (cache state machine, eviction with sink frames, RoPE start frame, dispatch
+between Monarch, dense first chunk, dense fallback and refinement passes, block-order cache rows) against what the
+reference's own `CausalWanSelfAttention.forward` did, call by call, on the same scripted sequences
+(tests/golden/cache_reference_vectors.npz, written by tests/golden/make_cache_reference_vectors.py; scenarios and seeds in
+tests/golden/block_fixture.py).  CPU, float64, oracle operators."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import self_forcing_amd as sfa
+from oracle.ops import OracleOps
+
+sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+import block_fixture as fx  # noqa: E402
+
+cm = sfa.causal_model
+GOLD = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "cache_reference_vectors.npz"))
+
+
+def _module(local, sink, cache_frames, flags):
+    total = cache_frames * fx.A_FRAME if local == -1 else 7 * fx.A_FRAME
+    m = cm.CausalWanSelfAttention(fx.A_DIM, fx.A_HEADS, local, sink, True, fx.EPS, 0, (fx.A_H, fx.A_W), total,
+                                  cm.AttentionFlags(0, **flags), OracleOps(compute_dtype=torch.float64)).double().eval()
+    with torch.no_grad():
+        for k, p in m.named_parameters():
+            p.copy_(fx.attn_parameter(k, tuple(p.shape)))
+    return m
+
+
+@pytest.mark.parametrize("scen", sorted(fx.A_SCENARIOS))
+def test_cache_sequence_matches_the_reference_forward(scen):
+    local, sink, cache_frames, flags, calls = fx.A_SCENARIOS[scen]
+    m = _module(local, sink, cache_frames, flags)
+    d = fx.A_DIM // fx.A_HEADS
+    kv = {"k": torch.zeros(1, cache_frames * fx.A_FRAME, fx.A_HEADS, d, dtype=torch.float64),
+          "v": torch.zeros(1, cache_frames * fx.A_FRAME, fx.A_HEADS, d, dtype=torch.float64),
+          "global_end_index": torch.tensor([0], dtype=torch.long), "local_end_index": torch.tensor([0], dtype=torch.long)}
+    wts = torch.arange(1, fx.A_HEADS * d + 1, dtype=torch.float64).view(1, 1, fx.A_HEADS, d)
+    for i, (start_frame, frames) in enumerate(calls):
+        with torch.no_grad():
+            y = m(fx.attn_input(scen, i), (frames, fx.A_H, fx.A_W), kv, start_frame * fx.A_FRAME)
+        # the reference's pure-torch Monarch formulas take their softmaxes in float32 (the dense paths do not)
+        np.testing.assert_allclose(y.numpy(), GOLD[f"{scen}.{i}.out"], atol=1e-9 if flags.get("disable_monarch") else 5e-6, rtol=0,
+                                   err_msg=f"output of call {i}")
+        ends = (int(kv["global_end_index"].item()), int(kv["local_end_index"].item()))
+        assert ends == tuple(int(v) for v in GOLD[f"{scen}.{i}.ends"]), (i, ends)
+        np.testing.assert_allclose((kv["k"] * wts).sum(dim=(2, 3)).numpy(), GOLD[f"{scen}.{i}.k_rows"], atol=1e-9, rtol=0,
+                                   err_msg=f"K cache rows after call {i}")
+        np.testing.assert_allclose((kv["v"] * wts).sum(dim=(2, 3)).numpy(), GOLD[f"{scen}.{i}.v_rows"], atol=1e-9, rtol=0,
+                                   err_msg=f"V cache rows after call {i}")
+    np.testing.assert_allclose(kv["k"].numpy(), GOLD[f"{scen}.k"], atol=1e-10, rtol=0)
+    np.testing.assert_allclose(kv["v"].numpy(), GOLD[f"{scen}.v"], atol=1e-10, rtol=0)
+
+
+def test_a_wrong_sink_size_would_show():
+    """Sensitivity of the pin: the windowed scenario with the sink frame ignored ends with different cache rows."""
+    local, sink, cache_frames, flags, calls = fx.A_SCENARIOS["window_sink"]
+    m = _module(local, 0, cache_frames, flags)
+    d = fx.A_DIM // fx.A_HEADS
+    kv = {"k": torch.zeros(1, cache_frames * fx.A_FRAME, fx.A_HEADS, d, dtype=torch.float64),
+          "v": torch.zeros(1, cache_frames * fx.A_FRAME, fx.A_HEADS, d, dtype=torch.float64),
+          "global_end_index": torch.tensor([0], dtype=torch.long), "local_end_index": torch.tensor([0], dtype=torch.long)}
+    for i, (start_frame, frames) in enumerate(calls):
+        with torch.no_grad():
+            m(fx.attn_input("window_sink", i), (frames, fx.A_H, fx.A_W), kv, start_frame * fx.A_FRAME)
+    assert np.abs(kv["k"].numpy() - GOLD["window_sink.k"]).max() > 1e-2
