@@ -123,3 +123,43 @@ def attn_input(scenario, call):
     _, _, _, _, calls = A_SCENARIOS[scenario]
     frames = calls[call][1]
     return randn(zlib.crc32(f"{scenario}.{call}".encode()) & 0x7FFFFFFF, 1, frames * A_FRAME, A_DIM)
+
+
+# ---- the sampler's chunk loop (pipeline) ------------------------------------------------------------------------------
+P_FRAMES, P_C, P_H, P_W, P_FRAME_TOKENS = 6, 2, 4, 6, 6            # latents [1, 6, 2, 4, 6]; 6 tokens per frame after patching
+
+
+class GeneratorStandIn(nn.Module):
+    """Stands in for the wrapped DiT: a deterministic function of the noisy latents, the timestep, the chunk's start
+    token and the prompt, and a log of what it was called with."""
+
+    def __init__(self, scheduler):
+        super().__init__()
+        self.scheduler = scheduler
+        self.model = types_namespace(num_layers=2, num_heads=2, dim=8, local_attn_size=-1)
+        self.calls = []
+
+    def get_scheduler(self):
+        return self.scheduler
+
+    def forward(self, noisy_image_or_video, conditional_dict, timestep, kv_cache=None, crossattn_cache=None, current_start=None):
+        t = timestep.float()
+        self.calls.append((tuple(noisy_image_or_video.shape), [round(float(v), 3) for v in t.flatten().tolist()], int(current_start),
+                           int(kv_cache[0]["global_end_index"].item()), bool(crossattn_cache[0]["is_init"])))
+        for c in crossattn_cache:
+            c["is_init"] = True
+        for c in kv_cache:                                   # what the model's self-attention does to the counters
+            c["global_end_index"].fill_(int(current_start) + noisy_image_or_video.shape[1] * P_FRAME_TOKENS)
+        x0 = (0.8 * noisy_image_or_video + 0.1 * torch.sin(t / 100.0).view(*t.shape, 1, 1, 1) + 1e-3 * float(current_start)
+              + 0.05 * conditional_dict["prompt_embeds"].mean())
+        return -x0, x0
+
+
+def types_namespace(**kw):
+    import types
+    return types.SimpleNamespace(**kw)
+
+
+def pipeline_inputs():
+    g = torch.Generator().manual_seed(61)
+    return {"noise": torch.randn(1, P_FRAMES, P_C, P_H, P_W, generator=g), "prompt": torch.randn(1, 5, 4, generator=g)}
