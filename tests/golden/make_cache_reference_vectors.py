@@ -116,6 +116,20 @@ def main():
                 out[f"{scen}.v"] = kv["v"].numpy().copy()
             out[f"{scen}.{i}.ends"] = np.array([kv["global_end_index"].item(), kv["local_end_index"].item()])
         print(scen, "ok:", [tuple(out[f"{scen}.{i}.ends"]) for i in range(len(calls))])
+    # ---- cross-attention with its cache (model.py:733-768): first call fills the cache, the second reads it (the context
+    # it is given then is ignored)
+    cns = {"torch": torch, "flash_attention": lambda q, k, v, k_lens=None: softmax_attention(q, k, v)}
+    extract(f"{REF}/model.py", ("forward",), cns, cls="WanT2VCrossAttention")
+    me = types.SimpleNamespace(num_heads=fx.A_HEADS, head_dim=d, q=linear("cross.q"), k=linear("cross.k"), v=linear("cross.v"),
+                               o=linear("cross.o"), norm_q=norm("cross.norm_q"), norm_k=norm("cross.norm_k"))
+    cache = {"is_init": False, "k": None, "v": None}
+    xs = [fx.randn(71, 1, 30, fx.A_DIM), fx.randn(72, 1, 18, fx.A_DIM)]
+    ctx = [fx.randn(73, 1, 9, fx.A_DIM), fx.randn(74, 1, 9, fx.A_DIM)]
+    with torch.no_grad():
+        for i in range(2):
+            out[f"cross.{i}.out"] = cns["forward"](me, xs[i], ctx[i], None, crossattn_cache=cache).numpy()
+        out["cross.nocache"] = cns["forward"](me, xs[1], ctx[1], None).numpy()
+    out["cross.k"] = cache["k"].numpy()
     np.savez_compressed(OUT, **out)
     print("wrote", OUT, os.path.getsize(OUT), "bytes")
 

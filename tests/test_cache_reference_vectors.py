@@ -67,3 +67,20 @@ def test_a_wrong_sink_size_would_show():
         with torch.no_grad():
             m(fx.attn_input("window_sink", i), (frames, fx.A_H, fx.A_W), kv, start_frame * fx.A_FRAME)
     assert np.abs(kv["k"].numpy() - GOLD["window_sink.k"]).max() > 1e-2
+
+
+def test_cross_attention_with_its_cache_matches_the_reference_forward():
+    """model.py:733-768: the first call computes and keeps the text K/V, later calls read them whatever context they get."""
+    m = cm.WanT2VCrossAttention(fx.A_DIM, fx.A_HEADS, fx.EPS, OracleOps(compute_dtype=torch.float64)).double().eval()
+    with torch.no_grad():
+        for k, p in m.named_parameters():
+            p.copy_(fx.attn_parameter("cross." + k, tuple(p.shape)))
+    cache = {"is_init": False, "k": None, "v": None}
+    xs = [fx.randn(71, 1, 30, fx.A_DIM), fx.randn(72, 1, 18, fx.A_DIM)]
+    ctx = [fx.randn(73, 1, 9, fx.A_DIM), fx.randn(74, 1, 9, fx.A_DIM)]
+    with torch.no_grad():
+        for i in range(2):
+            np.testing.assert_allclose(m(xs[i], ctx[i], cache).numpy(), GOLD[f"cross.{i}.out"], atol=1e-9, rtol=0)
+        np.testing.assert_allclose(m(xs[1], ctx[1], None).numpy(), GOLD["cross.nocache"], atol=1e-9, rtol=0)
+    assert cache["is_init"]
+    np.testing.assert_allclose(cache["k"].numpy(), GOLD["cross.k"], atol=1e-10, rtol=0)
