@@ -57,6 +57,11 @@ def main():
         out[f"case{ci}_ref_op"] = fn["monarch_attn_ref_op"](q, k, v, s).numpy()
         for n in ITERS:
             out[f"case{ci}_slow{n}"] = fn["monarch_attn_slow"](q, k, v, s, num_iters=n).numpy()
+        # gradients of the one-iteration formula by autograd, for the cotangent drawn from seed + 1000
+        qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+        cot = torch.randn(q.shape, generator=torch.Generator().manual_seed(seed + 1000), dtype=torch.float64)
+        fn["monarch_attn_ref_op"](qa, ka, va, s).backward(cot)
+        out[f"case{ci}_dq"], out[f"case{ci}_dk"], out[f"case{ci}_dv"] = qa.grad.numpy(), ka.grad.numpy(), va.grad.numpy()
     # block-order permutation: token ids through rearrange_fn for several tilings (h=6, w=8, 3 frames)
     h, w, F = 6, 8, 3
     x = torch.arange(F * h * w, dtype=torch.float64).reshape(1, -1, 1, 1)

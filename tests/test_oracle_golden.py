@@ -44,3 +44,17 @@ def test_iterated_refinement_matches_reference_formula(ci, n):
 def test_block_order_matches_reference_permutation(tiling):
     idx = blocks.block_to_token_index(3 * 6 * 8, *tiling, 6, 8)
     assert np.array_equal(idx, GOLD["order_%d_%d_%d" % tiling])
+
+
+@pytest.mark.parametrize("ci", [0, 1, 2])
+def test_gradients_match_autograd_of_the_reference_formula(ci):
+    """dq, dk, dv of the one-iteration formula for a seeded cotangent: autograd through the oracle against autograd
+    through the reference's `monarch_attn_ref_op` (float32 softmaxes there: 1e-5)."""
+    q, k, v, s = _inputs(ci)
+    seed = int(GOLD[f"case{ci}_meta"][0])
+    cot = torch.randn(q.shape, generator=torch.Generator().manual_seed(seed + 1000), dtype=torch.float64)
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    monarch.monarch_1iter(qa, ka, va, s).backward(cot)
+    for name, t in (("dq", qa), ("dk", ka), ("dv", va)):
+        ref = GOLD[f"case{ci}_{name}"]
+        assert np.abs(t.grad.numpy() - ref).max() < 1e-5 * max(1.0, np.abs(ref).max()), name
