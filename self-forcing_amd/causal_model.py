@@ -359,10 +359,11 @@ class CausalWanAttentionBlock(nn.Module):
         self.ffn = nn.Sequential(nn.Linear(dim, ffn_dim), nn.GELU(approximate='tanh'), nn.Linear(ffn_dim, dim))
         self.modulation = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
 
-    def forward(self, x, e, grid, context, kv_cache, crossattn_cache, current_start):
-        """x [B, L, C]; e [B, F, 6, C] per-frame modulation."""
+    def forward(self, x, e, grid, context, kv_cache, crossattn_cache, current_start, e_summed=None):
+        """x [B, L, C]; e [B, F, 6, C] per-frame modulation; e_summed: `modulation + e` where the caller has already
+        formed it (the model does so for all blocks in one launch)."""
         ops = self.ops
-        e = (self.modulation.unsqueeze(1) + e).chunk(6, dim=2)
+        e = (self.modulation.unsqueeze(1) + e if e_summed is None else e_summed).chunk(6, dim=2)
         y = self.self_attn(ops.ln_modulate(x, e[1], e[0], self.eps), grid, kv_cache, current_start)
         if isinstance(self.norm3, nn.Identity):
             x = xn = ops.gate_residual(x, y, e[2])
@@ -442,6 +443,19 @@ class CausalWanModel(nn.Module):
         wgt = self.patch_embedding.weight.view(self.dim, C * ph * pw)
         return F.linear(p, wgt, self.patch_embedding.bias), (Fr, h, w)
 
+    def _summed_modulations(self, e0):
+        """`block.modulation + e0` of every block as one [layers, B, F, 6, C] tensor (one launch per pass instead of one
+        per block; the same sums).  The stacked parameters are rebuilt when one of them changes.  None where the blocks
+        are not this module's own (tests plug in stand-ins) or gradients are wanted."""
+        if torch.is_grad_enabled() or not all(isinstance(b, CausalWanAttentionBlock) for b in self.blocks):
+            return None
+        mods = [b.modulation for b in self.blocks]
+        key = tuple((m.data_ptr(), m._version) for m in mods)
+        if getattr(self, "_mod_stack", None) is None or self._mod_stack[0] != key:
+            with torch.no_grad():
+                self._mod_stack = (key, torch.stack([m.detach() for m in mods]).unsqueeze(2))     # [L, 1, 1, 6, C]
+        return self._mod_stack[1] + e0.unsqueeze(0)
+
     def unpatchify(self, x, grid):
         """[B, L, prod(patch)*C_out] -> [B, C_out, F, H, W] (causal_model.py:1896-1919)."""
         Fr, h, w = grid
@@ -463,8 +477,9 @@ class CausalWanModel(nn.Module):
             context = torch.cat([context, context.new_zeros(context.shape[0], self.text_len - context.shape[1],
                                                             context.shape[2])], dim=1)
         context = self.text_embedding(context)
+        e_all = self._summed_modulations(e0)
         for i, block in enumerate(self.blocks):
             x = block(x, e0, grid, context, kv_cache[i], crossattn_cache[i] if crossattn_cache is not None else None,
-                      current_start)
+                      current_start, **({} if e_all is None else {"e_summed": e_all[i]}))
         x = self.head(x, e.unflatten(0, t.shape).unsqueeze(2))
         return self.unpatchify(x.flatten(1, 2) if x.dim() == 4 else x, grid)

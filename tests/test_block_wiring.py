@@ -146,3 +146,20 @@ def test_head_is_linear_of_the_modulated_norm():
         plain = hd(x, -hd.modulation.unsqueeze(1).expand(1, FR, 2, DIM)).flatten(1, 2)
     assert torch.allclose(got, ref, atol=1e-5) and not torch.allclose(got, swapped, atol=1e-3)
     assert torch.allclose(plain, hd.head(ln), atol=1e-5)
+
+
+def test_model_sums_all_modulations_at_once_with_the_same_result():
+    """CausalWanModel forms `modulation + e0` for every block in one tensor; the blocks then see exactly what they would
+    have computed themselves, also after a parameter changes."""
+    torch.manual_seed(11)
+    m = cm.CausalWanModel(dim=32, ffn_dim=64, num_heads=2, num_layers=3, in_dim=4, out_dim=4, freq_dim=16, text_dim=8, text_len=4,
+                          frame_hw=(2, 3), ops=OracleOps()).eval()
+    e0 = torch.randn(2, 3, 6, 32)
+    with torch.no_grad():
+        got = m._summed_modulations(e0)
+        assert got.shape == (3, 2, 3, 6, 32)
+        for i, b in enumerate(m.blocks):
+            assert torch.equal(got[i], b.modulation.unsqueeze(1) + e0)
+        m.blocks[1].modulation.add_(1.0)
+        assert torch.equal(m._summed_modulations(e0)[1], m.blocks[1].modulation.unsqueeze(1) + e0)
+    assert m._summed_modulations(e0) is None                     # gradients wanted: every block adds its own
