@@ -279,6 +279,11 @@ def op_level(torch, sfa, args):
     s2_waves, s2_kb = B * H * A * B2, (F * B1 * 2 * D + 1023) // 1024
     read_us = C.c_float(0)
     L.check(lib.sfm_probe_row_stream(s2_waves, s2_kb, ws.data_ptr(), ws.numel(), stream, C.byref(read_us)))
+    # the rate at which all compute units together can be fed from L2 (one workgroup per CU streaming a shared 2 MB window)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    l2_us = C.c_float(0)
+    L.check(lib.sfm_probe_l2_read(cus, 64, ws.data_ptr(), ws.numel(), stream, C.byref(l2_us)))
+    l2_tbs = cus * 64 * 32768 / (l2_us.value * 1e-6) / 1e12
     del ws
 
     traffic = measured_traffic()
@@ -296,6 +301,7 @@ def op_level(torch, sfa, args):
                          "tflops": 8 * MONARCH_FLOPS / (iter_ms * 1e-3) / 1e12},
         "monarch_bwd": {"workload": "gradients of q and of all 21 cached K/V frames at the same shape",
                         "ms_per_call": bwd_ms, "ms_per_call_recomputing_statistics": bwd["recompute"]},
+        "l2_read_probe_tbs": l2_tbs,
         "dense_fallback": {"ms_per_call": dense_ms, "tflops": dense_tfl, "mfma_frac": dense_tfl / MFMA_BF16_PEAK_TFLOPS,
                            "mfma_probe_tflops": probe.value, "frac_of_probe": dense_tfl / probe.value,
                            "bwd_ms_per_call": dense_bwd["all_keys"], "bwd_ms_per_call_new_chunk_keys": dense_bwd["new_chunk_keys"]},

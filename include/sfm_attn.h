@@ -331,6 +331,14 @@ int sfm_probe_tile_traffic(int32_t tiles, int32_t rows_in, int32_t rows_out, int
 int sfm_probe_row_stream(int32_t waves, int32_t kb_per_block, const void* workspace, size_t workspace_bytes, void* stream,
                          float* us);
 
+/* Measurement aid with no counterpart in the reference: the rate at which the compute units can be fed from L2.
+ * `workgroups` workgroups each stream `stages` (4..64) stages of 32 KB of one shared 2 MB window of `workspace`
+ * (device memory, 256-byte aligned, >= 2 MiB + 256 bytes; read, plus 4 bytes written behind the window) into LDS.
+ * Runs on `stream`, waits, and returns the mean duration of one launch in microseconds: workgroups * stages * 32 KiB
+ * per that time is the aggregate L2 -> CU read rate (about 16 TB/s with one workgroup per compute unit on MI355X,
+ * twice that per compute unit when only an eighth of them ask). */
+int sfm_probe_l2_read(int32_t workgroups, int32_t stages, void* workspace, size_t workspace_bytes, void* stream, float* us);
+
 /* Implementation switches for measurements and tests; no counterpart in the reference.  The environment is read
  * ONCE, when the library is loaded: a variable of the same name as a bit below that is set to anything but "0" turns
  * the bit on (SFM_BWD_SIMT=1 ...), SFM_NO_ROCBLAS makes the library behave as where rocBLAS is absent, and SFM_S1_WGS=n

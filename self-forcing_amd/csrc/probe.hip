@@ -223,3 +223,78 @@ extern "C" int sfm_probe_row_stream(int32_t waves, int32_t kb_per_block, const v
     *us = ms * 1e3f / reps;
     return SFM_OK;
 }
+
+
+// ------------------------------------------------------------------------------------------------
+// L2 -> compute unit read rate: every workgroup streams `stages` stages of 32 KB (64-byte pieces of 512 rows that are
+// 4 KB apart, the next piece of every row per stage) of one 2 MB window that all workgroups share, i.e. that stays in
+// every XCD's L2, straight into LDS (global_load_lds_dwordx4, three stages in flight).  What a tile-streaming kernel
+// (one-kernel Monarch forward, block GEMM) can be fed at most when its tiles come from L2.
+// ------------------------------------------------------------------------------------------------
+namespace sfm {
+namespace {
+__device__ __forceinline__ void pr_load_lds16(const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
+}
+__global__ __launch_bounds__(256) void l2_read_kernel(const char* src, int stages, float* sink) {
+    extern __shared__ __attribute__((aligned(256))) char lds_pr[];
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds_pr;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint32_t off[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) off[j] = (uint32_t)((4 * j + wave) * 16 + (lane >> 2)) * 4096 + (lane & 3) * 16;
+    const char* base = src;
+    for (int s = 0; s < stages; ++s) {
+        const uint32_t mb = lds0 + (uint32_t)(s & 3) * 32768 + wave * 1024;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pr_load_lds16(base, off[j], mb + j * 4096);
+        base += 64;
+        if (s >= 3) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const u32x4 v = *(const u32x4*)(lds_pr + tid * 16);
+    if (v.x == 0x12345678u && v.y == 0x9abcdef0u) sink[0] = 1.f;        // keeps the loads; practically never true
+}
+}  // namespace
+}  // namespace sfm
+
+extern "C" int sfm_probe_l2_read(int32_t workgroups, int32_t stages, void* workspace, size_t workspace_bytes, void* stream, float* us) {
+    using namespace sfm;
+    if (workgroups < 1 || stages < 4 || stages > 64 || workspace == nullptr || us == nullptr) {
+        set_error("sfm_probe_l2_read: workgroups >= 1, 4 <= stages <= 64, workspace and us non-null");
+        return SFM_ERR_RANGE;
+    }
+    const size_t need = (size_t)512 * 4096 + 256;
+    if (need > workspace_bytes || ((uintptr_t)workspace & 255)) {
+        set_error("sfm_probe_l2_read: workspace of %zu bytes, 256-byte aligned, needed", need);
+        return SFM_ERR_WORKSPACE;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    if (hipFuncSetAttribute((const void*)l2_read_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 131072) != hipSuccess) {
+        set_error("sfm_probe_l2_read: hipFuncSetAttribute failed");
+        return SFM_ERR_HIP;
+    }
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        set_error("sfm_probe_l2_read: hipEventCreate failed");
+        return SFM_ERR_HIP;
+    }
+    const int reps = 10;
+    float* sink = (float*)((char*)workspace + (size_t)512 * 4096);
+    auto launch = [&] { hipLaunchKernelGGL(l2_read_kernel, dim3(workgroups), dim3(256), 131072, st, (const char*)workspace, stages, sink); };
+    launch();                                                // warm-up: the window is in L2 afterwards
+    (void)hipEventRecord(e0, st);
+    for (int i = 0; i < reps; ++i) launch();
+    (void)hipEventRecord(e1, st);
+    hipError_t e = hipEventSynchronize(e1);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (e != hipSuccess || ms <= 0.f) {
+        set_error("sfm_probe_l2_read: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    *us = ms * 1e3f / reps;
+    return SFM_OK;
+}

@@ -26,7 +26,7 @@ SYMBOLS = [
     "sfm_monarch_attn_with_kv_cache_static",
     "sfm_dense_fwd", "sfm_full_attention_with_kv_cache", "sfm_qk_prologue", "sfm_ln_modulate", "sfm_gate_residual",
     "sfm_rms_norm", "sfm_gate_residual_ln", "sfm_linear", "sfm_monarch_bwd_workspace_bytes", "sfm_monarch_bwd", "sfm_monarch_bwd_uses_gemm",
-    "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_dense_bwd_workspace_bytes", "sfm_dense_bwd", "sfm_probe_mfma_bf16", "sfm_probe_tile_traffic", "sfm_probe_row_stream", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_set_switches", "sfm_get_switches", "sfm_last_error", "sfm_version",
+    "sfm_monarch_stats_bytes", "sfm_monarch_fwd_stats", "sfm_monarch_bwd_saved", "sfm_dense_bwd_workspace_bytes", "sfm_dense_bwd", "sfm_probe_mfma_bf16", "sfm_probe_tile_traffic", "sfm_probe_row_stream", "sfm_probe_l2_read", "sfm_conv3d_cl", "sfm_vae_norm_act", "sfm_set_switches", "sfm_get_switches", "sfm_last_error", "sfm_version",
 ]
 
 
@@ -133,6 +133,7 @@ def load():
     lib.sfm_probe_mfma_bf16.argtypes = [C.c_int32, P, C.POINTER(C.c_float)]
     lib.sfm_probe_tile_traffic.argtypes = [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, P, C.c_size_t, P, C.POINTER(C.c_float)]
     lib.sfm_probe_row_stream.argtypes = [C.c_int32, C.c_int32, P, C.c_size_t, P, C.POINTER(C.c_float)]
+    lib.sfm_probe_l2_read.argtypes = [C.c_int32, C.c_int32, P, C.c_size_t, P, C.POINTER(C.c_float)]
     lib.sfm_set_switches.argtypes = [C.c_uint]
     lib.sfm_set_switches.restype = lib.sfm_get_switches.restype = C.c_uint
     for name in SYMBOLS:
