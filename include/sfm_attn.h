@@ -263,7 +263,8 @@ int sfm_gate_residual_ln(int32_t dtype, int64_t rows, int32_t C, float eps, void
  *                          gate = NULL: out = res + (x w^T + bias); res ([M, N], rows res_stride apart) may be `out`.
  * Rounding points are the eager chain's: the product plus bias is rounded to the tensor dtype, the GELU of that value
  * is rounded, the gated product is rounded, the residual sum is rounded.  K a multiple of 64, N a multiple of 8, all
- * strides multiples of 8 elements, pointers 16-byte aligned, operands below 4 GiB each. */
+ * strides multiples of 8 elements, pointers 16-byte aligned, operands below 4 GiB each.  `out` must not overlap x or
+ * w (SFM_ERR_RANGE): workgroups read whole rows of both while others already store. */
 #define SFM_EPI_NONE          0
 #define SFM_EPI_GELU_TANH     1
 #define SFM_EPI_GATE_RESIDUAL 2

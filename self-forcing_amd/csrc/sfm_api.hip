@@ -1116,6 +1116,18 @@ int sfm_linear(const sfm_linear_desc* d, const void* x, const void* w, const voi
         set_error("tensors must be 16-byte aligned");
         return SFM_ERR_ALIGN;
     }
+    // the product reads whole rows of x and w while other workgroups already write out: they must not overlap
+    // (res may be out: every element is read and written by the same lane)
+    const char* o0 = (const char*)out;
+    const char* o1 = o0 + ((size_t)(d->M - 1) * d->out_stride + d->N) * 2;
+    const char* x0 = (const char*)x;
+    const char* x1 = x0 + ((size_t)(d->M - 1) * d->x_stride + d->K) * 2;
+    const char* w0 = (const char*)w;
+    const char* w1 = w0 + (size_t)d->N * d->K * 2;
+    if ((x0 < o1 && o0 < x1) || (w0 < o1 && o0 < w1)) {
+        set_error("out overlaps x or w");
+        return SFM_ERR_RANGE;
+    }
     return launch_linear(*d, x, w, bias, gr ? res : nullptr, gr ? gate : nullptr, out, (hipStream_t)stream);
 }
 

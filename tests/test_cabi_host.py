@@ -369,3 +369,28 @@ def test_fp32_kernel_limits_are_reported_before_anything_is_written():
     d.q_stride = d.o_stride = (C.c_int64 * 3)(3 * 30 * 104 * 256, 256, 128)
     d.k_stride = d.v_stride = (C.c_int64 * 3)(6 * 30 * 104 * 256, 256, 128)
     assert _ws(d, 1)[0] == 0
+
+
+def test_linear_descriptor_errors():
+    """sfm_linear validates before any launch: these calls return their error codes without a GPU."""
+    lib = L.load()
+    d = L.LinearDesc()
+    d.dtype, d.epilogue, d.M, d.N, d.K = L.SFM_BF16, L.EPI_NONE, 256, 64, 128
+    d.x_stride, d.out_stride = 128, 64
+    call = lambda **kw: lib.sfm_linear(C.byref(d), kw.get("x", 0x10000), kw.get("w", 0x200000), None, kw.get("res"), None,
+                                       kw.get("out", 0x400000), None)
+    assert call(x=None) == -1
+    d.dtype = L.SFM_F32
+    assert call() == -2
+    d.dtype, d.K = L.SFM_BF16, 96
+    assert call() == -3 and b"multiple of 64" in lib.sfm_last_error()
+    d.K, d.epilogue = 128, 7
+    assert call() == -3
+    d.epilogue = L.EPI_GATE_RESIDUAL
+    assert call() == -1 and b"needs res" in lib.sfm_last_error()
+    d.epilogue, d.x_stride = L.EPI_NONE, 100
+    assert call() == -5
+    d.x_stride = 128
+    assert call(out=0x10000 + 256) == -4 and b"overlaps" in lib.sfm_last_error()  # out inside x
+    assert call(out=0x200000 - 64) == -4                                          # out runs into w
+    assert call(x=0x10008) == -7
