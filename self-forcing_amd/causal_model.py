@@ -359,18 +359,27 @@ class CausalWanAttentionBlock(nn.Module):
         self.ffn = nn.Sequential(nn.Linear(dim, ffn_dim), nn.GELU(approximate='tanh'), nn.Linear(ffn_dim, dim))
         self.modulation = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
 
-    def forward(self, x, e, grid, context, kv_cache, crossattn_cache, current_start, e_summed=None):
+    def forward(self, x, e, grid, context, kv_cache, crossattn_cache, current_start, e_summed=None, xn=None, next_mod=None):
         """x [B, L, C]; e [B, F, 6, C] per-frame modulation; e_summed: `modulation + e` where the caller has already
-        formed it (the model does so for all blocks in one launch)."""
+        formed it (the model does so for all blocks in one launch).  xn: norm1 + modulation of x where the block before
+        has already produced it; next_mod = (scale, shift) of the block that follows: the block then returns
+        (x, norm1 + modulation of x for that block), formed in the pass that adds the FFN's gated output (the same
+        values with one read and one write of x fewer per layer)."""
         ops = self.ops
         e = (self.modulation.unsqueeze(1) + e if e_summed is None else e_summed).chunk(6, dim=2)
-        y = self.self_attn(ops.ln_modulate(x, e[1], e[0], self.eps), grid, kv_cache, current_start)
+        y = self.self_attn(ops.ln_modulate(x, e[1], e[0], self.eps) if xn is None else xn, grid, kv_cache, current_start)
         if isinstance(self.norm3, nn.Identity):
             x = xn = ops.gate_residual(x, y, e[2])
         else:
             x, xn = ops.gate_residual_ln(x, y, e[2], self.eps, weight=self.norm3.weight, bias=self.norm3.bias)
         x, xn = ops.gate_residual_ln(x, self.cross_attn(xn, context, crossattn_cache), None, self.eps, scale=e[4], shift=e[3])
-        return ops.linear_gate_residual(x, ops.linear_gelu(xn, self.ffn[0]), self.ffn[2], e[5])
+        h = ops.linear_gelu(xn, self.ffn[0])
+        if next_mod is None:
+            return ops.linear_gate_residual(x, h, self.ffn[2], e[5])
+        if getattr(ops, "own_gemm", False):
+            x = ops.linear_gate_residual(x, h, self.ffn[2], e[5])
+            return x, ops.ln_modulate(x, next_mod[0], next_mod[1], self.eps)
+        return ops.gate_residual_ln(x, self.ffn[2](h), e[5], self.eps, scale=next_mod[0], shift=next_mod[1])
 
 
 class CausalHead(nn.Module):
@@ -395,6 +404,7 @@ WAN_CONFIGS = {
 
 
 class CausalWanModel(nn.Module):
+    fuse_next_norm = True     # block i also forms block i + 1's norm1 + modulation (same values, one pass over x fewer)
 
     def __init__(self, patch_size=(1, 2, 2), text_len=512, in_dim=16, dim=2048, ffn_dim=8192, freq_dim=256,
                  text_dim=4096, out_dim=16, num_heads=16, num_layers=32, local_attn_size=-1, sink_size=0, qk_norm=True,
@@ -478,8 +488,17 @@ class CausalWanModel(nn.Module):
                                                             context.shape[2])], dim=1)
         context = self.text_embedding(context)
         e_all = self._summed_modulations(e0)
-        for i, block in enumerate(self.blocks):
-            x = block(x, e0, grid, context, kv_cache[i], crossattn_cache[i] if crossattn_cache is not None else None,
-                      current_start, **({} if e_all is None else {"e_summed": e_all[i]}))
+        if e_all is None:
+            for i, block in enumerate(self.blocks):
+                x = block(x, e0, grid, context, kv_cache[i], crossattn_cache[i] if crossattn_cache is not None else None,
+                          current_start)
+        else:
+            # every block but the last also forms the next block's normalised, modulated input
+            xn, last = None, len(self.blocks) - 1
+            for i, block in enumerate(self.blocks):
+                nxt = None if i == last or not self.fuse_next_norm else (e_all[i + 1][:, :, 1:2], e_all[i + 1][:, :, 0:1])
+                r = block(x, e0, grid, context, kv_cache[i], crossattn_cache[i] if crossattn_cache is not None else None,
+                          current_start, e_summed=e_all[i], xn=xn, next_mod=nxt)
+                x, xn = r if nxt is not None else (r, None)
         x = self.head(x, e.unflatten(0, t.shape).unsqueeze(2))
         return self.unpatchify(x.flatten(1, 2) if x.dim() == 4 else x, grid)

@@ -163,3 +163,32 @@ def test_model_sums_all_modulations_at_once_with_the_same_result():
         m.blocks[1].modulation.add_(1.0)
         assert torch.equal(m._summed_modulations(e0)[1], m.blocks[1].modulation.unsqueeze(1) + e0)
     assert m._summed_modulations(e0) is None                     # gradients wanted: every block adds its own
+
+
+def test_model_forms_the_next_blocks_input_in_the_block_before_with_the_same_result():
+    """The model hands block i the modulation of block i + 1, gets block i + 1's normalised input back and passes it
+    on; the per-block route (every block normalises its own input) gives the same output and the same caches."""
+    torch.manual_seed(12)
+    m = cm.CausalWanModel(dim=32, ffn_dim=64, num_heads=2, num_layers=3, in_dim=4, out_dim=4, freq_dim=16, text_dim=8, text_len=4,
+                          frame_hw=(2, 3), total_seq_len=2 * 6, attention_flags=dict(disable_monarch=True), ops=OracleOps()).eval()
+    m.init_weights(zero_head=False)
+    g = torch.Generator().manual_seed(13)
+    x, ctx, t = torch.randn(1, 4, 2, 4, 6, generator=g), torch.randn(1, 4, 8, generator=g), torch.tensor([[500.0, 250.0]])
+
+    def run(model):
+        kv = [{"k": torch.zeros(1, 12, 2, 16), "v": torch.zeros(1, 12, 2, 16), "global_end_index": torch.tensor([0]),
+               "local_end_index": torch.tensor([0])} for _ in range(3)]
+        ca = [{"k": None, "v": None, "is_init": False} for _ in range(3)]
+        return model(x, t, ctx, kv_cache=kv, crossattn_cache=ca, current_start=0), kv
+
+    seen = []
+    for b in m.blocks:
+        b.register_forward_hook(lambda mod, args, kwargs, out: seen.append(kwargs.get("next_mod") is not None), with_kwargs=True)
+    fused, kv_f = run(m)
+    assert seen == [True, True, False]
+    m._summed_modulations = lambda e0: None
+    plain, kv_p = run(m)
+    assert seen[3:] == [False, False, False]
+    assert torch.equal(fused, plain)
+    for a, b in zip(kv_f, kv_p):
+        assert torch.equal(a["k"], b["k"]) and torch.equal(a["v"], b["v"])

@@ -118,3 +118,28 @@ def test_pipeline_decodes_each_chunk_as_it_is_finished():
     seen = []
     pipe.inference(noise, ctx, vae=vae, on_pixels=lambda i, px: seen.append((i, px.shape[1])))
     assert seen == [(0, 9), (1, 12)]
+
+
+def test_next_blocks_input_formed_in_the_block_before_changes_nothing():
+    """The model lets block i form block i + 1's normalised, modulated input in the pass that adds its FFN output.
+    Same kernels' arithmetic on the same rounded rows: output and caches equal those of the per-block route, bit for bit."""
+    _, dev_gen = _pair(use_framewise=True)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(1, 3, 16, 12, 104, generator=g).to(torch.bfloat16).to("cuda:0")
+    ctx = torch.randn(1, 16, 64, generator=g).to(torch.bfloat16).to("cuda:0")
+    t = torch.full((1, 3), 500.0, device="cuda:0")
+
+    def run():
+        kv = [{"k": torch.zeros(1, 6 * 312, 2, 128, dtype=torch.bfloat16, device="cuda:0"),
+               "v": torch.zeros(1, 6 * 312, 2, 128, dtype=torch.bfloat16, device="cuda:0"),
+               "global_end_index": torch.tensor([0], device="cuda:0"), "local_end_index": torch.tensor([0], device="cuda:0")}
+              for _ in range(2)]
+        ca = [{"k": None, "v": None, "is_init": False} for _ in range(2)]
+        return dev_gen(x, {"prompt_embeds": ctx}, t, kv, ca, 0)[0], kv
+
+    fused, kv_f = run()
+    dev_gen.model._summed_modulations = lambda e0: None
+    plain, kv_p = run()
+    assert torch.equal(fused, plain)
+    for a, b in zip(kv_f, kv_p):
+        assert torch.equal(a["k"], b["k"]) and torch.equal(a["v"], b["v"])
