@@ -146,7 +146,7 @@ def sinusoidal_embedding_1d(dim, position):
     """model.py:407-417: cat[cos, sin] of position * 10000^(-m/half), float64."""
     half = dim // 2
     position = position.type(torch.float64)
-    sinusoid = torch.outer(position, torch.pow(10000, -torch.arange(half).to(position).div(half)))
+    sinusoid = torch.outer(position, torch.pow(10000, -torch.arange(half, dtype=position.dtype, device=position.device).div(half)))
     return torch.cat([torch.cos(sinusoid), torch.sin(sinusoid)], dim=1)
 
 

@@ -55,9 +55,13 @@ class WanDiffusionWrapper(nn.Module):
 
     def _convert_flow_pred_to_x0(self, flow_pred, xt, timestep):
         """x0 = x_t - sigma_t * flow in float64 (wan_wrapper.py:172-196)."""
-        dt = flow_pred.dtype
-        sig = self.scheduler.sigmas.double().to(flow_pred.device)
-        ts = self.scheduler.timesteps.double().to(flow_pred.device)
+        dt, sch = flow_pred.dtype, self.scheduler
+        tab = getattr(self, "_x0_tables", None)
+        if tab is None or tab[0] is not sch.sigmas or tab[1] != flow_pred.device:
+            # float64 copies of the tables on the device, made once: no host copy per pass
+            self._x0_tables = tab = (sch.sigmas, flow_pred.device, sch.sigmas.double().to(flow_pred.device),
+                                     sch.timesteps.double().to(flow_pred.device))
+        sig, ts = tab[2], tab[3]
         idx = torch.argmin((ts.unsqueeze(0) - timestep.double().unsqueeze(1)).abs(), dim=1)
         return (xt.double() - sig[idx].reshape(-1, 1, 1, 1) * flow_pred.double()).to(dt)
 

@@ -46,3 +46,46 @@ def test_kv_cache_op_replays_from_a_graph(op):
         torch.cuda.synchronize()
         assert torch.equal(got, want), f"replay {it}"
         assert torch.equal(kc, kc2) and torch.equal(vc, vc2)
+
+
+def test_a_whole_model_pass_replays_from_a_graph():
+    """One pass of the causal DiT (2 layers, every operator of the block, time embedding, head) recorded once and
+    replayed with new latents and timesteps at the same addresses: every replay equals the eager pass on those inputs,
+    with eager work and synchronisation between the replays.  Nothing in the pass copies from the host or waits for
+    the device."""
+    cm, pl = sfa.causal_model, sfa.pipeline
+    torch.manual_seed(0)
+    model = cm.CausalWanModel(attention_flags=dict(use_framewise=True), dim=256, ffn_dim=512, num_heads=2, num_layers=2,
+                              text_dim=64, text_len=16, frame_hw=(6, 52), total_seq_len=6 * 6 * 52)
+    model.init_weights(zero_head=False)
+    gen = pl.WanDiffusionWrapper(model.to(torch.bfloat16).eval().to(DEV))
+    g = torch.Generator().manual_seed(7)
+    new_x = lambda: torch.randn(1, 3, 16, 12, 104, generator=g).to(torch.bfloat16).to(DEV)
+    x, t = new_x(), torch.full((1, 3), 750, device=DEV, dtype=torch.int64)
+    cond = {"prompt_embeds": torch.randn(1, 16, 64, generator=g).to(torch.bfloat16).to(DEV)}
+    kv = [{"k": torch.zeros(1, 6 * 312, 2, 128, dtype=torch.bfloat16, device=DEV),
+           "v": torch.zeros(1, 6 * 312, 2, 128, dtype=torch.bfloat16, device=DEV),
+           "global_end_index": torch.tensor([0], device=DEV), "local_end_index": torch.tensor([0], device=DEV)} for _ in range(2)]
+    ca = [{"k": None, "v": None, "is_init": False} for _ in range(2)]
+    gen(new_x(), cond, t, kv, ca, 0)                                  # the first chunk, eager: fills the cache's first half
+    call = lambda: gen(x, cond, t, kv, ca, 3 * 312)[1]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = call()
+    for it, step in enumerate((1000, 500, 250, 0)):
+        x.copy_(new_x())
+        t.fill_(step)
+        graph.replay()
+        torch.cuda.synchronize()
+        got, k_got = out.clone(), [c["k"].clone() for c in kv]
+        want = call()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {it}"
+        assert all(torch.equal(a, c["k"]) for a, c in zip(k_got, kv))
