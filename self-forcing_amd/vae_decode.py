@@ -225,8 +225,14 @@ class AttentionBlock(nn.Module):
     def forward_cl(self, x, state=None):
         t, h, w, c = x.shape
         qkv = F.linear(self.norm.forward_cl(x).reshape(t, h * w, c), self.to_qkv.weight.view(3 * c, c), self.to_qkv.bias)
-        q, k, v = (u.unsqueeze(1) for u in qkv.split(c, dim=-1))                           # [t, 1, hw, c]
-        o = F.scaled_dot_product_attention(q, k, v)[:, 0]
+        q, k, v = qkv.split(c, dim=-1)                                                     # [t, hw, c] each
+        if x.is_cuda and x.dtype in (torch.bfloat16, torch.float16):
+            # head_dim 384 is outside the fused attention kernels of the libraries: two plain matrix products with the
+            # logits kept in fp32 (6240 x 6240 per frame) and the softmax between them
+            p = torch.bmm(q, k.transpose(1, 2), out_dtype=torch.float32).mul_(c ** -0.5)
+            o = torch.bmm(torch.softmax(p, dim=-1, out=p).to(x.dtype), v)
+        else:
+            o = F.scaled_dot_product_attention(q.unsqueeze(1), k.unsqueeze(1), v.unsqueeze(1))[:, 0]
         return x + F.linear(o, self.proj.weight.view(c, c), self.proj.bias).reshape(t, h, w, c)
 
 
