@@ -49,6 +49,27 @@ def norm_act(x, gamma, act, out=None):
     return out
 
 
+_PADDED = {}
+
+
+def _padded(shape, cin, dtype, device):
+    """A zero-bordered input buffer of `shape`, one per (device, stream, shape, real input channels, dtype), kept for the life of the
+    process (release_padded() drops them): the kernel never writes its input, every call overwrites the interior, so
+    border, channel padding and anything else a call does not write stay zero and no call after the first fills the
+    buffer.  Calls that share a buffer are ordered by their stream.  Returns (buffer, it is new)."""
+    key = (device, torch.cuda.current_stream(device).cuda_stream, tuple(shape), cin, dtype)
+    buf = _PADDED.get(key)
+    if buf is not None:
+        return buf, False
+    buf = _PADDED[key] = torch.zeros(shape, dtype=dtype, device=device)
+    return buf, True
+
+
+def release_padded():
+    """Drop the cached padded input buffers (they are rebuilt on demand)."""
+    _PADDED.clear()
+
+
 def conv_cl(x, conv, history=None, up2x=False, norm=None, want_tail=False, res=None):
     """x [T, H, W, Cin] -> [T, H', W', Cout] for a causal Conv3d (kt - 1 frames of `history`, zeros where it is
     shorter) or a Conv2d applied per frame; with up2x the nearest x2 upsampling in front of a 3x3 Conv2d is folded
@@ -65,10 +86,12 @@ def conv_cl(x, conv, history=None, up2x=False, norm=None, want_tail=False, res=N
     if past == 0 and pad == 0 and cin_p == cin and x.is_contiguous() and norm is None:
         xp = x
     else:
-        xp = torch.zeros(T + past, H + 2 * pad, W + 2 * pad, cin_p, dtype=x.dtype, device=x.device)
-        if history is not None and past > 0:
-            n = min(history.shape[0], past)
+        xp, new = _padded((T + past, H + 2 * pad, W + 2 * pad, cin_p), cin, x.dtype, x.device)
+        n = min(history.shape[0], past) if history is not None else 0
+        if n > 0:
             xp[past - n:past, pad:pad + H, pad:pad + W, :cin] = history[-n:]
+        if n < past and not new:
+            xp[:past - n].zero_()                   # no history yet: these frames hold an earlier call's
         inner = xp[past:, pad:pad + H, pad:pad + W, :cin]
         if norm is None:
             inner.copy_(x)

@@ -98,3 +98,29 @@ def test_norm_act_matches_fp32(C_, act, dt):
     tol = (2.0 ** -8 if dt == torch.bfloat16 else 2.0 ** -11) * max(1.0, ref.abs().max().item()) * 1.01
     assert (out.float() - ref).abs().max().item() <= tol
     assert big[:2].abs().max() == 0 and big[:, 0].abs().max() == 0 and big[..., C_:].abs().max() == 0   # nothing outside the view
+
+
+def test_conv_cl_reuses_its_padded_input_buffer_without_stale_values():
+    """Calls of one padded shape share one zero-bordered buffer that is filled once.  A call without history after a
+    call with history (a new stream after an old one), and a call with fewer real input channels in the same padded
+    shape, must not see what the earlier call left there: each result equals the one from a fresh buffer, bit for bit."""
+    torch.manual_seed(3)
+    conv = nn.Conv3d(96, 96, 3).cuda().to(torch.bfloat16)
+    conv16 = nn.Conv3d(80, 96, 3).cuda().to(torch.bfloat16)           # 80 real channels in the same 96-channel padded shape
+    x = torch.randn(2, 9, 11, 96, device="cuda").to(torch.bfloat16)
+    h = torch.randn(2, 9, 11, 96, device="cuda").to(torch.bfloat16)
+    co.release_padded()
+    fresh_none = co.conv_cl(x, conv, None)
+    co.release_padded()
+    fresh_one = co.conv_cl(x, conv, h[:1])
+    co.release_padded()
+    fresh_16 = co.conv_cl(x[..., :80].contiguous(), conv16, None)
+    co.release_padded()
+    with_h, tail = co.conv_cl(x, conv, h, want_tail=True)
+    assert torch.equal(tail, x)                                        # the last two frames of (history + input)
+    assert len(co._PADDED) == 1
+    assert torch.equal(co.conv_cl(x, conv, h[:1]), fresh_one)          # one history frame: the other one is zero again
+    assert torch.equal(co.conv_cl(x, conv, None), fresh_none)
+    assert torch.equal(co.conv_cl(x[..., :80].contiguous(), conv16, None), fresh_16)
+    assert len(co._PADDED) == 2                                        # fewer real channels: a buffer of its own
+    assert not torch.equal(with_h, fresh_none)
