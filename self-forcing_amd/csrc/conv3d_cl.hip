@@ -70,8 +70,16 @@ __global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
     const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave % WN, wm = wave / WN;
-    const int64_t v0 = (int64_t)blockIdx.x * kVox;
-    const int co0 = blockIdx.y * kCo;
+    // consecutive workgroup ids go to the 8 XCDs in turn: give each XCD a contiguous range of voxel tiles, so that the
+    // input rows that neighbouring tiles share (taps one row up and down) meet in one L2
+    // and the channel blocks of one voxel tile follow each other within the XCD
+    const int ny = (p.Cout_pad + kCo - 1) / kCo;
+    const int per_xcd = (int)gridDim.x / 8;               // the grid is a multiple of 8 long
+    const int seq = (int)(blockIdx.x >> 3);
+    const int tile = (int)(blockIdx.x & 7) * (per_xcd / ny) + seq / ny;
+    if ((int64_t)tile * kVox >= p.voxels) return;
+    const int64_t v0 = (int64_t)tile * kVox;
+    const int co0 = (seq % ny) * kCo;
 
     // ---- what this lane stages: for each of the wave's row groups one 16-byte chunk of one row
     // lane -> (line, quarter, chunk) of the group's 1 KB; the row sitting in that quarter is quarter ^ line
@@ -242,7 +250,8 @@ template <class E, int CB, int WN>
 int launch_cfg(const ConvArgs& a, hipStream_t st) {
     constexpr int kVox = 64 * (4 / WN), kCo = 32 * CB * WN, kCoRows = (kCo + 63) / 64 * 64;
     constexpr int ldsb = 2 * (kCoRows + kVox) * kRowBytes;
-    dim3 grid((unsigned)((a.voxels + kVox - 1) / kVox), (unsigned)((a.Cout_pad + kCo - 1) / kCo));
+    const unsigned tiles = (unsigned)((a.voxels + kVox - 1) / kVox);
+    dim3 grid((tiles + 7) / 8 * 8 * (unsigned)((a.Cout_pad + kCo - 1) / kCo));
     if (a.up2x) hipLaunchKernelGGL((conv3d_cl_kernel<E, CB, WN, true>), grid, dim3(256), ldsb, st, a);
     else hipLaunchKernelGGL((conv3d_cl_kernel<E, CB, WN, false>), grid, dim3(256), ldsb, st, a);
     hipError_t e = hipGetLastError();
