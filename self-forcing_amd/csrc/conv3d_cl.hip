@@ -52,10 +52,68 @@ __device__ __forceinline__ void cv_load_lds16(const char* base, uint32_t off, ui
 }
 __device__ __forceinline__ void cv_wait_stage() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Epilogue of one voxel (t, h, w) of a lane: residual and bias added in fp32, one rounding, CB blocks of 32 channels
+// from channel cbase0 on.  Lane half hf of block cb holds channels 8 g + 4 hf + (e & 3) in acc[cb][vb][4 g + (e & 3)].
+template <class E, int CB>
+__device__ __forceinline__ void store_voxel(const ConvArgs& p, f32x16 (&acc)[CB][2], int vb, bool vok, int t, int h, int w,
+                                            int cbase0, int hf) {
+    const int64_t yoff = ((int64_t)t * p.ys_t + (int64_t)h * p.ys_h + (int64_t)w * p.ys_w) * 2;
+    char* yrow = p.y + yoff;
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        const int cbase = cbase0 + 32 * cb;
+        if (p.res != nullptr && vok) {
+            // the block of the voxel that this lane completes: channels 8 g + 4 hf + 0..3
+            const char* rrow = p.res + yoff;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int co = cbase + 8 * g + 4 * hf;
+                if (co + 4 <= p.Cout) {
+                    const u32x2 rv = *(const u32x2*)(rrow + co * 2);
+                    acc[cb][vb][4 * g + 0] += E::to_float((uint16_t)(rv.x & 0xffffu));
+                    acc[cb][vb][4 * g + 1] += E::to_float((uint16_t)(rv.x >> 16));
+                    acc[cb][vb][4 * g + 2] += E::to_float((uint16_t)(rv.y & 0xffffu));
+                    acc[cb][vb][4 * g + 3] += E::to_float((uint16_t)(rv.y >> 16));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (co + e < p.Cout) acc[cb][vb][4 * g + e] += E::to_float(*(const uint16_t*)(rrow + (co + e) * 2));
+                }
+            }
+        }
+        if (p.bias != nullptr) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int co = cbase + 8 * (e >> 2) + 4 * hf + (e & 3);
+                acc[cb][vb][e] += co < p.Cout ? p.bias[co] : 0.f;
+            }
+        }
+        if (cbase + 32 <= p.Cout) {
+#pragma unroll
+            for (int gp = 0; gp < 2; ++gp) {
+                const int g0 = 2 * gp, g1 = 2 * gp + 1;
+                auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[cb][vb][4 * g0 + 0], acc[cb][vb][4 * g0 + 1]),
+                                                           pack2<E>(acc[cb][vb][4 * g1 + 0], acc[cb][vb][4 * g1 + 1]), false, false);
+                auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[cb][vb][4 * g0 + 2], acc[cb][vb][4 * g0 + 3]),
+                                                           pack2<E>(acc[cb][vb][4 * g1 + 2], acc[cb][vb][4 * g1 + 3]), false, false);
+                u32x4 o = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
+                if (vok) *(u32x4*)(yrow + (cbase + 16 * gp + 8 * hf) * 2) = o;
+            }
+        } else {
+            // a partial last block (e.g. the 3 channels of the decoder's head): element stores
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int co = cbase + 8 * (e >> 2) + 4 * hf + (e & 3);
+                if (vok && co < p.Cout) *(uint16_t*)(yrow + co * 2) = E::from_float(acc[cb][vb][e]);
+            }
+        }
+    }
+}
+
 // CB: 32-channel blocks per wave; WN: waves along the output channels (the other 4 / WN waves split the voxels);
 // UP: the input is at half resolution (nearest x2 upsampling folded into the addresses).
 template <class E, int CB, int WN, bool UP>
-__global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
+__global__ __launch_bounds__(256, 2) void conv3d_cl_kernel(ConvArgs p) {
     constexpr int WM = 4 / WN;
     constexpr int kVox = 64 * WM;                         // voxels per workgroup
     constexpr int kCo = 32 * CB * WN;                     // output channels per workgroup
@@ -192,58 +250,157 @@ __global__ __launch_bounds__(256) void conv3d_cl_kernel(ConvArgs p) {
         const int64_t vc = vok ? v : 0;
         const int w = (int)(vc % p.W);
         const int64_t r = vc / p.W;
-        const int h = (int)(r % p.H), t = (int)(r / p.H);
-        char* yrow = p.y + (t * p.ys_t + h * p.ys_h + w * p.ys_w) * 2;
+        store_voxel<E, CB>(p, acc, vb, vok, (int)(r / p.H), (int)(r % p.H), w, co0 + 32 * CB * wn, hf);
+    }
+}
+
+// The 3x3 spatial kernels on a contiguous padded input (x_stride = {(H + 2)(W + 2) Cin, (W + 2) Cin, Cin}): outputs are
+// computed for every position u of the padded grid from its first to its last interior voxel (the two border columns
+// between rows and the border rows between frames come out as garbage and are not stored: 0.7 % more work at 480 x
+// 832), so that tap (dt, dh, dw) of position u is input row u + dt FS + (dh - 1) WP + (dw - 1) for all u alike.  A
+// stage then holds one run of 258 consecutive input rows and the weights of the three taps of a kernel row: the
+// three taps read the run at row offsets 0, 1, 2.  Per matrix instruction 3.9 staged rows instead of 7.3: the kernel
+// above is bound by what the L2s deliver to the compute units.  One workgroup: 256 positions x CB x 32 channels.
+template <class E, int CB>
+__global__ __launch_bounds__(256, 2) void conv3d_row3_kernel(ConvArgs p) {
+    constexpr int kVox = 256, kCo = 32 * CB;
+    constexpr int kWRows = 3 * kCo;                       // weights of the three taps
+    constexpr int kNWG = kWRows / 16, kNXG = 17;          // 16-row groups: weights, input run (258 rows -> 272)
+    constexpr int kNG = kNWG + kNXG;
+    constexpr int kPer = (kNG + 3) / 4;                   // groups a wave stages (the last one may repeat group kNG - 1)
+    constexpr int kStage = kNG * 1024;
+    extern __shared__ __attribute__((aligned(256))) char lds[];
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
+
+    const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int WP = p.W + 2;
+    const int64_t FS = (int64_t)(p.H + 2) * WP;
+    const int64_t u_first = WP + 1, u_last = (int64_t)(p.T - 1) * FS + (int64_t)p.H * WP + p.W;
+    const int ny = p.Cout_pad / kCo;
+    const int per_xcd = (int)gridDim.x / 8;               // as in conv3d_cl_kernel
+    const int seq = (int)(blockIdx.x >> 3);
+    const int64_t u0 = u_first + ((int64_t)(blockIdx.x & 7) * (per_xcd / ny) + seq / ny) * kVox;
+    if (u0 > u_last) return;
+    const int co0 = (seq % ny) * kCo;
+
+    const int g_line = lane >> 4, g_q = (lane >> 2) & 3, g_c = lane & 3;
+    const int g_row = g_line * 4 + (g_q ^ g_line);
+    uint32_t src[kPer];
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            const int cbase = co0 + 32 * (cb + CB * wn);
-            if (p.res != nullptr && vok) {
-                // the block of the voxel that this lane completes: channels 8 g + 4 hf + 0..3
-                const char* rrow = p.res + (t * p.ys_t + h * p.ys_h + w * p.ys_w) * 2;
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int co = cbase + 8 * g + 4 * hf;
-                    if (co + 4 <= p.Cout) {
-                        const u32x2 rv = *(const u32x2*)(rrow + co * 2);
-                        acc[cb][vb][4 * g + 0] += E::to_float((uint16_t)(rv.x & 0xffffu));
-                        acc[cb][vb][4 * g + 1] += E::to_float((uint16_t)(rv.x >> 16));
-                        acc[cb][vb][4 * g + 2] += E::to_float((uint16_t)(rv.y & 0xffffu));
-                        acc[cb][vb][4 * g + 3] += E::to_float((uint16_t)(rv.y >> 16));
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (co + e < p.Cout) acc[cb][vb][4 * g + e] += E::to_float(*(const uint16_t*)(rrow + (co + e) * 2));
-                    }
-                }
-            }
-            if (p.bias != nullptr) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int co = cbase + 8 * (e >> 2) + 4 * hf + (e & 3);
-                    acc[cb][vb][e] += co < p.Cout ? p.bias[co] : 0.f;
-                }
-            }
-            if (cbase + 32 <= p.Cout) {
-#pragma unroll
-                for (int gp = 0; gp < 2; ++gp) {
-                    const int g0 = 2 * gp, g1 = 2 * gp + 1;
-                    auto rx = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[cb][vb][4 * g0 + 0], acc[cb][vb][4 * g0 + 1]),
-                                                               pack2<E>(acc[cb][vb][4 * g1 + 0], acc[cb][vb][4 * g1 + 1]), false, false);
-                    auto ry = __builtin_amdgcn_permlane32_swap(pack2<E>(acc[cb][vb][4 * g0 + 2], acc[cb][vb][4 * g0 + 3]),
-                                                               pack2<E>(acc[cb][vb][4 * g1 + 2], acc[cb][vb][4 * g1 + 3]), false, false);
-                    u32x4 o = {(uint32_t)rx[0], (uint32_t)ry[0], (uint32_t)rx[1], (uint32_t)ry[1]};
-                    if (vok) *(u32x4*)(yrow + (cbase + 16 * gp + 8 * hf) * 2) = o;
-                }
-            } else {
-                // a partial last block (e.g. the 3 channels of the decoder's head): element stores
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int co = cbase + 8 * (e >> 2) + 4 * hf + (e & 3);
-                    if (vok && co < p.Cout) *(uint16_t*)(yrow + co * 2) = E::from_float(acc[cb][vb][e]);
-                }
-            }
+    for (int i = 0; i < kPer; ++i) {
+        const int g = min(wave + 4 * i, kNG - 1);
+        const int j = g * 16 + g_row;
+        if (g < kNWG) {
+            const int dw = j / kCo, r = j - dw * kCo;
+            src[i] = (uint32_t)(((int64_t)dw * p.Cout_pad + co0 + r) * p.Cin * 2 + g_c * 16);
+        } else {
+            // staged row s is the input row of tap (dt = 0, dh = 0, dw = 0) of position u0 + s; rows past the last
+            // position's taps repeat the last one
+            const int64_t u = min(u0 + (j - kWRows), u_last + 2) - WP - 1;
+            src[i] = (uint32_t)(u * p.Cin * 2 + g_c * 16);
         }
     }
+
+    const int cin_steps = p.Cin / kKC;
+    const int nstage = p.kt * 3 * cin_steps;
+    const char* f_w = p.wt;
+    const char* f_x = p.x;
+    const int64_t w_next_row = 3 * (int64_t)p.Cout_pad * p.Cin * 2 - (int64_t)p.Cin * 2;      // next kernel row: three taps on
+    const int64_t x_next_row = ((int64_t)WP - 1) * p.Cin * 2;
+    const int64_t x_next_frame = (FS - 3 * (int64_t)WP) * p.Cin * 2;
+    int f_cs = 0, f_dh = 0;
+    auto stage = [&](uint32_t buf) {
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            const int g = min(wave + 4 * i, kNG - 1);
+            cv_load_lds16(g < kNWG ? f_w : f_x, src[i], lds0 + buf + (uint32_t)g * 1024);
+        }
+        f_w += kKC * 2;
+        f_x += kKC * 2;
+        if (++f_cs == cin_steps) {
+            f_cs = 0;
+            f_w += w_next_row;
+            f_x += x_next_row;
+            if (++f_dh == 3) {
+                f_dh = 0;
+                f_x += x_next_frame;
+            }
+        }
+    };
+
+    f32x16 acc[CB][2];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int vb = 0; vb < 2; ++vb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[cb][vb][v] = 0.f;
+
+    uint32_t a_off[CB], b_off[2][3];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) a_off[cb] = tile_off(32 * cb + m, hf);
+#pragma unroll
+    for (int vb = 0; vb < 2; ++vb)
+#pragma unroll
+        for (int dw = 0; dw < 3; ++dw) b_off[vb][dw] = tile_off(kWRows + 64 * wave + 32 * vb + m + dw, hf);
+
+    stage(0);
+    for (int s = 0; s < nstage; ++s) {
+        const uint32_t buf = (uint32_t)(s & 1) * kStage;
+        cv_wait_stage();
+        if (s + 1 < nstage) stage(buf ^ kStage);
+#pragma unroll
+        for (int dw = 0; dw < 3; ++dw)
+#pragma unroll
+            for (int ks = 0; ks < kKC / 16; ++ks) {
+                u32x4 a[CB], b[2];
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) a[cb] = *(const u32x4*)(lds + buf + a_off[cb] + dw * (kCo * kRowBytes) + ks * 32);
+#pragma unroll
+                for (int vb = 0; vb < 2; ++vb) b[vb] = *(const u32x4*)(lds + buf + b_off[vb][dw] + ks * 32);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                    for (int vb = 0; vb < 2; ++vb) acc[cb][vb] = E::mfma32(a[cb], b[vb], acc[cb][vb]);
+            }
+    }
+
+#pragma unroll
+    for (int vb = 0; vb < 2; ++vb) {
+        const int64_t u = u0 + 64 * wave + 32 * vb + m;
+        const int64_t uc = min(u, u_last);
+        const int t = (int)(uc / FS);
+        const int rem = (int)(uc - (int64_t)t * FS);
+        const int hp = rem / WP, wp = rem - hp * WP;
+        const bool vok = u <= u_last && hp >= 1 && hp <= p.H && wp >= 1 && wp <= p.W;
+        store_voxel<E, CB>(p, acc, vb, vok, vok ? t : 0, vok ? hp - 1 : 0, vok ? wp - 1 : 0, co0, hf);
+    }
+}
+
+template <class E, int CB>
+int launch_row3(const ConvArgs& a, hipStream_t st) {
+    constexpr int ldsb = 2 * (3 * 32 * CB / 16 + 17) * 1024;
+    static bool configured = false;                       // per instantiation; racing callers set the same value
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)conv3d_row3_kernel<E, CB>, hipFuncAttributeMaxDynamicSharedMemorySize, ldsb);
+        if (e != hipSuccess) {
+            set_error("sfm_conv3d_cl: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+            return SFM_ERR_HIP;
+        }
+        configured = true;
+    }
+    const int64_t WP = a.W + 2, FS = (int64_t)(a.H + 2) * WP;
+    const int64_t positions = (int64_t)(a.T - 1) * FS + (int64_t)(a.H - 1) * WP + a.W;     // first to last interior voxel
+    const unsigned tiles = (unsigned)((positions + 255) / 256);
+    hipLaunchKernelGGL((conv3d_row3_kernel<E, CB>), dim3((tiles + 7) / 8 * 8 * (unsigned)(a.Cout_pad / (32 * CB))), dim3(256), ldsb,
+                       st, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_error("sfm_conv3d_cl: launch failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    return SFM_OK;
 }
 
 template <class E, int CB, int WN>
@@ -264,6 +421,10 @@ int launch_cfg(const ConvArgs& a, hipStream_t st) {
 
 template <class E>
 int launch_dtype(const ConvArgs& a, hipStream_t st) {
+    const bool run = a.kh == 3 && !a.up2x && a.xs_w == a.Cin && a.xs_h == (int64_t)(a.W + 2) * a.Cin &&
+                     a.xs_t == (int64_t)(a.H + 2) * (a.W + 2) * a.Cin && 3 * (int64_t)a.Cout_pad * a.Cin * 2 < ((int64_t)1 << 32);
+    if (run && a.Cout_pad % 96 == 0) return launch_row3<E, 3>(a, st);
+    if (run && a.Cout_pad == 32) return launch_row3<E, 1>(a, st);
     if (a.Cout_pad % 192 == 0) return launch_cfg<E, 3, 2>(a, st);
     if (a.Cout_pad % 96 == 0) return launch_cfg<E, 3, 1>(a, st);
     return launch_cfg<E, 1, 1>(a, st);                    // Cout_pad a multiple of 32
