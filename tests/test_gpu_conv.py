@@ -124,3 +124,32 @@ def test_conv_cl_reuses_its_padded_input_buffer_without_stale_values():
     assert torch.equal(co.conv_cl(x[..., :80].contiguous(), conv16, None), fresh_16)
     assert len(co._PADDED) == 2                                        # fewer real channels: a buffer of its own
     assert not torch.equal(with_h, fresh_none)
+
+
+def test_strided_padded_input_takes_the_general_kernel_with_the_same_result():
+    """The 3x3 kernels run on a contiguous padded input as one run of rows per kernel row; a padded input that is a
+    view into a wider buffer goes through the general kernel.  Same convolution: the two agree to the rounding of the
+    result (the taps are summed in a different order)."""
+    import ctypes as C
+    from self_forcing_amd import lib as L
+    torch.manual_seed(5)
+    T, H, W, c = 3, 10, 13, 96
+    conv = nn.Conv3d(c, c, 3).cuda().to(torch.bfloat16)
+    x = torch.randn(T, H, W, c, device="cuda").to(torch.bfloat16)
+    h = torch.randn(2, H, W, c, device="cuda").to(torch.bfloat16)
+    want = co.conv_cl(x, conv, h)
+    wt, bias, kt, k, cout, cin, cin_p, cout_p = co.prepared(conv, x.dtype, x.device)
+    wide = torch.zeros(T + 2, H + 2, W + 6, c, device="cuda", dtype=torch.bfloat16)
+    xp = wide[:, :, 2:2 + W + 2]                                   # the padded input, rows W + 6 columns apart
+    xp[:2, 1:1 + H, 1:1 + W] = h
+    xp[2:, 1:1 + H, 1:1 + W] = x
+    y = torch.empty(T, H, W, c, device="cuda", dtype=torch.bfloat16)
+    d = L.ConvDesc()
+    d.dtype, d.T, d.H, d.W, d.Cin, d.Cout, d.Cout_pad, d.kt, d.kh, d.kw, d.up2x = L.SFM_BF16, T, H, W, c, c, cout_p, 3, 3, 3, 0
+    for i in range(3):
+        d.x_stride[i], d.y_stride[i] = xp.stride(i), y.stride(i)
+    L.check(L.load().sfm_conv3d_cl(C.byref(d), xp.data_ptr(), wt.data_ptr(), bias.data_ptr(), None, y.data_ptr(),
+                                   torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert (y.float() - want.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, want.float().abs().max().item())
+    assert not torch.equal(y, torch.zeros_like(y))
