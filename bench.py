@@ -417,6 +417,7 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="accepted for the profile commands; the 1 GiB device copies (known HBM traffic, for scaling rocprof "
                          "counters) always run")
+    ap.add_argument("--vae-only", action="store_true", help="the streaming VAE decode leg alone (profile runs)")
     ap.add_argument("--gemm-legs", action="store_true",
                     help="only the table of the block's GEMM shapes: hipBLASLt (+ tail kernel) against sfm_linear with the tail fused")
     ap.add_argument("--write-traffic", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
@@ -435,6 +436,9 @@ def main():
     torch.cuda.set_device(0)
     if args.gemm_legs:
         print(json.dumps({"metric": "block GEMM shapes, us per call", "gemm": gemm_legs(torch, sfa)}))
+        return
+    if args.vae_only:
+        print(json.dumps({"metric": "streaming VAE decode", "vae_decode": vae_decode_leg(torch, sfa)}))
         return
     entry, size, flags, what = ROLLOUTS[args.config]
     rec = {"metric": f"latent frames/s, causal Wan-{size} 480x832 bf16 (+ Monarch attn ms/call, MFMA %)",

@@ -11,7 +11,7 @@
 // GEMM view: M = output channels (A operand, rows of wt with ci contiguous), N = output voxels (B operand, rows of
 // xp), K = taps x input channels, walked one tap and 32 channels at a time.  Each K step stages 64-byte rows
 // (32 channels) of both operands straight into LDS (global_load_lds_dwordx4), four rows to a 256-byte line with
-// the rows of a line rotated by the line index so that operand reads are conflict-free; two stage buffers, one
+// the 16-byte chunks of a row rotated by the line index so that operand reads are conflict-free; two stage buffers, one
 // barrier per stage.  A wave owns CB x 32 output channels by 64 voxels; accumulators leave through the same
 // half-swap as the attention kernels (8 consecutive channels = 16 bytes per lane and voxel).
 
@@ -41,10 +41,12 @@ struct ConvArgs {
     int64_t voxels;           // T * H * W
 };
 
-// byte offset of chunk c (16 bytes) of row r in a tile of 64-byte rows
+// byte offset of chunk c (16 bytes) of row r in a tile of 64-byte rows: four rows to a 256-byte line, the chunks of a
+// row stored at position c ^ (line & 3).  The 16 lanes that one cycle of a ds_read_b128 serves read the same chunk of 16
+// consecutive rows, i.e. of four lines: the rotation puts them on 16 different 16-byte bank groups.
 __device__ __forceinline__ uint32_t tile_off(int r, int c) {
     const int line = r >> 2;
-    return (uint32_t)(line * 256 + (((r & 3) ^ (line & 3)) << 6) + (c << 4));
+    return (uint32_t)(line * 256 + ((r & 3) << 6) + ((c ^ (line & 3)) << 4));
 }
 
 __device__ __forceinline__ void cv_load_lds16(const char* base, uint32_t off, uint32_t lds_addr) {
@@ -141,8 +143,8 @@ __global__ __launch_bounds__(256, 2) void conv3d_cl_kernel(ConvArgs p) {
 
     // ---- what this lane stages: for each of the wave's row groups one 16-byte chunk of one row
     // lane -> (line, quarter, chunk) of the group's 1 KB; the row sitting in that quarter is quarter ^ line
-    const int g_line = lane >> 4, g_q = (lane >> 2) & 3, g_c = lane & 3;
-    const int g_row = g_line * 4 + (g_q ^ g_line);
+    // lane -> 16-byte slot of the group's 1 KB: line, row of the line, position; the chunk sitting there is position ^ line
+    const int g_line = lane >> 4, g_row = lane >> 2, g_c = (lane & 3) ^ g_line;
     uint32_t w_off[kWG];                                  // byte offset of the weight row (without tap and channel step)
     uint32_t x_off[kVG];                                  // byte offset of the voxel's first tap (with UP: of its frame only)
     int vh[kVG], vw[kVG];
@@ -217,11 +219,13 @@ __global__ __launch_bounds__(256, 2) void conv3d_cl_kernel(ConvArgs p) {
             for (int v = 0; v < 16; ++v) acc[cb][vb][v] = 0.f;
 
     // operand read offsets within a stage: row r0 + m, chunk 2 ks + hf
-    uint32_t a_off[CB], b_off[2];
+    // blocks of 32 rows keep a row's line & 3, so one offset per k-step serves all blocks of an operand
+    uint32_t a_off[2], b_off[2];
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb) a_off[cb] = tile_off(32 * (cb + CB * wn) + m, hf);
-#pragma unroll
-    for (int vb = 0; vb < 2; ++vb) b_off[vb] = tile_off(kCoRows + 64 * wm + 32 * vb + m, hf);
+    for (int ks = 0; ks < 2; ++ks) {
+        a_off[ks] = tile_off(32 * CB * wn + m, 2 * ks + hf);
+        b_off[ks] = tile_off(kCoRows + 64 * wm + m, 2 * ks + hf);
+    }
 
     stage(0);
     for (int s = 0; s < nstage; ++s) {
@@ -232,9 +236,9 @@ __global__ __launch_bounds__(256, 2) void conv3d_cl_kernel(ConvArgs p) {
         for (int ks = 0; ks < kKC / 16; ++ks) {
             u32x4 a[CB], b[2];
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) a[cb] = *(const u32x4*)(lds + buf + a_off[cb] + ks * 32);
+            for (int cb = 0; cb < CB; ++cb) a[cb] = *(const u32x4*)(lds + buf + a_off[ks] + cb * (32 * kRowBytes));
 #pragma unroll
-            for (int vb = 0; vb < 2; ++vb) b[vb] = *(const u32x4*)(lds + buf + b_off[vb] + ks * 32);
+            for (int vb = 0; vb < 2; ++vb) b[vb] = *(const u32x4*)(lds + buf + b_off[ks] + vb * (32 * kRowBytes));
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
@@ -284,8 +288,8 @@ __global__ __launch_bounds__(256, 2) void conv3d_row3_kernel(ConvArgs p) {
     if (u0 > u_last) return;
     const int co0 = (seq % ny) * kCo;
 
-    const int g_line = lane >> 4, g_q = (lane >> 2) & 3, g_c = lane & 3;
-    const int g_row = g_line * 4 + (g_q ^ g_line);
+    // lane -> 16-byte slot of the group's 1 KB: line, row of the line, position; the chunk sitting there is position ^ line
+    const int g_line = lane >> 4, g_row = lane >> 2, g_c = (lane & 3) ^ g_line;
     uint32_t src[kPer];
 #pragma unroll
     for (int i = 0; i < kPer; ++i) {
@@ -337,13 +341,15 @@ __global__ __launch_bounds__(256, 2) void conv3d_row3_kernel(ConvArgs p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[cb][vb][v] = 0.f;
 
-    uint32_t a_off[CB], b_off[2][3];
+    // blocks of 32 rows (and the weights of the next tap, kCo rows on) keep a row's line & 3: one offset per k-step
+    // for the weights, one per k-step and tap for the input rows
+    uint32_t a_off[2], b_off[3][2];
 #pragma unroll
-    for (int cb = 0; cb < CB; ++cb) a_off[cb] = tile_off(32 * cb + m, hf);
+    for (int ks = 0; ks < 2; ++ks) {
+        a_off[ks] = tile_off(m, 2 * ks + hf);
 #pragma unroll
-    for (int vb = 0; vb < 2; ++vb)
-#pragma unroll
-        for (int dw = 0; dw < 3; ++dw) b_off[vb][dw] = tile_off(kWRows + 64 * wave + 32 * vb + m + dw, hf);
+        for (int dw = 0; dw < 3; ++dw) b_off[dw][ks] = tile_off(kWRows + 64 * wave + m + dw, 2 * ks + hf);
+    }
 
     stage(0);
     for (int s = 0; s < nstage; ++s) {
@@ -356,9 +362,9 @@ __global__ __launch_bounds__(256, 2) void conv3d_row3_kernel(ConvArgs p) {
             for (int ks = 0; ks < kKC / 16; ++ks) {
                 u32x4 a[CB], b[2];
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb) a[cb] = *(const u32x4*)(lds + buf + a_off[cb] + dw * (kCo * kRowBytes) + ks * 32);
+                for (int cb = 0; cb < CB; ++cb) a[cb] = *(const u32x4*)(lds + buf + a_off[ks] + (dw * kCo + 32 * cb) * kRowBytes);
 #pragma unroll
-                for (int vb = 0; vb < 2; ++vb) b[vb] = *(const u32x4*)(lds + buf + b_off[vb][dw] + ks * 32);
+                for (int vb = 0; vb < 2; ++vb) b[vb] = *(const u32x4*)(lds + buf + b_off[dw][ks] + vb * (32 * kRowBytes));
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
