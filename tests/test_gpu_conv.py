@@ -153,3 +153,24 @@ def test_strided_padded_input_takes_the_general_kernel_with_the_same_result():
     torch.cuda.synchronize()
     assert (y.float() - want.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, want.float().abs().max().item())
     assert not torch.equal(y, torch.zeros_like(y))
+
+
+@pytest.mark.parametrize("cin,cout,T,H,W", [(96, 96, 12, 480, 832), (192, 192, 12, 240, 416), (96, 3, 12, 480, 832)])
+def test_conv_cl_at_the_decoders_full_sizes(cin, cout, T, H, W):
+    """The decoder's largest convolutions (1.1 GB of padded input, 18 840 voxel tiles over the 8 XCDs, the 3-channel
+    head) against torch's fp32 convolution of the same bf16 operands, every output element."""
+    torch.manual_seed(cin + cout)
+    conv = nn.Conv3d(cin, cout, 3).cuda().to(torch.bfloat16)
+    x = torch.randn(T, H, W, cin, device="cuda").to(torch.bfloat16)
+    h = torch.randn(2, H, W, cin, device="cuda").to(torch.bfloat16)
+    y = co.conv_cl(x, conv, h)
+    xf = torch.cat([h, x]).float().permute(3, 0, 1, 2).unsqueeze(0)
+    ref = F.conv3d(F.pad(xf, (1, 1, 1, 1, 0, 0)), conv.weight.float(), conv.bias.float())[0].permute(1, 2, 3, 0)
+    del xf
+    assert y.shape == ref.shape
+    tol = 2.0 ** -8 * max(1.0, ref.abs().max().item()) * 1.01
+    worst = 0.0
+    for t in range(T):                                  # frame by frame: no second full-size fp32 temporary
+        worst = max(worst, (y[t].float() - ref[t]).abs().max().item())
+    assert worst <= tol
+    co.release_padded()
