@@ -492,8 +492,71 @@ __global__ __launch_bounds__(256) void vae_norm_act_kernel(NormArgs p) {
     }
 }
 
+// The decoder's channel counts are 96, 192, 384 = 24 x {4, 8, 16}: three 16-byte chunks per lane, GL lanes per voxel,
+// every lane busy and three loads in flight per lane.
+template <class E, int GL>
+__global__ __launch_bounds__(256) void vae_norm_act3_kernel(NormArgs p) {
+    const int tid = threadIdx.x;
+    const int sub = tid % GL;
+    const int64_t v = (int64_t)blockIdx.x * (256 / GL) + tid / GL;
+    const bool active = v < p.voxels;
+    const int64_t vc = active ? v : p.voxels - 1;
+    const int w = (int)(vc % p.W);
+    const int64_t r = vc / p.W;
+    const int h = (int)(r % p.H), t = (int)(r / p.H);
+    const char* src = p.x + (t * p.xs_t + h * p.xs_h + w * p.xs_w) * 2;
+    u32x4 raw[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) raw[k] = *(const u32x4*)(src + (sub + k * GL) * 16);
+    float f[3][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < 3; ++k)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[k][2 * i] = E::to_float((uint16_t)(raw[k][i] & 0xffffu));
+            f[k][2 * i + 1] = E::to_float((uint16_t)(raw[k][i] >> 16));
+            ss += f[k][2 * i] * f[k][2 * i] + f[k][2 * i + 1] * f[k][2 * i + 1];
+        }
+#pragma unroll
+    for (int o = GL / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, GL);
+    const float inv = sqrtf((float)p.C) / fmaxf(sqrtf(ss), 1e-12f);
+    if (active) {
+        char* dst = p.y + (t * p.ys_t + h * p.ys_h + w * p.ys_w) * 2;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) {
+            const u32x4 g = *(const u32x4*)(p.gamma + (sub + k * GL) * 8);
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float a = f[k][2 * i] * inv * E::to_float((uint16_t)(g[i] & 0xffffu));
+                float b = f[k][2 * i + 1] * inv * E::to_float((uint16_t)(g[i] >> 16));
+                if (p.act) {
+                    a = a / (1.f + __expf(-a));
+                    b = b / (1.f + __expf(-b));
+                }
+                o[i] = pack2<E>(a, b);
+            }
+            *(u32x4*)(dst + (sub + k * GL) * 16) = o;
+        }
+    }
+}
+
 template <class E>
 int launch_norm(const NormArgs& a, hipStream_t st) {
+    const int gl3 = a.C % 24 == 0 ? a.C / 24 : 0;
+    if (gl3 == 4 || gl3 == 8 || gl3 == 16) {
+        const unsigned blocks = (unsigned)((a.voxels + 256 / gl3 - 1) / (256 / gl3));
+        if (gl3 == 4) hipLaunchKernelGGL((vae_norm_act3_kernel<E, 4>), dim3(blocks), dim3(256), 0, st, a);
+        else if (gl3 == 8) hipLaunchKernelGGL((vae_norm_act3_kernel<E, 8>), dim3(blocks), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((vae_norm_act3_kernel<E, 16>), dim3(blocks), dim3(256), 0, st, a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            set_error("sfm_vae_norm_act: launch failed: %s", hipGetErrorString(e));
+            return SFM_ERR_HIP;
+        }
+        return SFM_OK;
+    }
     const int lanes = a.C / 8;
     const int gl = lanes <= 16 ? 16 : lanes <= 32 ? 32 : 64;
     const unsigned blocks = (unsigned)((a.voxels + 256 / gl - 1) / (256 / gl));
