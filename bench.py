@@ -58,7 +58,7 @@ def measured_traffic():
 
 
 def write_traffic(fetch_csv, write_csv):
-    """Turns the counter_collection CSVs of two rocprofv3 runs of `bench.py --op-only --no-cpu-baseline --copy-probe`
+    """Turns the counter_collection CSVs of two rocprofv3 runs of `bench.py --op-only --skip-simt --no-cpu-baseline --copy-probe`
     (`--pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`; KiB per dispatch) into profiles/traffic.json.  Each counter is scaled
     by what it reads for the run's own 1 GiB device-to-device copies, whose traffic is known (1 GiB read, 1 GiB written)."""
     import collections
@@ -100,7 +100,7 @@ def write_traffic(fetch_csv, write_csv):
     dirty = subprocess.run(["git", "-C", ROOT, "status", "--porcelain", "--", "self-forcing_amd/csrc"], capture_output=True,
                            text=True).stdout.strip()
     rec = {"commit": (commit + ("+uncommitted kernel changes" if dirty else "")) or None,
-           "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -- python3 bench.py --op-only "
+           "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -- python3 bench.py --op-only --skip-simt "
                       "--no-cpu-baseline --copy-probe, then python bench.py --write-traffic FETCH.csv WRITE.csv",
            "copy_kernel": "__amd_rocclr_copyBuffer", "copy_dispatches": [n_f, n_w], "fetch_factor": f_fac,
            "write_factor": w_fac, "kernels": kernels}
