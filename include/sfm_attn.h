@@ -298,7 +298,10 @@ typedef struct sfm_conv_desc {
  * for a 3x3 spatial kernel, a one-pixel zero border, i.e. [T + kt - 1][H + kh - 1][W + kw - 1][Cin] (with up2x:
  * [T + kt - 1][H/2 + 2][W/2 + 2][Cin]); `wt` is the weight as [kt][kh][kw][Cout_pad][Cin]; `bias` (fp32, [Cout])
  * may be NULL; `res` (a residual input added to the result, the `x + h` of vae.py:220; same layout and strides as
- * `y`) may be NULL; `y` is [T][H][W][Cout].  One call's input must stay below 4 GiB. */
+ * `y`) may be NULL; `y` is [T][H][W][Cout].  One call's input must stay below 4 GiB.  A 3x3 spatial kernel on a contiguous padded
+ * input (x_stride = {(H + 2)(W + 2) Cin, (W + 2) Cin, Cin}) with Cout_pad a multiple of 96 or equal to 32 runs the kernel
+ * that stages one run of input rows for the three taps of a kernel row; any other strides run the general kernel
+ * (same result up to the order of the fp32 sums). */
 int sfm_conv3d_cl(const sfm_conv_desc* desc, const void* x, const void* wt, const float* bias, const void* res, void* y,
                   void* stream);
 
