@@ -118,6 +118,13 @@ def test_pipeline_decodes_each_chunk_as_it_is_finished():
     seen = []
     pipe.inference(noise, ctx, vae=vae, on_pixels=lambda i, px: seen.append((i, px.shape[1])))
     assert seen == [(0, 9), (1, 12)]
+    # the decoder on a stream of its own, beside the generator's next passes: same latents, same pixels
+    pipe._seed_count = 0
+    lat_a, vid_a = pipe.inference(noise, ctx, vae=vae)
+    pipe._seed_count = 0
+    lat_b, vid_b = pipe.inference(noise, ctx, vae=vae, decode_stream=torch.cuda.Stream())
+    torch.cuda.synchronize()
+    assert torch.equal(lat_a, lat_b) and torch.equal(vid_a, vid_b)
 
 
 def test_next_blocks_input_formed_in_the_block_before_changes_nothing():
