@@ -649,7 +649,7 @@ size_t monarch_fused_bytes(int na, int nf, int b1, int b2, int nunits) {
 }
 
 template <class E>
-static int launch_fused_t(const MonarchArgs& a, int nunits, void* ws, hipStream_t stream, const StepEvents* ev) {
+static int launch_fused_t(const MonarchArgs& a, int nunits, void* ws, size_t ws_bytes, hipStream_t stream, const StepEvents* ev) {
     const FusedPlan pl = fused_plan(a.na, a.nf, a.b1, a.b2, nunits, cu_count());
     FusedArgs f;
     memset(&f, 0, sizeof(f));
@@ -676,6 +676,10 @@ static int launch_fused_t(const MonarchArgs& a, int nunits, void* ws, hipStream_
     const size_t blocks = (size_t)nunits * pl.nslots * f.ncols;
     f.part_o = ws;
     f.part_lse = (float*)((char*)ws + (blocks * a.b1 * kPitch + 255) / 256 * 256);
+    if (monarch_fused_bytes(a.na, a.nf, a.b1, a.b2, nunits) > ws_bytes) {
+        set_error("internal: the one-kernel forward's pass of %d units does not fit the workspace", nunits);
+        return SFM_ERR_WORKSPACE;
+    }
     if ((int64_t)a.nf * a.b1 * nunits >= ((int64_t)1 << 31) || pl.lds > (size_t)kLdsMax || pl.rc < 8) {
         set_error("internal: fused Monarch launch shape");
         return SFM_ERR_UNSUPPORTED;
@@ -698,8 +702,8 @@ static int launch_fused_t(const MonarchArgs& a, int nunits, void* ws, hipStream_
     return SFM_OK;
 }
 
-int launch_monarch_fused(const MonarchArgs& a, int dtype, int nunits, void* ws, hipStream_t stream, const StepEvents* ev) {
-    return dtype == SFM_BF16 ? launch_fused_t<BF16>(a, nunits, ws, stream, ev) : launch_fused_t<F16>(a, nunits, ws, stream, ev);
+int launch_monarch_fused(const MonarchArgs& a, int dtype, int nunits, void* ws, size_t ws_bytes, hipStream_t stream, const StepEvents* ev) {
+    return dtype == SFM_BF16 ? launch_fused_t<BF16>(a, nunits, ws, ws_bytes, stream, ev) : launch_fused_t<F16>(a, nunits, ws, ws_bytes, stream, ev);
 }
 
 }  // namespace sfm

@@ -150,9 +150,17 @@ struct MonarchPlan {
     size_t per_unit;   // workspace bytes of a pass over one (batch x head) unit: the least a call needs
 };
 
-// Workspace of a pass over n units.
+// Workspace of passes over up to n units.  The one-kernel forward's scratch is not monotonic in the units of a pass
+// (fewer units mean shorter tile ranges per workgroup and more partial-result slots per unit), and the last pass of a
+// call may be shorter than the others, so its size is the largest over every pass length up to n.
 static size_t pass_bytes(const MonarchPlan& pl, int n) {
-    return pl.fused ? monarch_fused_bytes(pl.na, pl.nf, pl.b1, pl.b2, n) : pl.per_unit * (size_t)n;
+    if (!pl.fused) return pl.per_unit * (size_t)n;
+    size_t mx = 0;
+    for (int m = 1; m <= n; ++m) {
+        const size_t b = monarch_fused_bytes(pl.na, pl.nf, pl.b1, pl.b2, m);
+        if (b > mx) mx = b;
+    }
+    return mx;
 }
 
 static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
@@ -365,7 +373,7 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
                         set_error("hipEventCreate failed");
                         return SFM_ERR_HIP;
                     }
-            rc = launch_monarch_fused(a, desc->dtype, n, workspace, (hipStream_t)stream, step_ms ? &se : nullptr);
+            rc = launch_monarch_fused(a, desc->dtype, n, workspace, workspace_bytes, (hipStream_t)stream, step_ms ? &se : nullptr);
             if (step_ms) {
                 float t1 = 0.f, t2 = 0.f;
                 hipError_t e = rc ? hipSuccess : hipEventSynchronize(se.ev[2]);
@@ -407,8 +415,12 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
                 return SFM_ERR_UNSUPPORTED;
             }
             if (pl.iter_mfma) {
-                a.stats = (float*)((char*)a.wgt + rows * sizeof(float) * upp);
+                // the kernels index the row statistics with the global unit (as the caller's buffer of
+                // sfm_monarch_fwd_stats needs); the scratch holds one pass, so its base is moved back by the
+                // pass's first unit
                 a.stats_ld = 32;
+                const uintptr_t stats0 = (uintptr_t)a.wgt + rows * sizeof(float) * upp;
+                a.stats = (float*)(stats0 - (size_t)u0 * pl.na * pl.b2 * a.stats_ld * sizeof(float));
                 rc = launch_monarch_iter_mfma(a, desc->dtype, n, desc->num_iters, (hipStream_t)stream);
             } else {
                 rc = launch_monarch_iter(a, desc->dtype, n, desc->num_iters, (hipStream_t)stream);

@@ -187,7 +187,7 @@ bool monarch_mfma_supported(int dtype, int D, int b2);
 // one-kernel forward (monarch_fused.hip): Kbar / Y stay in LDS; `ws` holds monarch_fused_bytes for a pass of nunits units
 bool monarch_fused_supported(int dtype, int D, int b1, int b2, int causal);
 size_t monarch_fused_bytes(int na, int nf, int b1, int b2, int nunits);
-int launch_monarch_fused(const MonarchArgs& a, int dtype, int nunits, void* ws, hipStream_t stream, const StepEvents* ev);
+int launch_monarch_fused(const MonarchArgs& a, int dtype, int nunits, void* ws, size_t ws_bytes, hipStream_t stream, const StepEvents* ev);
 int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
 // the refinement on the MFMA kernels (16-bit, head_dim 64 / 128, b1 <= 32, b2 <= 64): a.rep in the tensor dtype, a.stats
 // [units][na * b2][a.stats_ld] scratch for the left factor's row statistics

@@ -30,3 +30,26 @@ def assert_close_16bit(got, ref, dtype, atol_scale=1.0):
     assert bad == 0, f"{bad} of {g.numel()} elements outside atol=rtol={tol}; max-abs {max_abs(g, r):.3e}"
     assert max_abs(g, r) < 2e-2
     assert per_head_cosine(got, ref) > 0.999
+
+
+def monarch_fwd_exact_workspace(q, k, v, tiling, heads_per_pass, num_iters=1, one_kernel=False, kv_block_order=0):
+    """sfm_monarch_fwd through the C ABI with a workspace of exactly sfm_monarch_workspace_bytes(heads_per_pass) and
+    64 KiB of canary bytes behind it; returns the output after checking that the canary is untouched."""
+    import ctypes as C
+
+    import self_forcing_amd as sfa
+    from self_forcing_amd import lib as L
+
+    f_tied, h_reduce, w_reduce, h, w = tiling
+    out = torch.full_like(q, float("nan"))
+    d = sfa.monarch_attn._desc(q, k, v, out, f_tied, h_reduce, w_reduce, h, w, q.shape[-1] ** -0.5, kv_block_order, 0,
+                               num_iters, one_kernel)
+    n = sfa.monarch_attn.monarch_workspace_bytes(d, heads_per_pass)
+    pad = 64 * 1024
+    buf = torch.full((n + pad,), 0xA5, dtype=torch.uint8, device=q.device)
+    stream = C.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
+    L.check(L.load().sfm_monarch_fwd(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), buf.data_ptr(), n,
+                                     stream))
+    torch.cuda.synchronize()
+    assert bool((buf[n:] == 0xA5).all()), "bytes behind the workspace were overwritten"
+    return out

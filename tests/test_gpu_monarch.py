@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import self_forcing_amd as sfa
-from gpu_util import assert_close_16bit, max_abs, per_head_cosine, randn
+from gpu_util import assert_close_16bit, max_abs, monarch_fwd_exact_workspace, per_head_cosine, randn
 from oracle import blocks, dense, monarch
 
 pytestmark = pytest.mark.gpu
@@ -70,6 +70,24 @@ def test_head_passes_give_identical_results(heads_per_pass):
     one = mattn.monarch_attn(q, k, v, 1, 1, 1, 6, 20, heads_per_pass=heads_per_pass, one_kernel=True)
     assert_close_16bit(one, ref, torch.bfloat16)
     assert max_abs(one, mattn.monarch_attn(q, k, v, 1, 1, 1, 6, 20, heads_per_pass=5, one_kernel=True)) <= 2 ** -6
+
+
+@pytest.mark.parametrize("one_kernel", [False, True])
+@pytest.mark.parametrize("shape,heads,heads_per_pass", [
+    ((3, 3, 6, 20), 5, 3),         # last pass of 2 units: the one-kernel forward needs more slots for it than for 3
+    ((3, 3, 6, 20), 5, 2),
+    ((2, 4, 12, 16), 7, 4),
+])
+def test_shorter_last_pass_stays_inside_an_exactly_sized_workspace(one_kernel, shape, heads, heads_per_pass):
+    """units % heads_per_pass != 0: the last pass is shorter.  The workspace is exactly what the query returns, with
+    canary bytes behind it."""
+    a, f, b1, b2 = shape
+    q, k, v = (randn((1, n * b1 * b2, heads, 128), 120 + i, torch.bfloat16).to(DEV) for i, n in enumerate((a, f, f)))
+    out = monarch_fwd_exact_workspace(q, k, v, (1, 1, 1, b1, b2), heads_per_pass, one_kernel=one_kernel)
+    ref = monarch.monarch_attn(q.cpu(), k.cpu(), v.cpu(), 1, 1, 1, b1, b2, dtype=torch.float32)
+    assert_close_16bit(out, ref, torch.bfloat16)
+    if not one_kernel:
+        assert torch.equal(out, mattn.monarch_attn(q, k, v, 1, 1, 1, b1, b2))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import self_forcing_amd as sfa
-from gpu_util import assert_close_16bit, max_abs, randn
+from gpu_util import assert_close_16bit, max_abs, monarch_fwd_exact_workspace, randn
 from oracle import monarch
 
 pytestmark = pytest.mark.gpu
@@ -135,3 +135,20 @@ def test_mfma_refinement_golden_vectors_in_bf16():
         assert max_abs(out, gold) < 4e-2
         ref = monarch.monarch_attn(tok(q).cpu(), tok(k).cpu(), tok(v).cpu(), 1, 1, 1, b1, b2, sm_scale=s, num_iters=n, dtype=torch.float32)
         assert_close_16bit(out, ref, torch.bfloat16)
+
+
+@pytest.mark.parametrize("dtype,heads_per_pass", [(torch.bfloat16, 1), (torch.bfloat16, 2), (torch.float32, 1)])
+def test_refinement_in_several_passes_stays_inside_its_workspace(dtype, heads_per_pass):
+    """num_iters = 2 with fewer heads per pass than heads: every pass's scratch (the left factor's row statistics
+    included) lies inside a workspace of exactly the queried size, and the passes give the bits of one pass."""
+    h, w, H, D = 6, 20, 3, 128
+    q = randn((1, 2 * h * w, H, D), 400, dtype).to(DEV)
+    k, v = (randn((1, 3 * h * w, H, D), 401 + i, dtype).to(DEV) for i in range(2))
+    part = monarch_fwd_exact_workspace(q, k, v, (1, 1, 1, h, w), heads_per_pass, num_iters=2)
+    full = monarch_fwd_exact_workspace(q, k, v, (1, 1, 1, h, w), H, num_iters=2)
+    assert torch.equal(part, full)
+    ref = monarch.monarch_attn(q.cpu(), k.cpu(), v.cpu(), 1, 1, 1, h, w, num_iters=2, dtype=torch.float32)
+    if dtype == torch.float32:
+        assert max_abs(part, ref) < 2e-5
+    else:
+        assert_close_16bit(part, ref, dtype)

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def _call_pair(B, H, D, h, w, nq_frames, nc_frames, tiling, dtype, seed):
+def _call_pair(B, H, D, h, w, nq_frames, nc_frames, tiling, dtype, seed, num_iters=1):
     """Runs both entry points on the same inputs; returns (static out, workspace out, caches of both, oracle inputs)."""
     f_tied, h_reduce, w_reduce = tiling
     nq, nc = nq_frames * h * w, nc_frames * h * w
@@ -28,7 +28,7 @@ def _call_pair(B, H, D, h, w, nq_frames, nc_frames, tiling, dtype, seed):
     for static in (True, False):
         kc, vc = kc0.clone(), vc0.clone()
         out = torch.full_like(q, float("nan"))
-        d = sfa.monarch_attn._desc(q, kc, vc, out, f_tied, h_reduce, w_reduce, h, w, D ** -0.5, 1, 0, 1)
+        d = sfa.monarch_attn._desc(q, kc, vc, out, f_tied, h_reduce, w_reduce, h, w, D ** -0.5, 1, 0, num_iters)
         args = (C.byref(d), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), nk.data_ptr(), nv.data_ptr(), L.strides3(nk),
                 nc - nq, nc, out.data_ptr())
         if static:
@@ -57,3 +57,33 @@ def test_static_scratch_matches_workspace_entry_point_twice():
         ref = monarch.monarch_attn_with_kv_cache(q.cpu(), kc0.cpu(), vc0.cpu(), nk.cpu(), nv.cpu(), nc - nq, nc, *tiling, h, w,
                                                  dtype=torch.float32)
         assert_close_16bit(o_static, ref, dtype)
+
+
+@pytest.mark.parametrize("num_iters", [1, 2])
+def test_static_scratch_splits_the_heads_over_several_passes(num_iters):
+    """12 heads against a 21-frame cache of 30 x 52 tokens need 624 MB of scratch (1.2 GB with refinement), so the
+    128 MiB array serves them in several passes; outputs and caches equal the caller-workspace entry point's, which
+    runs one pass."""
+    (o_static, o_ws), ((kc_s, vc_s), (kc_w, vc_w)), _ = _call_pair(1, 12, 128, 30, 52, 3, 21, (1, 1, 1), torch.bfloat16, 720,
+                                                                  num_iters)
+    assert not torch.isnan(o_static.float()).any()
+    assert torch.equal(o_static, o_ws)
+    assert torch.equal(kc_s, kc_w) and torch.equal(vc_s, vc_w)
+
+
+def test_static_scratch_rejects_a_unit_that_does_not_fit():
+    """One head of fp32 tensors at 30 x 52 with 21 frames and h_reduce = 2 needs 2 matrices of 6 x 52 x 640 rows x
+    128 x 4 B = 204 MB > 128 MiB: refused with SFM_ERR_WORKSPACE before anything is written."""
+    h, w, D = 30, 52, 128
+    q = randn((1, 3 * h * w, 1, D), 730).to(DEV)
+    kc, vc = randn((1, 21 * h * w, 1, D), 731).to(DEV), randn((1, 21 * h * w, 1, D), 732).to(DEV)
+    kc0 = kc.clone()
+    out = torch.zeros_like(q)
+    d = sfa.monarch_attn._desc(q, kc, vc, out, 1, 2, 1, h, w, D ** -0.5, 1, 0, 1)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = L.load().sfm_monarch_attn_with_kv_cache_static(C.byref(d), q.data_ptr(), kc.data_ptr(), vc.data_ptr(), q.data_ptr(),
+                                                        q.data_ptr(), L.strides3(q), 18 * h * w, 21 * h * w, out.data_ptr(),
+                                                        stream)
+    torch.cuda.synchronize()
+    assert L.ERR_NAMES[rc] == "SFM_ERR_WORKSPACE"
+    assert torch.equal(kc, kc0) and not out.any()
