@@ -8,6 +8,7 @@ Alongside, the attention op alone at the chunk shape (configs[1]): ms/call, per-
 roofline of the dominant hot-path kernel, dense fallback, and a CPU baseline.  Prints ONE JSON line.
 """
 import argparse
+import gc
 import ctypes as C
 import json
 import os
@@ -158,11 +159,17 @@ def op_level(torch, sfa, args):
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(0)
     bf = torch.bfloat16
-    q = torch.randn(B, SQ, H, D, generator=g).to(bf).to(dev)
-    kc = torch.randn(B, SKV, H, D, generator=g).to(bf).to(dev)
-    vc = torch.randn(B, SKV, H, D, generator=g).to(bf).to(dev)
-    nk = torch.randn(B, SQ, H, D, generator=g).to(bf).to(dev)
-    nv = torch.randn(B, SQ, H, D, generator=g).to(bf).to(dev)
+    # configs[1]: Q, K RMS-normalised + 3-D RoPE'd, V ~ N(0,1).  The projections' outputs are drawn ~ N(0,1) and go
+    # through the fused prologue chunk by chunk, which fills the 21-frame cache (block order = token order for the
+    # framewise tiling) and leaves the last chunk's query.
+    kc = torch.empty(B, SKV, H, D, dtype=bf, device=dev)
+    vc = torch.empty(B, SKV, H, D, dtype=bf, device=dev)
+    ones = torch.ones(H * D, dtype=bf, device=dev)
+    rope = sfa.prologue.rope_table(D, device=dev)
+    for c in range(F // A):
+        xq, xk, xv = (torch.randn(B, SQ, H * D, generator=g).to(bf).to(dev) for _ in range(3))
+        q = sfa.prologue.qk_prologue(xq, xk, xv, ones, ones, H, (A, B1, B2), A * c, rope, kc, vc, c * SQ)
+    nk, nv = kc[:, SKV - SQ:].clone(), vc[:, SKV - SQ:].clone()
     start, end = SKV - SQ, SKV
 
     def step():
@@ -301,7 +308,8 @@ def op_level(torch, sfa, args):
     tfl = MONARCH_FLOPS / (ms_call * 1e-3) / 1e12
     return {
         "monarch_attn": {"workload": "configs[1]: monarch_attn_with_kv_cache, B1 H12 D128, a=3 f=21 b1=30 b2=52 "
-                                     "(4680 q x 32760 kv), new chunk written at tokens 28080..32760",
+                                     "(4680 q x 32760 kv), new chunk written at tokens 28080..32760; Q, K RMS-normalised + 3-D "
+                                     "RoPE'd (N(0,1) projections through qk_prologue), V ~ N(0,1), seed 0",
                          "ms_per_call": ms_call, "tflops": tfl, "mfma_frac": tfl / MFMA_BF16_PEAK_TFLOPS,
                          "kernel_ms": {"monarch_step1": s1_ms, "monarch_step2": s2_ms}},
         "monarch_iter": {"workload": "monarch_attn, num_iters = 8 (monarch_attn_slow), same shape and cache",
@@ -375,6 +383,34 @@ def gemm_legs(torch, sfa):
     return out
 
 
+def rollout_leg(torch, sfa, name, steps, warmup, own_gemm):
+    """Seconds per video of the rollout configuration `name`: `warmup` untimed videos, then `steps` timed ones between
+    device synchronisations.  The generator and its caches are freed afterwards."""
+    _, size, flags, _ = ROLLOUTS[name]
+    pl = sfa.pipeline
+    pl.use_tuned_gemms()          # hipBLASLt solution per GEMM shape (shipped selections; unknown shapes tuned in warm-up)
+    gen = pl.build_generator(size, attention_flags=flags, ops=sfa.causal_model.HipAttentionOps(own_gemm=own_gemm),
+                             init_on_device=size == "14B")
+    pipe = pl.CausalInferencePipeline(gen)
+    g = torch.Generator().manual_seed(0)
+    noise = torch.randn(1, 21, 16, 60, 104, generator=g).to(torch.bfloat16).cuda()
+    ctx = torch.randn(1, 512, 4096, generator=g).to(torch.bfloat16).cuda()
+    for _ in range(warmup):
+        pipe.inference(noise, ctx)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = pipe.inference(noise, ctx)
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / steps
+    assert torch.isfinite(out).all()
+    del pipe, gen, out
+    gc.collect()
+    torch.cuda.empty_cache()
+    torch.cuda.tunable.tuning_enable(False)       # later legs keep the selections made so far and tune nothing new
+    return sec
+
+
 def vae_decode_leg(torch, sfa):
     """Streaming decode of one video's latents (outside the headline metric, which excludes the VAE): random-init
     decoder of the Wan 2.1 VAE shape, bf16, 21 latent frames in 7 chunks of 3 -> 81 frames of 480x832."""
@@ -410,9 +446,12 @@ def main():
     ap.add_argument("--rollout-only", action="store_true",
                     help="for kernel traces: the rollout alone, without the op-level legs, the VAE leg and the CPU baseline "
                          "(the line then carries no roofline)")
-    ap.add_argument("--own-gemm", action="store_true",
-                    help="rollout with the FFN's linear layers on the library's own fused-epilogue kernel (sfm_linear) instead of "
-                         "hipBLASLt + element-wise kernels")
+    ap.add_argument("--own-gemm", choices=("auto", "all", "none"), default="auto",
+                    help="which linear layers of the rollout run on the library's own kernel (sfm_linear): auto = the block's "
+                         "square projections (where it beats hipBLASLt), all = also the FFN with GELU / gated residual in the "
+                         "epilogue, none = hipBLASLt everywhere")
+    ap.add_argument("--no-extra-rollouts", action="store_true",
+                    help="skip the short legs of the other rollout configurations (c4, dense, c5) that follow the c3 headline")
     ap.add_argument("--one-kernel", action="store_true",
                     help="op-level figures of the opt-in one-kernel Monarch forward (Kbar / Y kept in LDS) instead of the default "
                          "two kernels; kernel_ms then holds the fused kernel and its merge kernel")
@@ -451,33 +490,23 @@ def main():
                                   "cache-refresh pass per chunk, per-layer KV cache, text context [1,512,4096] ~ N(0,1); "
                                   "VAE and text encoder excluded",
                       "name": args.config, "heads_per_pass": args.heads_per_pass}}
+    own = {"auto": "auto", "all": True, "none": False}[args.own_gemm]
     if not args.op_only:
-        pl = sfa.pipeline
-        pl.use_tuned_gemms()          # hipBLASLt solution per GEMM shape (shipped selections; unknown shapes tuned in warm-up)
-        gen = pl.build_generator(size, attention_flags=flags,
-                                 ops=sfa.causal_model.HipAttentionOps(own_gemm=True) if args.own_gemm else None)
-        rec["config"]["own_gemm"] = bool(args.own_gemm)
-        pipe = pl.CausalInferencePipeline(gen)
-        g = torch.Generator().manual_seed(0)
-        noise = torch.randn(1, 21, 16, 60, 104, generator=g).to(torch.bfloat16).cuda()
-        ctx = torch.randn(1, 512, 4096, generator=g).to(torch.bfloat16).cuda()
-        for _ in range(args.warmup):
-            pipe.inference(noise, ctx)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            out = pipe.inference(noise, ctx)
-        torch.cuda.synchronize()
-        sec = (time.perf_counter() - t0) / args.steps
-        assert torch.isfinite(out).all()
+        sec = rollout_leg(torch, sfa, args.config, args.steps, args.warmup, own)
+        rec["config"]["own_gemm"] = args.own_gemm
         rec["value"] = 21.0 / sec
         rec["ms_per_step"] = sec * 1e3
-        del pipe, gen
-        torch.cuda.empty_cache()
-        torch.cuda.tunable.tuning_enable(False)       # the legs below keep the selections made so far and tune nothing new
     if args.rollout_only:
         print(json.dumps(rec))
         return
+    if not args.op_only and args.config == "c3" and not args.no_extra_rollouts:
+        # the other rollout configurations, 1 warm-up + 2 timed videos each (the headline fields above are c3's)
+        rec["rollouts"] = {}
+        for name in ("c4", "dense", "c5"):
+            sec = rollout_leg(torch, sfa, name, 2, 1, own)
+            entry, size, _, what = ROLLOUTS[name]
+            rec["rollouts"][name] = {"workload": f"{entry}: {what}", "value": 21.0 / sec, "unit": "latent frames/s",
+                                     "ms_per_step": sec * 1e3, "steps": 2, "warmup": 1}
     rec.update(op_level(torch, sfa, args))
     if args.config == "c3":
         rec["vae_decode"] = vae_decode_leg(torch, sfa)

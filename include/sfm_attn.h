@@ -275,7 +275,7 @@ typedef struct sfm_linear_desc {
     int32_t N, K;
     int64_t x_stride, out_stride, res_stride, gate_stride;   /* elements */
     int32_t rows_per_frame;   /* rows sharing one gate row (GATE_RESIDUAL with a gate) */
-    int32_t reserved;
+    int32_t tile_rows;        /* output rows per workgroup: 0 = chosen from the shape, 128 or 256 = forced (measurements) */
 } sfm_linear_desc;
 int sfm_linear(const sfm_linear_desc* desc, const void* x, const void* w, const void* bias, const void* res, const void* gate,
                void* out, void* stream);

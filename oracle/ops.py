@@ -60,6 +60,9 @@ class OracleOps:
             return x, self.ln_affine(x, weight, bias, eps)
         return x, self.ln_modulate(x, scale, shift, eps)
 
+    def linear(self, x, linear):
+        return linear(x)
+
     def linear_gelu(self, x, linear):
         return torch.nn.functional.gelu(linear(x), approximate='tanh')
 

@@ -39,12 +39,23 @@ class HipAttentionOps:
     may pass another object with the same methods (e.g. one built on the CPU oracle and eager torch ops) to
     obtain a reference run of the same module code.
 
-    own_gemm=True runs the FFN's two linear layers on the library's own matrix-product kernel with the GELU and the
-    gated residual update in its epilogue (`linear.linear`) instead of hipBLASLt + a separate element-wise kernel; it is
-    off by default because hipBLASLt's kernels are faster on MI355X at these shapes."""
+    own_gemm selects which linear layers run on the library's own matrix-product kernel (`linear.linear`) instead of
+    hipBLASLt: "auto" (default) the square projections of the block (attention output, cross-attention q and output:
+    N, K <= 2048), where the own kernel's 128 x 256 tiles fill the chip and hipBLASLt's tile choice does not (26 vs
+    29 us at 4680 x 1536 x 1536); True additionally the FFN with the GELU and the gated residual update in the GEMM's
+    epilogue (slower than hipBLASLt on MI355X at these shapes); False none."""
 
-    def __init__(self, own_gemm=False):
-        self.own_gemm = bool(own_gemm)
+    def __init__(self, own_gemm="auto"):
+        self.own_gemm = own_gemm is True
+        self.own_square = own_gemm is True or own_gemm == "auto"
+
+    def linear(self, x, linear):
+        """nn.Linear forward for inference: the own kernel for the block's square projections, else the library."""
+        w = linear.weight
+        if (self.own_square and not torch.is_grad_enabled() and w.shape[0] <= 2048 and w.shape[1] <= 2048 and x.dim() == 3
+                and _lin.supported(x, w)):
+            return _lin.linear(x, w, linear.bias)
+        return linear(x)
 
     def rope_table(self, head_dim, device):
         return _pro.rope_table(head_dim, device=device)
@@ -311,7 +322,7 @@ class CausalWanSelfAttention(nn.Module):
         else:
             y = self.ops.monarch_cached(q, k_view, v_view, f_tied, fl.h_reduce, fl.w_reduce, h, w, fl.num_iters)
         cache_commit(kv_cache, current_end, local_end)
-        return self.o(y.flatten(2))
+        return self.ops.linear(y.flatten(2), self.o)
 
 
 class WanT2VCrossAttention(nn.Module):
@@ -330,7 +341,7 @@ class WanT2VCrossAttention(nn.Module):
 
     def forward(self, x, context, crossattn_cache=None):
         b, n, d = x.size(0), self.num_heads, self.head_dim
-        q = self.ops.rms_norm(self.q(x), self.norm_q.weight, self.norm_q.eps).view(b, -1, n, d)
+        q = self.ops.rms_norm(self.ops.linear(x, self.q), self.norm_q.weight, self.norm_q.eps).view(b, -1, n, d)
         if crossattn_cache is not None and crossattn_cache["is_init"]:
             k, v = crossattn_cache["k"], crossattn_cache["v"]
         else:
@@ -339,7 +350,7 @@ class WanT2VCrossAttention(nn.Module):
             if crossattn_cache is not None:
                 crossattn_cache["is_init"] = True
                 crossattn_cache["k"], crossattn_cache["v"] = k, v
-        return self.o(self.ops.dense(q, k, v).flatten(2))
+        return self.ops.linear(self.ops.dense(q, k, v).flatten(2), self.o)
 
 
 class CausalWanAttentionBlock(nn.Module):

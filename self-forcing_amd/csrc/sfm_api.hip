@@ -1109,6 +1109,10 @@ int sfm_linear(const sfm_linear_desc* d, const void* x, const void* w, const voi
         set_error("M=%lld, N=%d, K=%d: need M >= 1, N a multiple of 8 and K a multiple of 64", (long long)d->M, d->N, d->K);
         return SFM_ERR_SHAPE;
     }
+    if (d->tile_rows != 0 && d->tile_rows != 128 && d->tile_rows != 256) {
+        set_error("tile_rows must be 0, 128 or 256");
+        return SFM_ERR_SHAPE;
+    }
     const bool gr = d->epilogue == SFM_EPI_GATE_RESIDUAL;
     if (gr && !res) {
         set_error("the gated-residual epilogue needs res");

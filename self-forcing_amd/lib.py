@@ -39,7 +39,7 @@ class ConvDesc(C.Structure):
 class LinearDesc(C.Structure):
     _fields_ = [("dtype", C.c_int32), ("epilogue", C.c_int32), ("M", C.c_int64), ("N", C.c_int32), ("K", C.c_int32),
                 ("x_stride", C.c_int64), ("out_stride", C.c_int64), ("res_stride", C.c_int64), ("gate_stride", C.c_int64),
-                ("rows_per_frame", C.c_int32), ("reserved", C.c_int32)]
+                ("rows_per_frame", C.c_int32), ("tile_rows", C.c_int32)]
 
 
 EPI_NONE, EPI_GELU_TANH, EPI_GATE_RESIDUAL = 0, 1, 2

@@ -18,10 +18,11 @@ def supported(x, weight):
             and x.shape[0] * x.shape[1] * x.stride(1) * 2 < 2 ** 32)
 
 
-def linear(x, weight, bias=None, epilogue="none", res=None, gate=None, out=None):
+def linear(x, weight, bias=None, epilogue="none", res=None, gate=None, out=None, tile_rows=0):
     """x: [B, L, K]; weight: [N, K]; bias: [N] or None.
     epilogue "none": x @ weight.T + bias; "gelu_tanh": GELU (tanh form) of that; "gate_residual": res + (that) * gate with
-    gate a per-frame modulation tensor [B, F, 1, N] (None: res + that), written to `out` (default: in place into res)."""
+    gate a per-frame modulation tensor [B, F, 1, N] (None: res + that), written to `out` (default: in place into res).
+    `tile_rows` (0, 128, 256) forces the output rows per workgroup; 0 lets the library choose from the shape."""
     if epilogue not in _EPI:
         raise ValueError(f"unknown epilogue {epilogue!r}")
     if x.dtype not in (torch.bfloat16, torch.float16):
@@ -40,6 +41,7 @@ def linear(x, weight, bias=None, epilogue="none", res=None, gate=None, out=None)
     B, L = x.shape[:2]
     d = _l.LinearDesc()
     d.dtype, d.epilogue, d.M, d.N, d.K, d.x_stride = _DT[x.dtype], _EPI[epilogue], rows, N, K, xs
+    d.tile_rows = tile_rows
     g = None
     if epilogue == "gate_residual":
         if res is None:

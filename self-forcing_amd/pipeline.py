@@ -240,13 +240,19 @@ def use_tuned_gemms(filename=None, tune=True):
 
 
 def build_generator(size="1.3B", dtype=torch.bfloat16, device="cuda:0", seed=0, zero_head=False, timestep_shift=5.0,
-                    **model_overrides):
-    """Random-init causal Wan generator of a named size (reference init, optionally with a non-zero head)."""
+                    init_on_device=False, **model_overrides):
+    """Random-init causal Wan generator of a named size (reference init, optionally with a non-zero head).
+    `init_on_device` draws the weights on `device` instead of on the host (other values for the same seed; the 14B
+    model's 56 GB of fp32 parameters take over a minute to draw on the host)."""
     from .causal_model import WAN_CONFIGS
     cfg = dict(WAN_CONFIGS[size]) if size in WAN_CONFIGS else {}
     cfg.update(model_overrides)
     torch.manual_seed(seed)
-    model = CausalWanModel(**cfg)
+    if init_on_device:
+        with torch.device(device):
+            model = CausalWanModel(**cfg)
+    else:
+        model = CausalWanModel(**cfg)
     model.init_weights(zero_head=zero_head)
     model = model.to(dtype=dtype, device=device).eval()
     return WanDiffusionWrapper(model, timestep_shift=timestep_shift)

@@ -40,12 +40,16 @@ def _assert_rounding_close(got, ref, dtype, frac=1e-2, steps=1, scale=None):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (300, 264, 128), (1, 8, 64), (517, 1000, 192), (4680, 1536, 1536)])
-def test_plain_linear(dtype, M, N, K):
+@pytest.mark.parametrize("tile_rows", [0, 128, 256])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (300, 264, 128), (1, 8, 64), (517, 1000, 192), (130, 520, 256), (640, 304, 320),
+                                   (4680, 1536, 1536)])
+def test_plain_linear(dtype, tile_rows, M, N, K):
+    """K from one to 24 stages of 64 (the first, second-to-last and last stages of the load ring are separate code);
+    both tile heights, and the library's own choice."""
     x, w, b = randn((1, M, K), 1, dtype).to(DEV), (randn((N, K), 2, dtype) * K ** -0.5).to(dtype).to(DEV), randn((N,), 3, dtype).to(DEV)
-    out = lin.linear(x, w, b)
+    out = lin.linear(x, w, b, tile_rows=tile_rows)
     _assert_rounding_close(out, _ref(x, w, b, dtype, "none"), dtype)
-    out = lin.linear(x, w, None)
+    out = lin.linear(x, w, None, tile_rows=tile_rows)
     _assert_rounding_close(out, _ref(x, w, None, dtype, "none"), dtype)
 
 
@@ -63,10 +67,11 @@ def test_strided_rows_and_batches(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tile_rows", [128, 256])
 @pytest.mark.parametrize("M,N,K", [(300, 264, 128), (4680, 8960, 1536)])
-def test_gelu_tanh_epilogue(dtype, M, N, K):
+def test_gelu_tanh_epilogue(dtype, tile_rows, M, N, K):
     x, w, b = randn((1, M, K), 7, dtype).to(DEV), (randn((N, K), 8, dtype) * K ** -0.5).to(dtype).to(DEV), randn((N,), 9, dtype).to(DEV)
-    out = lin.linear(x, w, b, epilogue="gelu_tanh")
+    out = lin.linear(x, w, b, epilogue="gelu_tanh", tile_rows=tile_rows)
     # a product that lands one rounding step away moves the result by |gelu'(y)| steps of y: in the left tail, where
     # the result itself is tiny, that is many steps of the result, so the steps are measured at |gelu(y)| + |y gelu'(y)|
     y = _ref(x, w, b, dtype, "none").float().requires_grad_(True)
@@ -79,7 +84,8 @@ def test_gelu_tanh_epilogue(dtype, M, N, K):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,F,rpf,N,K,gated", [(1, 3, 100, 264, 128, True), (2, 2, 60, 136, 192, True), (1, 3, 1560, 1536, 8960, True),
                                                (1, 1, 300, 264, 128, False)])
-def test_gate_residual_epilogue(dtype, B, F, rpf, N, K, gated):
+@pytest.mark.parametrize("tile_rows", [128, 256])
+def test_gate_residual_epilogue(dtype, tile_rows, B, F, rpf, N, K, gated):
     L = F * rpf
     x, w, b = randn((B, L, K), 10, dtype).to(DEV), (randn((N, K), 11, dtype) * K ** -0.5).to(dtype).to(DEV), randn((N,), 12, dtype).to(DEV)
     res = randn((B, L, N), 13, dtype).to(DEV)
@@ -87,11 +93,11 @@ def test_gate_residual_epilogue(dtype, B, F, rpf, N, K, gated):
     ref = _ref(x, w, b, dtype, "gate_residual", res, gate, rpf)
     mag = res.float().abs() + (ref.float() - res.float()).abs()        # |res| + |gated product|
     keep = res.clone()
-    out = lin.linear(x, w, b, epilogue="gate_residual", res=res, gate=gate)
+    out = lin.linear(x, w, b, epilogue="gate_residual", res=res, gate=gate, tile_rows=tile_rows)
     assert out.data_ptr() == res.data_ptr()                     # in place, like `x = x + y * e`
     _assert_rounding_close(out, ref, dtype, frac=2e-2, steps=3, scale=mag)
     out2 = torch.empty_like(keep)
-    lin.linear(x, w, b, epilogue="gate_residual", res=keep, gate=gate, out=out2)
+    lin.linear(x, w, b, epilogue="gate_residual", res=keep, gate=gate, out=out2, tile_rows=tile_rows)
     assert torch.equal(out2, out)
 
 
