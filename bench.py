@@ -446,10 +446,10 @@ def main():
     ap.add_argument("--rollout-only", action="store_true",
                     help="for kernel traces: the rollout alone, without the op-level legs, the VAE leg and the CPU baseline "
                          "(the line then carries no roofline)")
-    ap.add_argument("--own-gemm", choices=("auto", "all", "none"), default="auto",
-                    help="which linear layers of the rollout run on the library's own kernel (sfm_linear): auto = the block's "
-                         "square projections (where it beats hipBLASLt), all = also the FFN with GELU / gated residual in the "
-                         "epilogue, none = hipBLASLt everywhere")
+    ap.add_argument("--own-gemm", choices=("auto", "all", "none"), default="none",
+                    help="which linear layers of the rollout run on the library's own kernel (sfm_linear): none = hipBLASLt "
+                         "everywhere (fastest), auto = the block's square projections, all = also the FFN with GELU / gated "
+                         "residual in the epilogue")
     ap.add_argument("--no-extra-rollouts", action="store_true",
                     help="skip the short legs of the other rollout configurations (c4, dense, c5) that follow the c3 headline")
     ap.add_argument("--one-kernel", action="store_true",

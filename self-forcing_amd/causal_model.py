@@ -40,12 +40,12 @@ class HipAttentionOps:
     obtain a reference run of the same module code.
 
     own_gemm selects which linear layers run on the library's own matrix-product kernel (`linear.linear`) instead of
-    hipBLASLt: "auto" (default) the square projections of the block (attention output, cross-attention q and output:
-    N, K <= 2048), where the own kernel's 128 x 256 tiles fill the chip and hipBLASLt's tile choice does not (26 vs
-    29 us at 4680 x 1536 x 1536); True additionally the FFN with the GELU and the gated residual update in the GEMM's
-    epilogue (slower than hipBLASLt on MI355X at these shapes); False none."""
+    hipBLASLt: False (default) none; "auto" the square projections of the block (attention output, cross-attention q
+    and output: N, K <= 2048), where the own kernel's 128 x 256 tiles are level with hipBLASLt in isolation (26 vs
+    25-29 us at 4680 x 1536 x 1536) and 0.5 % slower over a rollout; True additionally the FFN with the GELU and the
+    gated residual update in the GEMM's epilogue (10-15 % slower than the tuned hipBLASLt kernels at those shapes)."""
 
-    def __init__(self, own_gemm="auto"):
+    def __init__(self, own_gemm=False):
         self.own_gemm = own_gemm is True
         self.own_square = own_gemm is True or own_gemm == "auto"
 

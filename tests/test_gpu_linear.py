@@ -150,3 +150,19 @@ def test_block_ffn_on_the_own_kernel_matches_the_library_path():
     assert (h.float() - lib_ops.linear_gelu(xn, up).float()).abs().max() <= 2.0 ** -6
     err = (got.float() - want.float()).abs()
     assert err.max() <= 2.0 ** -4 and err.mean() < 2e-3, (err.max().item(), err.mean().item())
+
+
+def test_square_projection_on_the_own_kernel_matches_the_library():
+    """HipAttentionOps(own_gemm="auto").linear: N, K <= 2048 run on sfm_linear, wider layers and the default stay on
+    the library; same values up to the fp32 summation order."""
+    cm = sfa.causal_model
+    dtype = torch.bfloat16
+    torch.manual_seed(5)
+    sq, wide = torch.nn.Linear(512, 512).to(DEV, dtype), torch.nn.Linear(512, 2304).to(DEV, dtype)
+    x = randn((1, 700, 512), 50, dtype).to(DEV)
+    with torch.no_grad():
+        auto, none = cm.HipAttentionOps(own_gemm="auto"), cm.HipAttentionOps()
+        assert none.linear(x, wide).data_ptr() != 0 and not none.own_square and auto.own_square and not auto.own_gemm
+        _assert_rounding_close(auto.linear(x, sq), sq(x), dtype)
+        assert torch.equal(auto.linear(x, wide), wide(x))           # too wide for "auto": the library runs it
+        assert torch.equal(none.linear(x, sq), sq(x))
