@@ -421,7 +421,7 @@ Parts make_parts(const MonarchArgs& p, int dtype, const int64_t* dks) {
     const bool q_rows_ok = (p.qs[0] | p.qs[1] | p.qs[2] | p.os[0] | p.os[1] | p.os[2]) % 8 == 0 &&       // 16-byte rows of q, dout, out
                            (int64_t)p.na * p.b1 * p.b2 * p.qs[1] * 2 < ((int64_t)1 << 32);
     f.left = h16 && q_rows_ok && monarch_bwd_left_supported(dtype, p.D, p.b1) && !(sw & SFM_SW_BWD_LEFT_GEMM);
-    f.fwd = f.left && monarch_mfma_supported(dtype, p.D, p.b2) && !(sw & SFM_SW_BWD_FWD_GEMM);
+    f.fwd = f.left && monarch_mfma_supported(dtype, p.D, p.b2) && p.b2 <= 64 && !(sw & SFM_SW_BWD_FWD_GEMM);   // R rows of 64 values
     f.dqa = f.left && !(sw & SFM_SW_BWD_DQA_GEMM);
     const bool direct_ok = (dks[0] | dks[1] | dks[2] | p.vs[0] | p.vs[1] | p.vs[2] | p.ks[0] | p.ks[1] | p.ks[2]) % 8 == 0 &&      // 16-byte rows of k, v, dk, dv
                            (int64_t)p.nf * p.b1 * p.b2 * p.ks[1] * 2 < ((int64_t)1 << 32);

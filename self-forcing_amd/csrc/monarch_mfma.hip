@@ -1,4 +1,4 @@
-// Monarch attention forward on gfx950 MFMA (bf16 / fp16, head_dim 64 or 128, block cols b2 <= 64).
+// Monarch attention forward on gfx950 MFMA (bf16 / fp16, head_dim 64 or 128, block cols b2 <= 128).
 //
 // Two kernels per pass over a group of (batch x head) units:
 //
@@ -47,21 +47,25 @@ template <int CPR>
 __device__ __forceinline__ int s1_swz(int r) {
     return CPR >= 16 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
 }
-template <int D>
+template <int D, int NT>
 struct S1Lds {
-    static constexpr int kPitch = 2 * D, kTile = 64 * kPitch;
+    static constexpr int kRows = NT <= 2 ? 64 : 32 * NT;     // rows of a K / V tile
+    static constexpr int kPitch = 2 * D, kTile = kRows * kPitch;
     static constexpr int kGroup = 4 * kTile;                 // [buffer][K tile | V tile]
     static __host__ __device__ constexpr size_t bytes() { return (size_t)kGroup; }
 };
 
-// NT: 32-row tiles of the key axis l (2 when b2 > 32).
+// NT: 32-row tiles of the key axis l (b2 <= 32 NT).  Up to two tiles a workgroup is two wave groups of at most 5 waves
+//     (170 registers per wave); three and four tiles (b2 up to 128: the 720p and 1080p grids) run one group of up to 8
+//     waves with 256 registers, whose tile buffers take 96 / 128 KB of LDS.
 // WR: also write the right factor R (16 bit, 64 values per scratch row) to p.rb; the backward uses it.
 // IT: a pass of the iterated refinement (wan/modules/monarch_attn.py:1716-1722): the logits are scaled per (a, f, k, j)
 //     column and, after the first pass, the query operand of tile (f, k) is the column's representative p.rep[a, j, (f, k)]
 //     instead of Q[a, k, j]; the operand is then fetched for every tile.
 template <class E, int D, int NT, bool WR = false, bool IT = false>
-__global__ __launch_bounds__(640) __attribute__((amdgpu_waves_per_eu(3, 3))) void monarch_step1_kernel(MonarchArgs p) {
-    using L = S1Lds<D>;
+__global__ __launch_bounds__(NT > 2 ? 512 : 640) __attribute__((amdgpu_waves_per_eu(NT > 2 ? 2 : 3, NT > 2 ? 2 : 3)))
+void monarch_step1_kernel(MonarchArgs p) {
+    using L = S1Lds<D, NT>;
     constexpr int CPR = D / 8;   // 16-byte chunks of a K/V row
     constexpr int DS = D / 16;   // contraction steps of the logits
     extern __shared__ __attribute__((aligned(256))) char lds_s1[];
@@ -720,7 +724,7 @@ __global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
 // host launch
 // ------------------------------------------------------------------------------------------------
 bool monarch_mfma_supported(int dtype, int D, int b2) {
-    return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 >= 1 && b2 <= 64;
+    return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b2 >= 1 && b2 <= 128;
 }
 
 int cu_count() {
@@ -746,11 +750,18 @@ static int enqueue_step1(const MonarchArgs& a, int nunits, hipStream_t stream, c
         set_error("internal: step-1 launch shape (a_chunk=%d, b2=%d)", a.a_chunk, a.b2);
         return SFM_ERR_UNSUPPORTED;
     }
-    const int groups = nwaves <= 5 ? 2 : 1;             // wave groups per workgroup (<= 10 waves in all)
-    const size_t lds1 = S1Lds<D>::bytes() * groups;
+    const int nt = (a.b2 + 31) / 32;
+    const int groups = nwaves <= 5 && nt <= 2 ? 2 : 1;  // wave groups per workgroup (<= 10 waves in all)
+    const size_t lds1 = (nt == 4 ? S1Lds<D, 4>::bytes() : nt == 3 ? S1Lds<D, 3>::bytes() : S1Lds<D, 2>::bytes()) * groups;
+    if (nt > 2 && a.rb) {
+        set_error("internal: the right factor is written for b2 <= 64 only");
+        return SFM_ERR_UNSUPPORTED;
+    }
     const void* fn = fn_override ? fn_override
-                     : a.b2 > 32 ? (a.rb ? (const void*)monarch_step1_kernel<E, D, 2, true> : (const void*)monarch_step1_kernel<E, D, 2, false>)
-                                 : (a.rb ? (const void*)monarch_step1_kernel<E, D, 1, true> : (const void*)monarch_step1_kernel<E, D, 1, false>);
+                     : nt == 4 ? (const void*)monarch_step1_kernel<E, D, 4, false>
+                     : nt == 3 ? (const void*)monarch_step1_kernel<E, D, 3, false>
+                     : nt == 2 ? (a.rb ? (const void*)monarch_step1_kernel<E, D, 2, true> : (const void*)monarch_step1_kernel<E, D, 2, false>)
+                               : (a.rb ? (const void*)monarch_step1_kernel<E, D, 1, true> : (const void*)monarch_step1_kernel<E, D, 1, false>);
     if (lds1 > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1);
         if (e != hipSuccess) {
@@ -812,7 +823,7 @@ int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_
 }
 
 bool monarch_iter_mfma_supported(int dtype, int D, int b1, int b2) {
-    return monarch_mfma_supported(dtype, D, b2) && b1 >= 1 && b1 <= 32;
+    return monarch_mfma_supported(dtype, D, b2) && b2 <= 64 && b1 >= 1 && b1 <= 32;
 }
 
 // num_iters passes of [step 1 with the pass's query operands | step 2 | representatives for the next pass]; the last

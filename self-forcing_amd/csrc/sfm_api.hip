@@ -339,7 +339,7 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
     int rc = plan_monarch(desc, &pl);
     if (rc) return rc;
     if (stats && (!pl.mfma || pl.iter)) {
-        set_error("row statistics come from the MFMA forward only (16-bit tensors, head_dim 64 or 128, b2 <= 64, num_iters 1)");
+        set_error("row statistics come from the MFMA forward only (16-bit tensors, head_dim 64 or 128, b2 <= 128, num_iters 1)");
         return SFM_ERR_UNSUPPORTED;
     }
     if (!q || !k || !v || !out) {

@@ -161,12 +161,49 @@ def test_block_causal_no_cache(dtype):
             assert_close_16bit(out, ref, dtype, atol_scale=2.0)      # the reference's causal bar is 2e-2
 
 
-def test_generic_path_wide_blocks():
-    """b2 = 80 (the 720p grid) is outside the MFMA kernels and runs the fp32 generic kernels."""
-    q, k, v = (randn((1, n * 3 * 80, 2, 128), 60 + i, torch.bfloat16) for i, n in enumerate((2, 3, 3)))
-    ref = monarch.monarch_attn(q, k, v, 1, 1, 1, 3, 80, dtype=torch.float32)
-    out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, 3, 80)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("a,f,b1,b2,D", [
+    (2, 3, 3, 80, 128),            # 80 columns: three 32-row key tiles
+    (3, 4, 45, 80, 128),           # the 720p grid (utils/resolution.py:14-27): 45 x 80 tokens per frame
+    (2, 3, 67, 120, 128),          # the 1080p grid: 67 x 120, four key tiles, two query block-frames per workgroup
+    (3, 2, 5, 128, 64),            # full 128-wide blocks, head_dim 64
+    (1, 2, 4, 97, 128),            # odd width
+    (3, 6, 90, 52, 128),           # the reference's default tiling at 480p: three frames tied, b1 = 90
+])
+def test_wide_and_tall_blocks_run_on_the_mfma_kernels(dtype, a, f, b1, b2, D):
+    """b2 in (64, 128] (the reference's 720p / 1080p grids) and b1 > 32 (f_tied = 3) against the oracle; the fp32 path
+    for the same 16-bit tensors (reached with fp32 copies) must agree as well."""
+    q, k, v = (randn((1, n * b1 * b2, 2, D), 60 + i, dtype) for i, n in enumerate((a, f, f)))
+    ref = monarch.monarch_attn(q, k, v, 1, 1, 1, b1, b2, dtype=torch.float32)
+    out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, b1, b2)
+    assert_close_16bit(out, ref, dtype)
+
+
+def test_720p_kv_cache_call_with_block_order_cache():
+    """monarch_attn_with_kv_cache at 45 x 80 with h_reduce = 3 (b1 = 15, b2 = 80): cache rows bit-exact in block order."""
+    h, w, H, D = 45, 80, 2, 128
+    dtype = torch.bfloat16
+    nq, nc = 3 * h * w, 6 * h * w
+    q, nk, nv = (randn((1, nq, H, D), 130 + i, dtype) for i in range(3))
+    kc, vc = randn((1, nc, H, D), 133, dtype), randn((1, nc, H, D), 134, dtype)
+    kc_o, vc_o = kc.clone(), vc.clone()
+    ref = monarch.monarch_attn_with_kv_cache(q, kc_o, vc_o, nk, nv, nc - nq, nc, 1, 3, 1, h, w, dtype=torch.float32)
+    kd, vd = kc.to(DEV), vc.to(DEV)
+    out = mattn.monarch_attn_with_kv_cache(q.to(DEV), kd, vd, nk.to(DEV), nv.to(DEV), nc - nq, nc, 1, 3, 1, h, w)
+    assert torch.equal(kd.cpu(), kc_o) and torch.equal(vd.cpu(), vc_o)
+    assert_close_16bit(out, ref, dtype)
+
+
+def test_generic_path_very_wide_blocks():
+    """b2 = 144 is outside the MFMA kernels (b2 <= 128) and runs the fp32 generic kernels; b2 = 160 at head_dim 128 is
+    past their LDS budget and is refused before anything runs."""
+    q, k, v = (randn((1, n * 3 * 144, 2, 128), 60 + i, torch.bfloat16) for i, n in enumerate((2, 3, 3)))
+    ref = monarch.monarch_attn(q, k, v, 1, 1, 1, 3, 144, dtype=torch.float32)
+    out = mattn.monarch_attn(q.to(DEV), k.to(DEV), v.to(DEV), 1, 1, 1, 3, 144)
     assert_close_16bit(out, ref, torch.bfloat16)
+    q, k, v = (randn((1, n * 3 * 160, 1, 128), 60 + i, torch.bfloat16).to(DEV) for i, n in enumerate((1, 1, 1)))
+    with pytest.raises(sfa.lib.SfmError, match="SFM_ERR_UNSUPPORTED"):
+        mattn.monarch_attn(q, k, v, 1, 1, 1, 3, 160)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
