@@ -553,13 +553,25 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
 //   rep[a, j, r, :] = sum_i L[i, r] Q[a, i, j, :],   wgt[a, j, r] = sum_i L[i, r],   r = (f, k)
 // with L[i, r] = exp2(s log2e <Q_i, Kbar_r> - cl_r - stats_i), stats = the left factor's row statistics that step 2 wrote.
 // Step 2 with the operands' roles exchanged: one wave per (a, j) streams the column's Kbar rows 32 at a time through its
-// LDS; the logits come out as S[i, r] (A = the lane's query row, in registers; B = Kbar rows), so that a lane holds a
-// column r, and rep^T[d, r] = sum_i Q^T[d, i] L[i, r] takes Q^T from transposing reads of the column's query rows, which
-// sit in the (otherwise unused) Y slot of the wave's first buffer.  b1 <= 32.
+// LDS; the logits come out as S[i, r] (A = query rows, B = Kbar rows), so that a lane holds a column r, and
+// rep^T[d, r] = sum_i Q^T[d, i] L[i, r] takes Q^T from transposing reads of the column's query rows, which sit in the
+// wave's LDS for the whole kernel.  NQ = 32-row tiles of the query rows i (b1 <= 32 NQ <= 128: three frames tied per
+// block give b1 = 90); with one tile the logits' A operand stays in registers, with more it is read from the LDS rows.
+// A workgroup is 4 waves (NQ <= 2) or 3 (more LDS per wave).
 // ------------------------------------------------------------------------------------------------
-template <class E, int D>
+template <int D, int NQ>
+struct RepLds {
+    static constexpr int kPitch = 2 * D, kTile = 32 * kPitch;
+    static constexpr int kBuf = kTile + 256;               // [Kbar chunk | cl values]
+    static constexpr int kQ = 2 * kBuf;                    // offset of the query rows
+    static constexpr int kWave = 2 * kBuf + NQ * kTile;
+    static constexpr int kWaves = NQ <= 2 ? 4 : 3;
+    static __host__ __device__ constexpr size_t bytes() { return (size_t)kWaves * kWave; }
+};
+
+template <class E, int D, int NQ>
 __global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
-    using L = S2Lds<D>;
+    using L = RepLds<D, NQ>;
     constexpr int DS = D / 16, DT = D / 32, CPR = D / 8;
     extern __shared__ __attribute__((aligned(256))) char lds_s2[];
 
@@ -570,9 +582,9 @@ __global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
     const int hf = lane >> 5;
 
     const int b2 = p.b2;
-    const int njg = (b2 + 3) / 4;
+    const int njg = (b2 + L::kWaves - 1) / L::kWaves;
     const int a = blockIdx.x / njg;
-    const int jraw = (blockIdx.x % njg) * 4 + wave;
+    const int jraw = (blockIdx.x % njg) * L::kWaves + wave;
     if (jraw >= b2) return;                               // the waves of a workgroup share nothing
     const int j = jraw;
     const int ul = blockIdx.y;
@@ -589,21 +601,20 @@ __global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
 
     char* const wl = lds_s2 + wave * L::kWave;
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)wl;
-    char* const qt = wl + L::kTile;                       // the column's query rows, laid out like a chunk of scratch rows
+    char* const qt = wl + L::kQ;                          // the column's query rows, laid out like chunks of scratch rows
 
     const uint16_t* qg = (const uint16_t*)p.q + (int64_t)b * p.qs[0] + (int64_t)h * p.qs[2];
     // query rows into LDS (rows past b1 repeat the last one; their weights are zero)
 #pragma unroll
-    for (int g = 0; g < CPR / 2; ++g) {
+    for (int g = 0; g < NQ * (CPR / 2); ++g) {
         const int P = g * 64 + lane;
         const int r = P / CPR, c = (P % CPR) ^ s1_swz<CPR>(r);
         const uint32_t off = (uint32_t)((p.qmap.row(a, min(r, p.b1 - 1)) + j) * p.qs[1] * 2) + (uint32_t)c * 16;
-        s1_load_lds16((const char*)qg, off, lds0 + L::kTile + (uint32_t)g * 1024);
+        s1_load_lds16((const char*)qg, off, lds0 + L::kQ + (uint32_t)g * 1024);
     }
-    // logits operand (A): this lane's query row Q[a, m, j, :] (zero past b1), and the statistics of the 16 rows whose
-    // logits this lane will hold
+    // one tile: the logits operand (A) is this lane's query row Q[a, m, j, :] (zero past b1), kept in registers
     u32x4 qa[DS];
-    {
+    if constexpr (NQ == 1) {
         const uint16_t* qrow = qg + (p.qmap.row(a, min(m, p.b1 - 1)) + j) * p.qs[1] + 8 * hf;
 #pragma unroll
         for (int ds = 0; ds < DS; ++ds) qa[ds] = *(const u32x4*)(qrow + 16 * ds);
@@ -614,16 +625,21 @@ __global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
             for (int ds = 0; ds < DS; ++ds) qa[ds] = u32x4{0u, 0u, 0u, 0u};
         }
     }
-    float st[16];
+    // the statistics of the 16 NQ rows whose logits this lane will hold
+    float st[NQ][16];
     {
         const float* sp = p.stats + ((int64_t)unit * (p.na * b2) + a * b2 + j) * p.stats_ld;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
-            st[v] = i < p.b1 ? sp[i] : 0.f;
-        }
+        for (int qi = 0; qi < NQ; ++qi)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) asm volatile("" : "+v"(st[v]));
+            for (int v = 0; v < 16; ++v) {
+                const int i = 32 * qi + 8 * (v >> 2) + 4 * hf + (v & 3);
+                st[qi][v] = i < p.b1 ? sp[i] : 0.f;
+            }
+#pragma unroll
+        for (int qi = 0; qi < NQ; ++qi)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) asm volatile("" : "+v"(st[qi][v]));
     }
 
     // chunk n of the Kbar rows (and their cl values) into buffer `buf`
@@ -636,9 +652,9 @@ __global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
             const uint32_t off = (uint32_t)min(32 * n + r, r_lim - 1) * (2 * D) + (uint32_t)c * 16;
             s1_load_lds16(kb, off, dst + (uint32_t)g * 1024);
         }
-        s2_load_lds4(clp, (uint32_t)(32 * n + m) * 4, dst + 2 * L::kTile);
+        s2_load_lds4(clp, (uint32_t)(32 * n + m) * 4, dst + L::kTile);
     };
-    const uint32_t b_off = (uint32_t)m * L::kPitch + (uint32_t)((hf ^ s1_swz<CPR>(m)) << 4);   // Kbar row m as the logits' B operand
+    const uint32_t b_off = (uint32_t)m * L::kPitch + (uint32_t)((hf ^ s1_swz<CPR>(m)) << 4);   // row m of a 32-row tile as an MFMA operand
     uint32_t tr[DT][2];            // Q^T as the representatives' A operand: transposing reads, as step 2 reads Y^T
     {
         const int s16 = lane & 15, g16 = lane >> 4;
@@ -667,44 +683,51 @@ __global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         const char* kt = wl + (n & 1) * L::kBuf;
-
-        f32x16 s;                  // S[i = 8 g + 4 hf + e, r = 32 n + m]
-#pragma unroll
-        for (int ds = 0; ds < DS; ++ds) {
-            const u32x4 bk = *(const u32x4*)(kt + (b_off ^ (uint32_t)(ds << 5)));
-            s = E::mfma32(qa[ds], bk, ds ? s : kZero);
-        }
-        const float cc = *(const float*)(kt + 2 * L::kTile + m * 4);
+        const float cc = *(const float*)(kt + L::kTile + m * 4);
         const bool rok = 32 * n + m < r_lim;
         float wsum = 0.f;
+        u32x4 pb[NQ][2];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
-            const float e = (rok && i < p.b1) ? exp2f(s[v] * sc2 - cc - st[v]) : 0.f;
-            s[v] = e;
-            wsum += e;
+        for (int qi = 0; qi < NQ; ++qi) {
+            f32x16 s;              // S[i = 32 qi + 8 g + 4 hf + e, r = 32 n + m]
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds) {
+                const u32x4 bk = *(const u32x4*)(kt + (b_off ^ (uint32_t)(ds << 5)));
+                u32x4 aq;
+                if constexpr (NQ == 1) aq = qa[ds];
+                else aq = *(const u32x4*)(qt + qi * L::kTile + (b_off ^ (uint32_t)(ds << 5)));
+                s = E::mfma32(aq, bk, ds ? s : kZero);
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int i = 32 * qi + 8 * (v >> 2) + 4 * hf + (v & 3);
+                const float e = (rok && i < p.b1) ? exp2f(s[v] * sc2 - cc - st[qi][v]) : 0.f;
+                s[v] = e;
+                wsum += e;
+            }
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                pb[qi][q].x = pack2<E>(s[8 * q + 0], s[8 * q + 1]);
+                pb[qi][q].y = pack2<E>(s[8 * q + 2], s[8 * q + 3]);
+                pb[qi][q].z = pack2<E>(s[8 * q + 4], s[8 * q + 5]);
+                pb[qi][q].w = pack2<E>(s[8 * q + 6], s[8 * q + 7]);
+            }
         }
         wsum = xhalf_sum(wsum);
         if (hf == 0) wgt[32 * n + m] = wsum;
-        u32x4 pb[2];
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-            pb[q].x = pack2<E>(s[8 * q + 0], s[8 * q + 1]);
-            pb[q].y = pack2<E>(s[8 * q + 2], s[8 * q + 3]);
-            pb[q].z = pack2<E>(s[8 * q + 4], s[8 * q + 5]);
-            pb[q].w = pack2<E>(s[8 * q + 6], s[8 * q + 7]);
-        }
         char* rrow = repb + (size_t)(32 * n + m) * (2 * D);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             f32x16 acc;
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const u32x2 lo = s1_read_tr(qt, tr[dt][0] + q * 16 * L::kPitch);
-                const u32x2 hi = s1_read_tr(qt, tr[dt][1] + q * 16 * L::kPitch);
-                const u32x4 aq = {lo.x, lo.y, hi.x, hi.y};
-                acc = E::mfma32(aq, pb[q], q ? acc : kZero);
-            }
+            for (int qi = 0; qi < NQ; ++qi)
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const u32x2 lo = s1_read_tr(qt + qi * L::kTile, tr[dt][0] + q * 16 * L::kPitch);
+                    const u32x2 hi = s1_read_tr(qt + qi * L::kTile, tr[dt][1] + q * 16 * L::kPitch);
+                    const u32x4 aq = {lo.x, lo.y, hi.x, hi.y};
+                    acc = E::mfma32(aq, pb[qi][q], (qi | q) ? acc : kZero);
+                }
             // rep^T[d = 32 dt + 8 g + 4 hf + e, r]: the half-swap leaves 8 consecutive d per lane
 #pragma unroll
             for (int gp = 0; gp < 2; ++gp) {
@@ -823,7 +846,20 @@ int launch_monarch_step1(const MonarchArgs& a, int dtype, int nunits, hipStream_
 }
 
 bool monarch_iter_mfma_supported(int dtype, int D, int b1, int b2) {
-    return monarch_mfma_supported(dtype, D, b2) && b2 <= 64 && b1 >= 1 && b1 <= 32;
+    return monarch_mfma_supported(dtype, D, b2) && b1 >= 1 && b1 <= 128;
+}
+
+template <class E, int D, int NQ>
+static int launch_rep_t(const MonarchArgs& a, int nunits, hipStream_t stream) {
+    using L = RepLds<D, NQ>;
+    hipError_t e = hipFuncSetAttribute((const void*)monarch_rep_kernel<E, D, NQ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)L::bytes());
+    if (e != hipSuccess) {
+        set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+        return SFM_ERR_HIP;
+    }
+    const int njg = (a.b2 + L::kWaves - 1) / L::kWaves;
+    hipLaunchKernelGGL((monarch_rep_kernel<E, D, NQ>), dim3(a.na * njg, nunits), dim3(64 * L::kWaves), L::bytes(), stream, a);
+    return SFM_OK;
 }
 
 // num_iters passes of [step 1 with the pass's query operands | step 2 | representatives for the next pass]; the last
@@ -831,11 +867,14 @@ bool monarch_iter_mfma_supported(int dtype, int D, int b1, int b2) {
 template <class E, int D>
 static int launch_iter_t(const MonarchArgs& a, int nunits, int num_iters, hipStream_t stream) {
     const int njg = (a.b2 + 3) / 4;
-    const dim3 g2(a.na * njg, nunits, 1);
-    const void* fn1 = a.b2 > 32 ? (const void*)monarch_step1_kernel<E, D, 2, false, true> : (const void*)monarch_step1_kernel<E, D, 1, false, true>;
+    const int nq = (a.b1 + 31) / 32;
+    const dim3 g2(a.na * njg, nunits, nq);
+    const int nt = (a.b2 + 31) / 32;
+    const void* fn1 = nt == 4 ? (const void*)monarch_step1_kernel<E, D, 4, false, true>
+                    : nt == 3 ? (const void*)monarch_step1_kernel<E, D, 3, false, true>
+                    : nt == 2 ? (const void*)monarch_step1_kernel<E, D, 2, false, true>
+                              : (const void*)monarch_step1_kernel<E, D, 1, false, true>;
     hipError_t e = hipFuncSetAttribute((const void*)monarch_step2_kernel<E, D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)S2Lds<D>::bytes());
-    if (e == hipSuccess)
-        e = hipFuncSetAttribute((const void*)monarch_rep_kernel<E, D>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)S2Lds<D>::bytes());
     if (e != hipSuccess) {
         set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
         return SFM_ERR_HIP;
@@ -849,7 +888,11 @@ static int launch_iter_t(const MonarchArgs& a, int nunits, int num_iters, hipStr
         MonarchArgs a2 = a;
         if (last) a2.stats = nullptr;
         hipLaunchKernelGGL((monarch_step2_kernel<E, D>), g2, dim3(256), S2Lds<D>::bytes(), stream, a2);
-        if (!last) hipLaunchKernelGGL((monarch_rep_kernel<E, D>), dim3(g2.x, g2.y), dim3(256), S2Lds<D>::bytes(), stream, a);
+        if (!last) {
+            const int rc = nq == 1 ? launch_rep_t<E, D, 1>(a, nunits, stream) : nq == 2 ? launch_rep_t<E, D, 2>(a, nunits, stream)
+                         : nq == 3 ? launch_rep_t<E, D, 3>(a, nunits, stream) : launch_rep_t<E, D, 4>(a, nunits, stream);
+            if (rc) return rc;
+        }
     }
     e = hipGetLastError();
     if (e != hipSuccess) {
@@ -860,7 +903,8 @@ static int launch_iter_t(const MonarchArgs& a, int nunits, int num_iters, hipStr
 }
 
 int launch_monarch_iter_mfma(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream) {
-    if (!monarch_iter_mfma_supported(dtype, a.D, a.b1, a.b2) || a.causal || !a.rep || !a.wgt || !a.stats || a.stats_ld < 32) {
+    if (!monarch_iter_mfma_supported(dtype, a.D, a.b1, a.b2) || a.causal || !a.rep || !a.wgt || !a.stats ||
+        (int)a.stats_ld < (a.b1 + 31) / 32 * 32) {
         set_error("internal: iterated MFMA launch");
         return SFM_ERR_UNSUPPORTED;
     }

@@ -232,7 +232,7 @@ static int plan_monarch(const sfm_monarch_desc* d, MonarchPlan* pl) {
     pl->iter_mfma = pl->iter && monarch_iter_mfma_supported(d->dtype, d->D, pl->b1, pl->b2) && !(switches() & SFM_SW_ITER_SIMT);
     const size_t rows = (size_t)pl->na * pl->b2 * pl->r_pad;
     pl->per_unit = rows * d->D * (pl->mfma || pl->iter_mfma ? 2 : 4) * (pl->iter ? 3 : 2) + rows * sizeof(float) * (pl->iter ? 2 : 1) +
-                   (pl->iter_mfma ? (size_t)pl->na * pl->b2 * 32 * sizeof(float) : 0);
+                   (pl->iter_mfma ? (size_t)pl->na * pl->b2 * ((pl->b1 + 31) / 32 * 32) * sizeof(float) : 0);
     pl->per_unit = (pl->per_unit + 255) / 256 * 256;
     // the fp32 kernels' own limits, checked here so that no entry point has written anything (the KV-cache entry points
     // write the cache before the forward is launched) when they are exceeded
@@ -418,7 +418,7 @@ static int monarch_fwd_impl(const sfm_monarch_desc* desc, const void* q, const v
                 // the kernels index the row statistics with the global unit (as the caller's buffer of
                 // sfm_monarch_fwd_stats needs); the scratch holds one pass, so its base is moved back by the
                 // pass's first unit
-                a.stats_ld = 32;
+                a.stats_ld = (uint32_t)((pl.b1 + 31) / 32 * 32);
                 const uintptr_t stats0 = (uintptr_t)a.wgt + rows * sizeof(float) * upp;
                 a.stats = (float*)(stats0 - (size_t)u0 * pl.na * pl.b2 * a.stats_ld * sizeof(float));
                 rc = launch_monarch_iter_mfma(a, desc->dtype, n, desc->num_iters, (hipStream_t)stream);

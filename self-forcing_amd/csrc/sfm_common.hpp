@@ -189,7 +189,7 @@ bool monarch_fused_supported(int dtype, int D, int b1, int b2, int causal);
 size_t monarch_fused_bytes(int na, int nf, int b1, int b2, int nunits);
 int launch_monarch_fused(const MonarchArgs& a, int dtype, int nunits, void* ws, size_t ws_bytes, hipStream_t stream, const StepEvents* ev);
 int launch_monarch_iter(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);
-// the refinement on the MFMA kernels (16-bit, head_dim 64 / 128, b1 <= 32, b2 <= 64): a.rep in the tensor dtype, a.stats
+// the refinement on the MFMA kernels (16-bit, head_dim 64 / 128, b1 <= 128, b2 <= 128): a.rep in the tensor dtype, a.stats
 // [units][na * b2][a.stats_ld] scratch for the left factor's row statistics
 bool monarch_iter_mfma_supported(int dtype, int D, int b1, int b2);
 int launch_monarch_iter_mfma(const MonarchArgs& a, int dtype, int nunits, int num_iters, hipStream_t stream);

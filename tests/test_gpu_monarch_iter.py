@@ -104,9 +104,15 @@ def switches():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("h,w,D,frames,n", [(6, 20, 128, (1, 3), 2), (8, 40, 64, (2, 3), 3), (30, 52, 128, (1, 2), 3),
-                                             (5, 33, 64, (2, 2), 8), (32, 64, 128, (1, 2), 2), (4, 8, 128, (3, 5), 8)])
+                                             (5, 33, 64, (2, 2), 8), (32, 64, 128, (1, 2), 2), (4, 8, 128, (3, 5), 8),
+                                             (40, 33, 128, (1, 2), 3),       # two 32-row query tiles
+                                             (90, 20, 64, (1, 2), 2),        # three (b1 = 90: three 30-row frames tied)
+                                             (100, 8, 128, (2, 1), 2),       # four
+                                             (6, 80, 128, (2, 3), 2),        # 80 columns: three key tiles in step 1
+                                             (5, 128, 64, (1, 2), 3),        # 128 columns
+                                             (45, 80, 128, (1, 2), 2)])      # the 720p grid
 def test_mfma_refinement_against_the_oracle_and_the_fp32_kernels(dtype, h, w, D, frames, n, switches):
-    """16-bit tensors with b1 <= 32, b2 <= 64 run the refinement on the MFMA kernels (representatives kept in the
+    """16-bit tensors with b1 <= 128, b2 <= 128 run the refinement on the MFMA kernels (representatives kept in the
     tensor dtype); the same call with SFM_SW_ITER_SIMT runs the fp32 kernels.  Both against the fp32 oracle at the
     reference's 16-bit bar, and against each other."""
     H = 2
