@@ -5,9 +5,11 @@
 
 Inputs are [B, S, H, D] CUDA tensors (bf16 / fp16 / fp32, head_dim contiguous) in token order;
 the KV cache holds rows in Monarch block order and is updated in place.  Under autograd the operators
-are torch.autograd.Functions whose backward runs the library's fp32 backward kernels (num_iters == 1).
+are torch.autograd.Functions whose backward runs the library's backward kernels (num_iters == 1).
 num_iters > 1 runs the alternating refinement the reference implements in pure torch
-(monarch_attn_slow, wan/modules/monarch_attn.py:1705-1751) as fp32 HIP kernels.
+(monarch_attn_slow, wan/modules/monarch_attn.py:1705-1751) as HIP kernels; under autograd its forward is still the HIP
+kernels and its backward differentiates a torch restatement of the passes on the GPU (the reference's own refinement is
+differentiable torch and has no backward kernels either).
 """
 import ctypes as C
 
@@ -252,6 +254,106 @@ class _MonarchCacheFn(torch.autograd.Function):
         return dq.to(q.dtype), dk_cache, dv_cache, dk_new, dv_new, None, None, None, None, None, None
 
 
+def _to_block_order(x, f_tied, h_reduce, w_reduce, h, w):
+    """The reference's rearrangement (monarch_attn.py:1696-1703) of a token-order [B, n, H, D] tensor: rows in Monarch
+    block order."""
+    if f_tied == 1 and h_reduce == 1 and w_reduce == 1:
+        return x
+    B, n, H, D = x.shape
+    x = x.reshape(B, -1, f_tied, h_reduce, h // h_reduce, w_reduce, w // w_reduce, H, D)
+    return x.permute(0, 1, 3, 5, 2, 4, 6, 7, 8).reshape(B, n, H, D)
+
+
+def _refinement_torch(qb, kb, vb, sm_scale, num_iters):
+    """The refinement passes (monarch_attn.py:1705-1751) as differentiable torch ops on block-ordered tensors
+    qb [B, a, b1, b2, H, D], kb / vb [B, f, b1, b2, H, D]; used for gradients only.  Pass p forms the right factor R from
+    the per-block query representatives of pass p - 1 (first pass: the queries themselves, weight 1), then the left
+    factor L; the last pass's factors are applied to V."""
+    rs = float(sm_scale) ** 0.5
+    q = qb.permute(0, 4, 1, 2, 3, 5) * rs                 # [B, H, a, i, j, D]
+    k = kb.permute(0, 4, 1, 2, 3, 5) * rs                 # [B, H, f, k, l, D]
+    v = vb.permute(0, 4, 1, 2, 3, 5)
+    nf = k.shape[2]
+    rep = q.unsqueeze(3).expand(-1, -1, -1, nf, -1, -1, -1)          # [B, H, a, f, k, j, D]: block row k of the queries
+    inv_w = q.new_full((), 1.0 / (1.0 + 1e-6))
+    for it in range(num_iters):
+        z = torch.einsum("bhafkjd,bhfkld->bhafkjl", rep, k) * inv_w
+        log_r = torch.log_softmax(z, -1)
+        r = log_r.exp()
+        kbar = torch.einsum("bhafkjl,bhfkld->bhafkjd", r, k)
+        neg_h = (r * log_r).sum(-1)                                   # [B, H, a, f, k, j]
+        s2 = torch.einsum("bhaijd,bhafkjd->bhaijfk", q, kbar) - neg_h.permute(0, 1, 2, 5, 3, 4).unsqueeze(3)
+        left = torch.softmax(s2.flatten(5), -1).reshape(s2.shape)    # [B, H, a, i, j, f, k]
+        if it + 1 < num_iters:
+            rep = torch.einsum("bhaijfk,bhaijd->bhafkjd", left, q)
+            inv_w = torch.clamp(1.0 / (left.sum(3).permute(0, 1, 2, 4, 5, 3) + 1e-6), max=1e4).unsqueeze(-1)
+    y = torch.einsum("bhafkjl,bhfkld->bhafkjd", r, v)
+    return torch.einsum("bhaijfk,bhafkjd->bhaijd", left, y).permute(0, 2, 3, 4, 1, 5)
+
+
+def _refinement_grads(q, k, v, dout, tiling, sm_scale, num_iters, kv_block_order):
+    """(dq, dk, dv) of the refinement for token-order q / dout and k, v in token order or (kv_block_order) block order;
+    gradients come back in the same orders, float32."""
+    f_tied, h_reduce, w_reduce, h, w = tiling
+    b1, b2 = f_tied * (h // h_reduce), w // w_reduce
+    with torch.enable_grad():
+        q_, k_, v_ = (t.detach().float().requires_grad_(True) for t in (q, k, v))
+        B, _, H, D = q.shape
+        qb = _to_block_order(q_, *tiling).reshape(B, -1, b1, b2, H, D)
+        kb = (k_ if kv_block_order else _to_block_order(k_, *tiling)).reshape(B, -1, b1, b2, H, D)
+        vb = (v_ if kv_block_order else _to_block_order(v_, *tiling)).reshape(B, -1, b1, b2, H, D)
+        ob = _refinement_torch(qb, kb, vb, sm_scale, num_iters)
+        out = _from_block_order(ob.reshape(B, -1, H, D), *tiling)
+        return torch.autograd.grad(out, (q_, k_, v_), dout.float())
+
+
+class _MonarchIterFn(torch.autograd.Function):
+    """monarch_attn with num_iters > 1 under autograd: HIP kernels forward, torch restatement for the gradients."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, tiling, sm_scale, num_iters, heads_per_pass, kv_block_order):
+        with torch.no_grad():
+            out = monarch_attn(q, k, v, *tiling, sm_scale=sm_scale, num_iters=num_iters, heads_per_pass=heads_per_pass,
+                               kv_block_order=kv_block_order)
+        ctx.save_for_backward(q, k, v)
+        ctx.cfg = (tiling, sm_scale, num_iters, kv_block_order)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v = ctx.saved_tensors
+        tiling, sm_scale, num_iters, kv_block_order = ctx.cfg
+        dq, dk, dv = _refinement_grads(q, k, v, dout, tiling, sm_scale, num_iters, kv_block_order)
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None, None
+
+
+class _MonarchCacheIterFn(torch.autograd.Function):
+    """monarch_attn_with_kv_cache with num_iters > 1 under autograd (cache written in place in the forward)."""
+
+    @staticmethod
+    def forward(ctx, q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, tiling, sm_scale, num_iters, grad_only_new_kv,
+                heads_per_pass):
+        with torch.no_grad():
+            out = monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx, *tiling, sm_scale=sm_scale,
+                                             num_iters=num_iters, heads_per_pass=heads_per_pass)
+        ctx.save_for_backward(q, k_cache, v_cache)
+        ctx.cfg = (start_idx, end_idx, tiling, sm_scale, num_iters, grad_only_new_kv)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k_cache, v_cache = ctx.saved_tensors
+        start_idx, end_idx, tiling, sm_scale, num_iters, grad_only_new_kv = ctx.cfg
+        dq, dkc, dvc = _refinement_grads(q, k_cache, v_cache, dout, tiling, sm_scale, num_iters, True)
+        dk_new = _from_block_order(dkc[:, start_idx:end_idx], *tiling).to(k_cache.dtype)
+        dv_new = _from_block_order(dvc[:, start_idx:end_idx], *tiling).to(v_cache.dtype)
+        if grad_only_new_kv:
+            dkc = dvc = None
+        else:
+            dkc, dvc = dkc.to(k_cache.dtype), dvc.to(v_cache.dtype)
+        return dq.to(q.dtype), dkc, dvc, dk_new, dv_new, None, None, None, None, None, None, None
+
+
 def _needs_grad(*ts):
     return torch.is_grad_enabled() and any(t.requires_grad for t in ts)
 
@@ -262,10 +364,12 @@ def monarch_attn_with_kv_cache(q, k_cache, v_cache, new_k, new_v, start_idx, end
     returns one-iteration Monarch attention of q against the whole cache view.  `heads_per_pass` and `one_kernel`
     (no counterparts in the reference) bound the scratch and select the forward that keeps its intermediates in LDS."""
     if _needs_grad(q, k_cache, v_cache, new_k, new_v):
-        if num_iters != 1:
-            raise NotImplementedError("num_iters > 1 has no backward")
         if sm_scale is None:
             sm_scale = q.shape[-1] ** -0.5
+        if num_iters != 1:
+            return _MonarchCacheIterFn.apply(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx,
+                                             (f_tied, h_reduce, w_reduce, h, w), sm_scale, num_iters, grad_only_new_kv,
+                                             heads_per_pass)
         return _MonarchCacheFn.apply(q, k_cache, v_cache, new_k, new_v, start_idx, end_idx,
                                      (f_tied, h_reduce, w_reduce, h, w), sm_scale, grad_only_new_kv, heads_per_pass)
     _check4("q", q)
@@ -326,10 +430,13 @@ def monarch_attn(q, k, v, f_tied, h_reduce, w_reduce, h, w, sm_scale=None, block
     that k, v are a KV-cache view whose rows are already in Monarch block order, e.g. after
     prologue.qk_prologue wrote them."""
     if _needs_grad(q, k, v):
-        if num_iters != 1:
-            raise NotImplementedError("num_iters > 1 has no backward")
         if sm_scale is None:
             sm_scale = q.shape[-1] ** -0.5
+        if num_iters != 1:
+            if block_causal_size is not None:
+                raise ValueError("causal currently only supported for num_iters=1")
+            return _MonarchIterFn.apply(q, k, v, (f_tied, h_reduce, w_reduce, h, w), sm_scale, num_iters, heads_per_pass,
+                                        kv_block_order)
         return _MonarchFn.apply(q, k, v, (f_tied, h_reduce, w_reduce, h, w), sm_scale, block_causal_size,
                                 heads_per_pass, kv_block_order)
     _check4("q", q)

@@ -62,6 +62,12 @@ def main():
         cot = torch.randn(q.shape, generator=torch.Generator().manual_seed(seed + 1000), dtype=torch.float64)
         fn["monarch_attn_ref_op"](qa, ka, va, s).backward(cot)
         out[f"case{ci}_dq"], out[f"case{ci}_dk"], out[f"case{ci}_dv"] = qa.grad.numpy(), ka.grad.numpy(), va.grad.numpy()
+        # the refinement is plain differentiable torch in the reference: its gradients for the same cotangent
+        for n in (2, 3):
+            qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+            fn["monarch_attn_slow"](qa, ka, va, s, num_iters=n).backward(cot)
+            out[f"case{ci}_slow{n}_dq"], out[f"case{ci}_slow{n}_dk"], out[f"case{ci}_slow{n}_dv"] = (
+                qa.grad.numpy(), ka.grad.numpy(), va.grad.numpy())
     # block-order permutation: token ids through rearrange_fn for several tilings (h=6, w=8, 3 frames)
     h, w, F = 6, 8, 3
     x = torch.arange(F * h * w, dtype=torch.float64).reshape(1, -1, 1, 1)

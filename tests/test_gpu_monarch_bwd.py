@@ -3,8 +3,8 @@ float64 CPU oracle.  Shapes follow the reference's harness (run_kv_cache_test / 
 monarch_attn.py:1880-1957) at sizes the oracle finishes in seconds.
 
 Tolerances: fp32 tensors <= 2e-4 of the gradient's max-abs (fp32 kernels, sums of ~10^3 terms); 16-bit tensors the
-reference's rtol = 1e-2 (bf16) / 1e-3 (fp16) with atol = the same fraction of the gradient's max-abs (the reference
-compares raw values of O(1) gradients from randn inputs)."""
+reference harness's own raw bar, atol = rtol = 1e-2 (bf16) / 1e-3 (fp16) on the unscaled gradients
+(monarch_attn.py:1908-1920)."""
 import pytest
 import torch
 
@@ -281,5 +281,5 @@ print("SUM", *(float(t.grad.double().abs().sum()) for t in (q, k, v)))
 
 def test_descriptor_errors():
     q = randn((1, 64, 1, 32), 140, torch.float32).to(DEV).requires_grad_(True)
-    with pytest.raises(NotImplementedError):
-        mattn.monarch_attn(q, q, q, 1, 1, 1, 4, 8, num_iters=2)
+    with pytest.raises(ValueError):                        # block-causal masking is defined for one iteration only
+        mattn.monarch_attn(q, q, q, 1, 1, 1, 4, 8, block_causal_size=32, num_iters=2)

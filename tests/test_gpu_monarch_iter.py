@@ -158,3 +158,63 @@ def test_refinement_in_several_passes_stays_inside_its_workspace(dtype, heads_pe
         assert max_abs(part, ref) < 2e-5
     else:
         assert_close_16bit(part, ref, dtype)
+
+
+@pytest.mark.parametrize("ci", [0, 1, 2])
+@pytest.mark.parametrize("n", [2, 3])
+def test_refinement_gradients_against_the_reference_golden_gradients(ci, n):
+    """dq, dk, dv of num_iters = 2, 3 under autograd (HIP forward, gradients from the torch restatement of the passes on
+    the GPU) against the gradients autograd gives through the reference's own `monarch_attn_slow` for the same seeded
+    cotangent (fp32 on the GPU against float64: 2e-4 of the gradient's max-abs)."""
+    q, k, v, s, (B, a, f, b1, b2, H, D) = _golden_inputs(ci)
+    seed = int(GOLD[f"case{ci}_meta"][0])
+    cot = torch.randn(q.shape, generator=torch.Generator().manual_seed(seed + 1000), dtype=torch.float64)
+    tok = lambda t: t.reshape(B, -1, H, D).float().to(DEV)
+    qd, kd, vd = (tok(t).requires_grad_(True) for t in (q, k, v))
+    out = mattn.monarch_attn(qd, kd, vd, 1, 1, 1, b1, b2, sm_scale=s, num_iters=n)
+    assert max_abs(out, torch.from_numpy(GOLD[f"case{ci}_slow{n}"]).reshape(B, -1, H, D)) < 2e-5
+    out.backward(tok(cot))
+    for name, t in (("dq", qd), ("dk", kd), ("dv", vd)):
+        ref = torch.from_numpy(GOLD[f"case{ci}_slow{n}_{name}"]).reshape(B, -1, H, D)
+        assert max_abs(t.grad, ref) < 2e-4 * max(1.0, ref.abs().max().item()), name
+
+
+@pytest.mark.parametrize("grad_only_new_kv", [False, True])
+def test_refinement_gradients_through_the_cache_entry_point(grad_only_new_kv):
+    """bf16, h_reduce = 2 (block order differs from token order), cache of 3 frames of which the last arrives with the
+    call: gradients of q, of the new K / V (token order) and of the cache (block order) against autograd through the
+    float64 oracle on the same rounded inputs; the reference's 16-bit bar."""
+    h, w, H, D, n = 6, 20, 2, 64, 2
+    tiling = (1, 2, 1)
+    dtype = torch.bfloat16
+    fr = h * w
+    q = randn((1, fr, H, D), 500, dtype)
+    kc, vc = randn((1, 3 * fr, H, D), 501, dtype), randn((1, 3 * fr, H, D), 502, dtype)
+    nk, nv = randn((1, fr, H, D), 503, dtype), randn((1, fr, H, D), 504, dtype)
+    cot = randn((1, fr, H, D), 505, dtype)
+    # oracle: float64 leaves, the cache assembled from the old rows and the new chunk
+    from oracle import blocks
+    qo, nko, nvo = (t.double().requires_grad_(True) for t in (q, nk, nv))
+    kco, vco = kc.double().requires_grad_(True), vc.double().requires_grad_(True)
+    new_rows_k = blocks.to_blocks(nko, *tiling, h, w).reshape(1, -1, H, D)
+    new_rows_v = blocks.to_blocks(nvo, *tiling, h, w).reshape(1, -1, H, D)
+    kfull = torch.cat((kco[:, :2 * fr], new_rows_k), 1)
+    vfull = torch.cat((vco[:, :2 * fr], new_rows_v), 1)
+    b1, b2 = h // 2, w
+    ob = monarch.monarch_iter(blocks.to_blocks(qo, *tiling, h, w), kfull.reshape(1, -1, b1, b2, H, D),
+                              vfull.reshape(1, -1, b1, b2, H, D), D ** -0.5, n)
+    blocks.from_blocks(ob, *tiling, h, w).backward(cot.double())
+    # device
+    qd, nkd, nvd = (t.to(DEV).requires_grad_(True) for t in (q, nk, nv))
+    kcd, vcd = kc.to(DEV).requires_grad_(True), vc.to(DEV).requires_grad_(True)
+    out = mattn.monarch_attn_with_kv_cache(qd, kcd, vcd, nkd, nvd, 2 * fr, 3 * fr, *tiling, h, w, num_iters=n,
+                                           grad_only_new_kv=grad_only_new_kv)
+    out.backward(cot.to(DEV))
+    tol = 1e-2
+    for got, ref in ((qd.grad, qo.grad), (nkd.grad, nko.grad), (nvd.grad, nvo.grad)):
+        assert torch.allclose(got.float().cpu(), ref.float(), atol=tol, rtol=tol), max_abs(got, ref)
+    if grad_only_new_kv:
+        assert kcd.grad is None and vcd.grad is None
+    else:
+        for got, ref in ((kcd.grad, kco.grad), (vcd.grad, vco.grad)):
+            assert torch.allclose(got[:, :2 * fr].float().cpu(), ref[:, :2 * fr].float(), atol=tol, rtol=tol)

@@ -58,3 +58,18 @@ def test_gradients_match_autograd_of_the_reference_formula(ci):
     for name, t in (("dq", qa), ("dk", ka), ("dv", va)):
         ref = GOLD[f"case{ci}_{name}"]
         assert np.abs(t.grad.numpy() - ref).max() < 1e-5 * max(1.0, np.abs(ref).max()), name
+
+
+@pytest.mark.parametrize("ci", [0, 1, 2])
+@pytest.mark.parametrize("n", [2, 3])
+def test_refinement_gradients_match_autograd_of_the_reference_formula(ci, n):
+    """dq, dk, dv of the iterated refinement (the reference's `monarch_attn_slow` is plain differentiable torch): autograd
+    through the oracle against autograd through the reference function, same cotangent as above."""
+    q, k, v, s = _inputs(ci)
+    seed = int(GOLD[f"case{ci}_meta"][0])
+    cot = torch.randn(q.shape, generator=torch.Generator().manual_seed(seed + 1000), dtype=torch.float64)
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    monarch.monarch_iter(qa, ka, va, s, n).backward(cot)
+    for name, t in (("dq", qa), ("dk", ka), ("dv", va)):
+        ref = GOLD[f"case{ci}_slow{n}_{name}"]
+        assert np.abs(t.grad.numpy() - ref).max() < 1e-5 * max(1.0, np.abs(ref).max()), name
