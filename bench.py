@@ -383,6 +383,45 @@ def gemm_legs(torch, sfa):
     return out
 
 
+def forward_shapes_leg(torch, sfa):
+    """ms per call of the two Monarch forwards (two kernels with Kbar / Y in HBM; one kernel with them in LDS) at the
+    chunk shapes of the rollout configurations: 3 query frames against a 21-frame cache in block order, bf16, random
+    operands.  The one-kernel forward covers b1 <= 32, b2 <= 64; elsewhere its column is null."""
+    dev, bf = "cuda:0", torch.bfloat16
+    shapes = [("c2: H12, 30x52 framewise (a=3 f=21 b1=30 b2=52)", 12, 30, 52, (1, 1, 1)),
+              ("c4: H12, 30x52 reduce2xh (a=6 f=42 b1=15 b2=52)", 12, 30, 52, (1, 2, 1)),
+              ("c5: H40, 30x52 framewise", 40, 30, 52, (1, 1, 1)),
+              ("reference default tiling: H12, 30x52, three frames tied (a=1 f=7 b1=90 b2=52)", 12, 30, 52, (3, 1, 1)),
+              ("720p: H12, 45x80 framewise (a=3 f=21 b1=45 b2=80)", 12, 45, 80, (1, 1, 1))]
+    out = {}
+    g = torch.Generator().manual_seed(1)
+    for name, heads, h, w, tiling in shapes:
+        q = torch.randn(1, 3 * h * w, heads, 128, generator=g).to(bf).to(dev)
+        k = torch.randn(1, 21 * h * w, heads, 128, generator=g).to(bf).to(dev)
+        v = torch.randn(1, 21 * h * w, heads, 128, generator=g).to(bf).to(dev)
+        b1, b2 = tiling[0] * h // tiling[1], w // tiling[2]
+        rec = {}
+        for key, one in (("two_kernels_ms", False), ("one_kernel_ms", True)):
+            if one and (b1 > 32 or b2 > 64):
+                rec[key] = None
+                continue
+            f = lambda: sfa.monarch_attn.monarch_attn(q, k, v, *tiling, h, w, kv_block_order=True, one_kernel=one)
+            for _ in range(3):
+                f()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(10):
+                f()
+            e1.record()
+            torch.cuda.synchronize()
+            rec[key] = e0.elapsed_time(e1) / 10
+        out[name] = rec
+        del q, k, v
+    sfa.monarch_attn.release_scratch()
+    torch.cuda.empty_cache()
+    return out
+
+
 def rollout_leg(torch, sfa, name, steps, warmup, own_gemm):
     """Seconds per video of the rollout configuration `name`: `warmup` untimed videos, then `steps` timed ones between
     device synchronisations.  The generator and its caches are freed afterwards."""
@@ -508,6 +547,7 @@ def main():
             rec["rollouts"][name] = {"workload": f"{entry}: {what}", "value": 21.0 / sec, "unit": "latent frames/s",
                                      "ms_per_step": sec * 1e3, "steps": 2, "warmup": 1}
     rec.update(op_level(torch, sfa, args))
+    rec["monarch_forward_shapes"] = forward_shapes_leg(torch, sfa)
     if args.config == "c3":
         rec["vae_decode"] = vae_decode_leg(torch, sfa)
     if args.op_only:

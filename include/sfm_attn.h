@@ -348,8 +348,8 @@ int sfm_probe_l2_read(int32_t workgroups, int32_t stages, void* workspace, size_
  * the bit on (SFM_BWD_SIMT=1 ...), SFM_NO_ROCBLAS makes the library behave as where rocBLAS is absent, and SFM_S1_WGS=n
  * overrides the step-1 workgroup count.  No entry point reads the environment afterwards; sfm_set_switches replaces the
  * mask for the whole process (returns the previous one; unknown bits are rejected with (unsigned)-1 and leave it
- * unchanged), which is how the tests reach every path from one process.  Workspace queries follow the mask, so change it
- * only between a query and the call it sizes, never in between. */
+ * unchanged), which is how the tests reach every path from one process.  Workspace queries follow the mask: do not
+ * change it between a workspace query and the call that uses that size. */
 #define SFM_SW_BWD_SIMT        0x01u  /* backward on the fp32 SIMT kernels */
 #define SFM_SW_BWD_LEFT_GEMM   0x02u  /* backward parts on the batched library GEMMs instead of their fused kernels: */
 #define SFM_SW_BWD_FWD_GEMM    0x04u

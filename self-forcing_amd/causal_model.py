@@ -303,7 +303,9 @@ class CausalWanSelfAttention(nn.Module):
             if roll[2] > 0:      # window eviction (causal_model.py:919-922)
                 src, dst, ln = roll
                 for key in ("k", "v"):
-                    kv_cache[key][:, dst:dst + ln] = kv_cache[key][:, src:src + ln].clone()
+                    moved = kv_cache[key][:, src:src + ln]
+                    # the ranges overlap when more rows stay than leave; only then is a temporary needed
+                    kv_cache[key][:, dst:dst + ln] = moved.clone() if src - dst < ln else moved
             view_len = local_end
         is_init = fl.use_dense_init and view_len == 3 * frame_seqlen
         dense = fl.disable_monarch or is_init

@@ -3,6 +3,7 @@
 Activations are [T, H, W, C] tensors (one video; channels contiguous).  Weights are re-laid out once per module
 as [kt, kh, kw, Cout_pad, Cin] and cached on it.  The reference's modules are nn.Conv3d / nn.Conv2d on
 [B, C, T, H, W] (wan/modules/vae.py:17-36, :76-79)."""
+import collections
 import ctypes as C
 
 import torch
@@ -49,19 +50,27 @@ def norm_act(x, gamma, act, out=None):
     return out
 
 
-_PADDED = {}
+_PADDED = collections.OrderedDict()
+PADDED_BUDGET_BYTES = 24 << 30      # one 480 x 832 decode stream keeps about 9 GB of padded inputs
 
 
 def _padded(shape, cin, dtype, device):
-    """A zero-bordered input buffer of `shape`, one per (device, stream, shape, real input channels, dtype), kept for the life of the
-    process (release_padded() drops them): the kernel never writes its input, every call overwrites the interior, so
-    border, channel padding and anything else a call does not write stay zero and no call after the first fills the
-    buffer.  Calls that share a buffer are ordered by their stream.  Returns (buffer, it is new)."""
+    """A zero-bordered input buffer of `shape`, one per (device, stream, shape, real input channels, dtype): the kernel
+    never writes its input, every call overwrites the interior, so border, channel padding and anything else a call does
+    not write stay zero and no call after the first fills the buffer.  Calls that share a buffer are ordered by their
+    stream.  The buffers are kept across calls up to PADDED_BUDGET_BYTES in all; past that the least recently used ones
+    are dropped (another chunk length, resolution or stream brings its own set), and release_padded() drops them all.
+    Returns (buffer, it is new)."""
     key = (device, torch.cuda.current_stream(device).cuda_stream, tuple(shape), cin, dtype)
     buf = _PADDED.get(key)
     if buf is not None:
+        _PADDED.move_to_end(key)
         return buf, False
     buf = _PADDED[key] = torch.zeros(shape, dtype=dtype, device=device)
+    total = sum(b.numel() * b.element_size() for b in _PADDED.values())
+    while total > PADDED_BUDGET_BYTES and len(_PADDED) > 1:
+        _, old = _PADDED.popitem(last=False)            # never the one just made: it is the newest
+        total -= old.numel() * old.element_size()
     return buf, True
 
 
