@@ -51,7 +51,7 @@ def norm_act(x, gamma, act, out=None):
 
 
 _PADDED = collections.OrderedDict()
-PADDED_BUDGET_BYTES = 24 << 30      # one 480 x 832 decode stream keeps about 9 GB of padded inputs
+PADDED_BUDGET_BYTES = 16 << 30      # one 480 x 832 decode stream keeps 29 buffers, 4.8 GB (the largest 1.0 GB)
 
 
 def _padded(shape, cin, dtype, device):

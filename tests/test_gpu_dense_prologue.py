@@ -25,6 +25,18 @@ def test_dense_reference_shapes(dtype, B, Lq, Lk, H, D):
     assert max_abs(lse, lse_ref) < 1e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,Lq,Lk,H,D", [(1, 4200, 333, 8, 128), (2, 2100, 130, 8, 64), (1, 4680, 512, 12, 128)])
+def test_dense_wide_workgroups(dtype, B, Lq, Lk, H, D):
+    """Enough query blocks for the 256-query workgroups (8 waves): ragged last query block and last key tile, both head
+    dims, and the cross-attention shape (4680 queries against 512 text tokens, 12 heads)."""
+    q, k, v = randn((B, Lq, H, D), 21, dtype), randn((B, Lk, H, D), 22, dtype), randn((B, Lk, H, D), 23, dtype)
+    ref, lse_ref = dense.attention(q, k, v, dtype=torch.float32, return_lse=True)
+    out, lse = sfa.attention.attention(q.to(DEV), k.to(DEV), v.to(DEV), dtype=dtype, return_lse=True)
+    assert_close_16bit(out, ref, dtype)
+    assert max_abs(lse, lse_ref) < 1e-3
+
+
 def test_attention_keeps_half_dtypes_and_returns_qs_dtype():
     """attention.py:62-70, 135-138: float16 / bfloat16 inputs are used as they are (not recast to the default
     bfloat16), anything else is computed in `dtype`; the result has q's original dtype."""
