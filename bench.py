@@ -59,7 +59,7 @@ def measured_traffic():
 
 
 def write_traffic(fetch_csv, write_csv):
-    """Turns the counter_collection CSVs of two rocprofv3 runs of `bench.py --op-only --skip-simt --no-cpu-baseline --copy-probe`
+    """Turns the counter_collection CSVs of two rocprofv3 runs of `bench.py --op-only --skip-simt --skip-shapes --no-cpu-baseline --copy-probe`
     (`--pmc FETCH_SIZE`, then `--pmc WRITE_SIZE`; KiB per dispatch) into profiles/traffic.json.  Each counter is scaled
     by what it reads for the run's own 1 GiB device-to-device copies, whose traffic is known (1 GiB read, 1 GiB written)."""
     import collections
@@ -102,7 +102,7 @@ def write_traffic(fetch_csv, write_csv):
                            text=True).stdout.strip()
     rec = {"commit": (commit + ("+uncommitted kernel changes" if dirty else "")) or None,
            "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --output-format csv -- python3 bench.py --op-only --skip-simt "
-                      "--no-cpu-baseline --copy-probe, then python bench.py --write-traffic FETCH.csv WRITE.csv",
+                      "--skip-shapes --no-cpu-baseline --copy-probe, then python bench.py --write-traffic FETCH.csv WRITE.csv",
            "copy_kernel": "__amd_rocclr_copyBuffer", "copy_dispatches": [n_f, n_w], "fetch_factor": f_fac,
            "write_factor": w_fac, "kernels": kernels}
     with open(os.path.join(ROOT, "profiles", "traffic.json"), "w") as f:
@@ -495,6 +495,9 @@ def main():
                     help="op-level figures of the opt-in one-kernel Monarch forward (Kbar / Y kept in LDS) instead of the default "
                          "two kernels; kernel_ms then holds the fused kernel and its merge kernel")
     ap.add_argument("--skip-simt", action="store_true", help="leave out the 0.7 s of fp32 SIMT refinement calls (profile runs)")
+    ap.add_argument("--skip-shapes", action="store_true",
+                    help="leave out the leg that times both forwards at other chunk shapes (counter runs: the per-dispatch "
+                         "averages of profiles/traffic.json must cover the configs[1] shape only)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="accepted for the profile commands; the 1 GiB device copies (known HBM traffic, for scaling rocprof "
                          "counters) always run")
@@ -547,7 +550,8 @@ def main():
             rec["rollouts"][name] = {"workload": f"{entry}: {what}", "value": 21.0 / sec, "unit": "latent frames/s",
                                      "ms_per_step": sec * 1e3, "steps": 2, "warmup": 1}
     rec.update(op_level(torch, sfa, args))
-    rec["monarch_forward_shapes"] = forward_shapes_leg(torch, sfa)
+    if not args.skip_shapes:
+        rec["monarch_forward_shapes"] = forward_shapes_leg(torch, sfa)
     if args.config == "c3":
         rec["vae_decode"] = vae_decode_leg(torch, sfa)
     if args.op_only:
