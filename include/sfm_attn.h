@@ -60,7 +60,9 @@ typedef struct sfm_monarch_desc {
                                  block-frames (monarch_attn.py:139-141, 804-807), requires Sq == Skv */
     float   sm_scale;         /* logit scale; the reference default is D^-0.5 (monarch_attn.py:1780-1781) */
     int32_t num_iters;        /* 1: the two-kernel fast path; > 1: alternating refinement of the two factors
-                                 (monarch_attn_slow, monarch_attn.py:1705-1751), fp32 kernels, no causal mask */
+                                 (monarch_attn_slow, monarch_attn.py:1705-1751), no causal mask.  Both run MFMA kernels
+                                 for 16-bit tensors with head_dim 64 / 128 and b2 <= 128 (refinement: b1 <= 128 as well),
+                                 fp32 SIMT kernels for everything else */
     int32_t flags;            /* 0, or SFM_MONARCH_ONE_KERNEL */
     int64_t q_stride[3];      /* batch, token, head */
     int64_t k_stride[3];
