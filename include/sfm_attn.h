@@ -119,7 +119,7 @@ typedef struct sfm_monarch_bwd_desc {
 
 int sfm_monarch_bwd_workspace_bytes(const sfm_monarch_bwd_desc* desc, int32_t heads_per_pass, size_t* bytes);
 /* 1 when rocBLAS was found at run time and the SFM_SW_BWD_SIMT switch is off.  The backward is a chain of parts, each a fused
- * MFMA kernel where the problem allows (16-bit tensors, head_dim 64 / 128, b1 <= 32, b2 <= 64 a multiple of 4, at
+ * MFMA kernel where the problem allows (16-bit tensors, head_dim 64 / 128, b1 <= 128, b2 <= 64 a multiple of 4, at
  * most 480 (a, j) columns) and batched rocBLAS GEMMs + row kernels otherwise; when every part is fused the chain
  * runs with or without rocBLAS, else without rocBLAS the fp32 SIMT kernels run.  The first GEMM call on a device
  * creates a rocBLAS handle, which allocates; every other entry point of this header allocates nothing.  No

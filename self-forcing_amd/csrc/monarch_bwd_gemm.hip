@@ -448,10 +448,11 @@ Layout make_layout(const MonarchArgs& p, int n, size_t e, const Parts& f) {
     l.dS1 = take(true, n * p.b1 * AJ * NL * e);
     l.Kbar = take(true, n * AJ * RR * D * e);
     l.Y = take(true, n * AJ * RR * D * e);
-    l.dKbar = take(true, n * AJ * RR * D * e);
-    l.dY = take(true, n * AJ * RR * D * e);
+    const size_t nz = f.left ? (size_t)(p.b1 + 31) / 32 : 1;      // the fused left factor writes one partial slab per 32 query rows
+    l.dKbar = take(true, nz * n * AJ * RR * D * e);
+    l.dY = take(true, nz * n * AJ * RR * D * e);
     l.c = take(true, n * AJ * RR * 4);
-    l.dc = take(true, n * AJ * RR * 4);
+    l.dc = take(true, nz * n * AJ * RR * 4);
     l.S2f = take(!f.left, n * AJ * p.b1 * RR * 4);
     l.dLmf = take(!f.left, n * AJ * p.b1 * RR * 4);
     l.L = take(!f.left, n * AJ * p.b1 * RR * e);

@@ -1,4 +1,4 @@
-// Left-factor part of the Monarch backward on gfx950 MFMA (bf16 / fp16, head_dim 64 or 128, block rows b1 <= 32).
+// Left-factor part of the Monarch backward on gfx950 MFMA (bf16 / fp16, head_dim 64 or 128, block rows b1 <= 128).
 //
 // Replaces, inside the backward of the two-step attention, the per-(a, j) products and row kernels
 //     S2 = q_i . Kbar_r,  dLm = dO_i . Y_r,  L = softmax_r(s S2 - c),  dS2 = L (dLm - sum_r L dLm),
@@ -13,6 +13,10 @@
 // S2[i, r] (A = query rows, B = Kbar rows), so that a lane owns one r and holds 16 of the i: the accumulator layout
 // is then directly the B operand [n = r, k = i] of dY^T = dO^T L and dKbar^T = s Q^T dS2, whose A operands are
 // transposing LDS reads of the dO / Q rows, and dc is an in-lane sum.
+//
+// More than 32 block rows (three frames tied per block: b1 = 90) run one grid slice per 32-row tile of the query rows
+// (blockIdx.z): a slice owns its rows' statistics and dS2 rows, and writes its own partial dKbar / dY / dc (sums over
+// its i) into a slab of its own; monarch_bwd_left_sum_kernel adds the slabs into the first one.
 
 #include <hip/hip_runtime.h>
 
@@ -44,6 +48,7 @@ struct LeftArgs {
     int stats_ld, unit0;
     int b1, b2, AJ, nf, RR, causal;
     float scale;
+    int64_t slab_rows, slab_dc;   // elements between the dkbar / dy slabs and between the dc slabs of two query-row tiles
 };
 
 typedef short bl_s16x4 __attribute__((ext_vector_type(4)));
@@ -93,6 +98,7 @@ __global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
     const bool aj_ok = ajraw < p.AJ;
     const int aj = aj_ok ? ajraw : p.AJ - 1;              // a wave past the end repeats the last column and stores nothing
     const int u = blockIdx.y;
+    const int i0 = blockIdx.z * 32;                       // first query row of this slice
     const int RR = p.RR, b1 = p.b1;
     const int64_t uaj = (int64_t)u * p.AJ + aj;
 
@@ -111,8 +117,8 @@ __global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
             const int r = cidx / CH, ch = cidx % CH;
             u32x4 a = {0u, 0u, 0u, 0u}, b = a;
             float dot = 0.f;
-            if (r < b1) {
-                const int64_t tok = p.qmap.row(a_q, r) + j_q;
+            if (i0 + r < b1) {
+                const int64_t tok = p.qmap.row(a_q, i0 + r) + j_q;
                 a = *(const u32x4*)(qg + tok * p.qs[1] * 2 + ch * 16);
                 b = *(const u32x4*)(dg + tok * p.os[1] * 2 + ch * 16);
                 if (saved) {                              // sum_r L dLm of row i is dO_i . O_i
@@ -214,7 +220,7 @@ __global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
-            lse[v] = st[min(i, b1 - 1)];
+            lse[v] = st[min(i0 + i, b1 - 1)];
             delta[v] = dls[i];
         }
     } else {
@@ -273,9 +279,9 @@ __global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
         tr0 = (uint32_t)(rl * kPitch + cl * 16 + (s16 & 1) * 8);
         tr1 = tr0 + 8 * kPitch;
     }
-    uint16_t* const dkb = p.dkbar + ((int64_t)u * RR * p.AJ + aj) * D;
-    uint16_t* const dyb = p.dy + ((int64_t)u * RR * p.AJ + aj) * D;
-    float* const dcp = p.dc + uaj * RR;
+    uint16_t* const dkb = p.dkbar + blockIdx.z * p.slab_rows + ((int64_t)u * RR * p.AJ + aj) * D;
+    uint16_t* const dyb = p.dy + blockIdx.z * p.slab_rows + ((int64_t)u * RR * p.AJ + aj) * D;
+    float* const dcp = p.dc + blockIdx.z * p.slab_dc + uaj * RR;
     uint16_t* const ds2p = p.ds2 + uaj * b1 * p.ds2_ld;
 
     request(0);
@@ -302,7 +308,7 @@ __global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
-                if (i < b1) ds2p[(int64_t)i * p.ds2_ld + r] = E::from_float(d[v]);
+                if (i0 + i < b1) ds2p[(int64_t)(i0 + i) * p.ds2_ld + r] = E::from_float(d[v]);
             }
         }
         u32x4 pl[2], pg[2];                              // B operands [n = r, k = i] for the two steps of 16 rows i
@@ -383,6 +389,43 @@ __global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
 }
 
 
+// slab 0 += slabs 1 .. nz - 1: 8 elements (16 bit) of dkbar / dy or one float of dc per thread
+template <class E>
+__global__ __launch_bounds__(256) void monarch_bwd_left_sum_kernel(uint16_t* dkbar, uint16_t* dy, int64_t slab_rows, float* dc,
+                                                                   int64_t slab_dc, int nz) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t n16 = slab_rows / 8;
+    if (t < 2 * n16) {
+        uint16_t* base = (t < n16 ? dkbar : dy) + (t < n16 ? t : t - n16) * 8;
+        float acc[8];
+        u32x4 w = *(const u32x4*)base;
+        const uint32_t w0[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc[2 * i] = E::to_float((uint16_t)(w0[i] & 0xffffu));
+            acc[2 * i + 1] = E::to_float((uint16_t)(w0[i] >> 16));
+        }
+        for (int z = 1; z < nz; ++z) {
+            const u32x4 x = *(const u32x4*)(base + z * slab_rows);
+            const uint32_t xx[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[2 * i] += E::to_float((uint16_t)(xx[i] & 0xffffu));
+                acc[2 * i + 1] += E::to_float((uint16_t)(xx[i] >> 16));
+            }
+        }
+        w.x = pack2<E>(acc[0], acc[1]); w.y = pack2<E>(acc[2], acc[3]); w.z = pack2<E>(acc[4], acc[5]); w.w = pack2<E>(acc[6], acc[7]);
+        *(u32x4*)base = w;
+    } else {
+        const int64_t c = t - 2 * n16;
+        if (c < slab_dc) {
+            float a = dc[c];
+            for (int z = 1; z < nz; ++z) a += dc[z * slab_dc + c];
+            dc[c] = a;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // dQ of the left factor, dQ[i, :] = s sum_r dS2[i, r] Kbar[r, :] per (unit, a, j), plus the right factor's part
 // (already reduced per (unit, k) by a library GEMM), written straight to the caller's dq rows.
@@ -417,6 +460,7 @@ __global__ __launch_bounds__(256) void monarch_bwd_dqa_kernel(DqaArgs p) {
     const bool aj_ok = ajraw < p.AJ;
     const int aj = aj_ok ? ajraw : p.AJ - 1;              // a wave past the end repeats the last column and stores nothing
     const int u = blockIdx.y;
+    const int i0 = blockIdx.z * 32;                       // first query row of this slice (b1 > 32: one slice per 32 rows)
     const int RR = p.RR, b1 = p.b1;
     const int64_t uaj = (int64_t)u * p.AJ + aj;
     const int nch = (RR + 31) / 32;
@@ -436,7 +480,7 @@ __global__ __launch_bounds__(256) void monarch_bwd_dqa_kernel(DqaArgs p) {
         }
     };
     // dS2 pieces of row i = m: r = 32 n + 16 ks + 4 hf + {0..3} and + 8 + {0..3}
-    const uint16_t* arow = p.ds2 + (uaj * b1 + min(m, b1 - 1)) * p.ds2_ld + 4 * hf;
+    const uint16_t* arow = p.ds2 + (uaj * b1 + min(i0 + m, b1 - 1)) * p.ds2_ld + 4 * hf;
     u32x4 acur[2], anext[2];
     auto load_a = [&](int n, u32x4 (&a)[2]) {
 #pragma unroll
@@ -510,7 +554,7 @@ __global__ __launch_bounds__(256) void monarch_bwd_dqa_kernel(DqaArgs p) {
     float* const out = p.dq + b * p.s0 + h * p.s2;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-        const int i = 8 * (v >> 2) + 4 * hf + (v & 3);
+        const int i = i0 + 8 * (v >> 2) + 4 * hf + (v & 3);
         if (i < b1) {
             const int64_t tok = p.map.row(a_blk, i) + j;
             const float* add = p.dqk + (((int64_t)u * b1 + i) * p.AJ + aj) * D;
@@ -523,7 +567,7 @@ __global__ __launch_bounds__(256) void monarch_bwd_dqa_kernel(DqaArgs p) {
 }  // namespace
 
 bool monarch_bwd_left_supported(int dtype, int D, int b1) {
-    return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b1 >= 1 && b1 <= 32;
+    return (dtype == SFM_BF16 || dtype == SFM_F16) && (D == 64 || D == 128) && b1 >= 1 && b1 <= 128;
 }
 
 int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int nf, int causal, float scale, const void* q,
@@ -548,7 +592,10 @@ int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int
     a.ds2 = (uint16_t*)ds2;
     a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.nf = nf; a.RR = nf * b1; a.causal = causal;
     a.scale = scale;
-    const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n);
+    const int nz = (b1 + 31) / 32;
+    a.slab_rows = (int64_t)n * a.RR * AJ * D;             // the caller's dkbar / dy / dc hold nz slabs
+    a.slab_dc = (int64_t)n * AJ * a.RR;
+    const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n, (unsigned)nz);
     const size_t ldsb = (size_t)4 * (D == 128 ? LeftLds<128>::kPerWave : LeftLds<64>::kPerWave);
     const void* fn = nullptr;
     if (dtype == SFM_BF16) fn = D == 128 ? (const void*)monarch_bwd_left_kernel<BF16, 128> : (const void*)monarch_bwd_left_kernel<BF16, 64>;
@@ -566,6 +613,12 @@ int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int
     } else {
         if (D == 128) hipLaunchKernelGGL((monarch_bwd_left_kernel<F16, 128>), grid, dim3(256), ldsb, stream, a);
         else hipLaunchKernelGGL((monarch_bwd_left_kernel<F16, 64>), grid, dim3(256), ldsb, stream, a);
+    }
+    if (nz > 1) {
+        const int64_t threads = 2 * (a.slab_rows / 8) + a.slab_dc;
+        const dim3 gs((unsigned)((threads + 255) / 256));
+        if (dtype == SFM_BF16) hipLaunchKernelGGL((monarch_bwd_left_sum_kernel<BF16>), gs, dim3(256), 0, stream, a.dkbar, a.dy, a.slab_rows, a.dc, a.slab_dc, nz);
+        else hipLaunchKernelGGL((monarch_bwd_left_sum_kernel<F16>), gs, dim3(256), 0, stream, a.dkbar, a.dy, a.slab_rows, a.dc, a.slab_dc, nz);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
@@ -591,7 +644,7 @@ int launch_monarch_bwd_dqa(int dtype, int D, int n, int b1, int b2, int AJ, int 
     a.map = map;
     a.ds2_ld = ds2_ld; a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.RR = nf * b1; a.H = H; a.unit0 = unit0;
     a.scale = scale;
-    const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n);
+    const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n, (unsigned)((b1 + 31) / 32));
     const size_t ldsb = (size_t)4 * 2 * 32 * 2 * D;
     if (dtype == SFM_BF16) {
         if (D == 128) hipLaunchKernelGGL((monarch_bwd_dqa_kernel<BF16, 128>), grid, dim3(256), ldsb, stream, a);

@@ -162,6 +162,9 @@ def test_480p_block_shape_bf16_one_head(bwd_path):
     (4, 20, 3, 9, 128, False, torch.bfloat16),     # 36 rows (f, k) per column: two chunks of the left factor, the second with 4 rows
     (8, 12, 2, 8, 64, False, torch.float16),       # 64 rows: two full chunks
     (6, 10, 6, 6, 128, True, torch.bfloat16),      # block-causal with two chunks: the visible rows end inside a chunk
+    (40, 12, 2, 2, 128, False, torch.bfloat16),    # b1 = 40: two 32-row query tiles in the left factor (partial slabs summed)
+    (90, 52, 1, 2, 128, False, torch.bfloat16),    # b1 = 90, b2 = 52: three frames of 30 x 52 tied per block, as the reference's default tiling
+    (100, 8, 3, 3, 64, True, torch.float16),       # four tiles, block-causal
 ])
 def test_16bit_gradients_across_the_fused_kernels_limits(h, w, Fq, Fk, D, causal, dtype):
     H = 2
@@ -283,3 +286,27 @@ def test_descriptor_errors():
     q = randn((1, 64, 1, 32), 140, torch.float32).to(DEV).requires_grad_(True)
     with pytest.raises(ValueError):                        # block-causal masking is defined for one iteration only
         mattn.monarch_attn(q, q, q, 1, 1, 1, 4, 8, block_causal_size=32, num_iters=2)
+
+
+@pytest.mark.parametrize("saved", [False, True])
+def test_three_frames_tied_480p_blocks_on_the_fused_kernels(saved):
+    """The reference's default tiling at 480p (f_tied = 3: b1 = 90, b2 = 52), 3 query frames against 6, through the tiling's
+    index maps; with the forward's saved output and statistics and recomputing them.  The fused chain must be the one
+    that runs: its workspace is smaller than the library chain's."""
+    h, w, H, D = 30, 52, 1, 128
+    dtype = torch.bfloat16
+    q0, do = (randn((1, 3 * h * w, H, D), 180 + i, dtype) for i in range(2))
+    k0, v0 = (randn((1, 6 * h * w, H, D), 182 + i, dtype) for i in range(2))
+    qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
+    monarch.monarch_attn(qr, kr, vr, 3, 1, 1, h, w).backward(do.double())
+    qd, kd, vd, dod = q0.to(DEV), k0.to(DEV), v0.to(DEV), do.to(DEV)
+    tiling = (3, 1, 1, h, w)
+    kept = {}
+    if saved:
+        out, stats = mattn._monarch_fwd_stats(qd, kd, vd, tiling, D ** -0.5, 0, 0)
+        assert stats is not None
+        kept = {"out": out, "stats": stats}
+    dq, dk, dv = mattn._monarch_bwd(qd, kd, vd, dod, tiling, D ** -0.5, 0, 0, **kept)
+    _close(dq, qr.grad, dtype)
+    _close(dk, kr.grad, dtype)
+    _close(dv, vr.grad, dtype)
