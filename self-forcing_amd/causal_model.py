@@ -120,9 +120,9 @@ class AttentionFlags:
         self.w_reduce = _env_int("MONARCH_ATTN_W_REDUCE", 1)
         self.use_framewise = bool(_env_int("MONARCH_ATTN_FRAMEWISE", 0))
         self.disable_monarch = bool(_env_int("DISABLE_MONARCH_ATTN", 0))
-        # no counterpart in the reference: keep a windowed KV cache (local_attn_size != -1) as a ring instead of
-        # shifting it down on every eviction (cache_step_ring)
-        self.ring_cache = bool(_env_int("SFM_RING_KV_CACHE", 0))
+        # no counterpart in the reference: a windowed KV cache (local_attn_size != -1) is kept as a ring instead of
+        # being shifted down on every eviction (cache_step_ring); 0 keeps the reference's row order in the cache
+        self.ring_cache = bool(_env_int("SFM_RING_KV_CACHE", 1))
         layers = os.getenv("MONARCH_ATTN_DISABLE_LAYERS")
         if layers is not None and block_num is not None and block_num in [int(x) for x in layers.split(",")]:
             self.disable_monarch = True
@@ -215,16 +215,37 @@ def cache_step_ring(kv_cache, current_start, num_new, frame_seqlen, sink_size):
     (causal_model.py:912-926 does the shift with a copy).  Attention over the cache is a sum over its rows, so
     the order in which block-frames sit in it does not change the result; the rotary phase is in the rows.
     Chunks must arrive in order (a re-run of the latest chunk lands in the same slot).
-    Returns (write_start, view_len, current_end), or None when chunks would straddle the end of the ring."""
+    Returns (write_start, view_len, current_end), or None when the chunk would straddle the end of the ring."""
     cache_len = kv_cache["k"].shape[1]
     sink = sink_size * frame_seqlen
     ring = cache_len - sink
     current_end = current_start + num_new
     if current_end <= cache_len:                       # still filling: positions are the global ones
         return current_start, current_end, current_end
-    if ring <= 0 or ring % num_new or current_start < sink or (current_start - sink) % num_new:
+    if ring <= 0 or current_start < sink:
         return None
-    return sink + (current_start - sink) % ring, cache_len, current_end
+    pos = sink + (current_start - sink) % ring
+    if pos + num_new > cache_len:
+        return None
+    return pos, cache_len, current_end
+
+
+def ring_to_window_order(kv_cache, sink_tokens):
+    """Leave the ring: rotate the rows after the sink frames so that the oldest comes first, which is the order the
+    reference's shift-down eviction keeps (causal_model.py:912-926), and set the local end as the reference has it for a
+    full window.  One copy of the cache; needed when a chunk arrives that would straddle the end of the ring."""
+    _sync_mirrors(kv_cache)
+    cache_len = kv_cache["k"].shape[1]
+    g_end = kv_cache["_global_end"]
+    if g_end > cache_len:
+        pos = sink_tokens + (g_end - sink_tokens) % (cache_len - sink_tokens)
+        if pos != sink_tokens:
+            for key in ("k", "v"):
+                t = kv_cache[key]
+                t[:, sink_tokens:] = torch.cat((t[:, pos:], t[:, sink_tokens:pos]), 1)
+        kv_cache["_local_end"] = cache_len
+        kv_cache.pop("_written", None)
+    kv_cache["_ring"] = False
 
 
 def cache_commit(kv_cache, current_end, local_end):
@@ -289,10 +310,14 @@ class CausalWanSelfAttention(nn.Module):
             self._rope = self.ops.rope_table(d, x.device)
 
         ring = None
+        if fl.ring_cache and self.local_attn_size != -1 and "_ring" not in kv_cache:
+            _sync_mirrors(kv_cache)
+            if kv_cache["_global_end"] > kv_cache["k"].shape[1]:
+                kv_cache["_ring"] = False       # filled past its window by a caller that shifts: keep that order
         if fl.ring_cache and self.local_attn_size != -1 and kv_cache.get("_ring", True):
             ring = cache_step_ring(kv_cache, current_start, s, frame_seqlen, self.sink_size)
             if ring is None and kv_cache.get("_ring"):
-                raise ValueError("ring KV cache: chunk sizes changed so that a chunk would straddle the end of the ring")
+                ring_to_window_order(kv_cache, self.sink_size * frame_seqlen)
             kv_cache["_ring"] = ring is not None
         if ring is not None:
             write_start, view_len, current_end = ring

@@ -129,7 +129,7 @@ def test_workspace_bytes_accounting():
     assert rc == 0 and nf32 == rows * 128 * 4 * 2 + rows * 4
     # iterated refinement on the MFMA kernels: 16-bit Kbar, Y and representatives, two fp32 scalars per row, and the left
     # factor's statistics (32 floats per (a, j) column); on the fp32 kernels (switch, or shapes the MFMA kernels do not
-    # take: b1 = 90 here) everything in float and no statistics
+    # take: b1 = 180 below) everything in float and no statistics
     rc, nit = _ws(_desc(num_iters=3), 1)
     assert rc == 0 and nit == rows * 128 * 2 * 3 + rows * 4 * 2 + 3 * 52 * 32 * 4
     lib = L.load()
@@ -140,9 +140,14 @@ def test_workspace_bytes_accounting():
     finally:
         lib.sfm_set_switches(old)
     assert rc == 0 and nsimt == rows * 128 * 4 * 3 + rows * 4 * 2
+    # three frames tied (b1 = 90): still the MFMA kernels, statistics rows padded to three 32-row query tiles
     rows3 = 1 * 52 * ((7 * 90 + 31) // 32 * 32)
     rc, ntied = _ws(_desc(num_iters=3, tiling=L.Tiling(3, 1, 1, 30, 52)), 1)
-    assert rc == 0 and ntied == (rows3 * 128 * 4 * 3 + rows3 * 4 * 2 + 255) // 256 * 256
+    assert rc == 0 and ntied == rows3 * 128 * 2 * 3 + rows3 * 4 * 2 + 52 * 96 * 4
+    # b1 = 180 is beyond them: the fp32 kernels
+    rows6 = 1 * 26 * ((7 * 180 + 31) // 32 * 32)
+    rc, nwide = _ws(_desc(num_iters=3, tiling=L.Tiling(3, 1, 1, 60, 26)), 1)
+    assert rc == 0 and nwide == (rows6 * 128 * 4 * 3 + rows6 * 4 * 2 + 255) // 256 * 256
 
 
 @pytest.mark.parametrize("kw,code", [

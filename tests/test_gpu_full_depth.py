@@ -6,7 +6,8 @@ same noise, same re-noising seeds.
 Stated end-to-end tolerance (bf16 weights and activations on both sides; the two sides' GEMMs sum in different orders
 and every layer adds to the residual stream, so the bar is wider than the per-operator one): clean latents of every
 chunk cosine > 0.9995 and max-abs < 3 % of the reference's range; K/V cache rows of the first and the last layer
-cosine > 0.999.  (Measured: cosine 0.99998, max-abs 1.0 % of the range, cache rows 0.99996.)"""
+cosine > 0.999.  (Measured: cosine 0.99998, max-abs 1.0 % of the range, cache rows 0.99996.)  The windowed case also
+holds the ring-ordered cache of the GPU side against the shifted cache of the reference's eviction."""
 import pytest
 import torch
 
@@ -22,18 +23,22 @@ def _cos(a, b):
     return torch.nn.functional.cosine_similarity(a.double().flatten().cpu(), b.double().flatten().cpu(), dim=0).item()
 
 
-@pytest.mark.parametrize("name,flags,chunks,steps", [
+@pytest.mark.parametrize("name,flags,chunks,steps,window", [
     # BASELINE configs[2]: framewise Monarch; one chunk, 4 denoising passes + the cache-refresh pass
-    ("c3", dict(use_framewise=True), 1, (1000, 750, 500, 250)),
+    ("c3", dict(use_framewise=True), 1, (1000, 750, 500, 250), -1),
     # configs[3]: reduce2xh tiling with a dense first chunk; the second chunk is the first Monarch one (6 cached
     # frames, a = 6, f = 12, b1 = 15); two denoising passes + the cache-refresh pass per chunk
-    ("c4", dict(use_framewise=True, h_reduce=2, use_dense_init=True), 2, (1000, 500)),
+    ("c4", dict(use_framewise=True, h_reduce=2, use_dense_init=True), 2, (1000, 500), -1),
+    # a window of 6 frames (local_attn_size = 6): the third chunk evicts the first.  The GPU side keeps the cache as a
+    # ring (its default), the CPU side shifts it down as the reference does (causal_model.py:912-926); one denoising pass
+    # + the cache-refresh pass per chunk
+    ("c3_window", dict(use_framewise=True), 3, (1000,), 6),
 ])
-def test_full_depth_rollout_against_the_oracle_model(name, flags, chunks, steps):
+def test_full_depth_rollout_against_the_oracle_model(name, flags, chunks, steps, window):
     torch.set_num_threads(16)
-    cfg = cm.WAN_CONFIGS["1.3B"]
+    cfg = dict(cm.WAN_CONFIGS["1.3B"], local_attn_size=window)
     torch.manual_seed(0)
-    ref = cm.CausalWanModel(ops=OracleOps(), attention_flags=flags, **cfg)
+    ref = cm.CausalWanModel(ops=OracleOps(), attention_flags=dict(flags, ring_cache=False), **cfg)
     ref.init_weights(zero_head=False)
     ref = ref.to(torch.bfloat16).eval()
     dev = cm.CausalWanModel(attention_flags=flags, **cfg).to(torch.bfloat16).eval()
@@ -43,12 +48,17 @@ def test_full_depth_rollout_against_the_oracle_model(name, flags, chunks, steps)
     g = torch.Generator().manual_seed(0)
     noise = torch.randn(1, 3 * chunks, 16, 60, 104, generator=g).to(torch.bfloat16)
     ctx = torch.randn(1, 512, 4096, generator=g).to(torch.bfloat16)
-    kw = dict(denoising_step_list=steps, num_cache_frames=3 * chunks)
+    kw = dict(denoising_step_list=steps, num_cache_frames=3 * chunks, local_attn_size=window)
     pipe_ref = pl.CausalInferencePipeline(pl.WanDiffusionWrapper(ref), **kw)
     pipe_dev = pl.CausalInferencePipeline(pl.WanDiffusionWrapper(dev), **kw)
     out = pipe_dev.inference(noise.to("cuda:0"), ctx.to("cuda:0"))
     want = pipe_ref.inference(noise, ctx)
     assert torch.isfinite(out).all() and want.float().abs().max() > 0.1
+    if window != -1:
+        for layer in (0, 29):       # the ring did wrap; put its rows into the reference's order for the comparison below
+            assert pipe_dev.kv_cache1[layer]["_ring"] and pipe_dev.kv_cache1[layer]["_local_end"] == 3 * 1560
+            assert pipe_dev.kv_cache1[layer]["k"].shape[1] == window * 1560
+            cm.ring_to_window_order(pipe_dev.kv_cache1[layer], 0)
     rng = want.float().abs().max().item()
     report = []
     for c in range(chunks):

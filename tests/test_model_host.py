@@ -186,3 +186,36 @@ def test_ring_cache_falls_back_when_chunks_would_straddle_the_ring():
     assert cm.cache_step_ring(kv, 54, 18, 6, 3) == (18, 54, 72)
     assert cm.cache_step_ring(kv, 72, 18, 6, 3) == (36, 54, 90)
     assert cm.cache_step_ring(kv, 90, 18, 6, 3) == (18, 54, 108)
+    # chunk sizes may change as long as no chunk straddles: two frames at the start of the ring, then four to its end
+    assert cm.cache_step_ring(kv, 108, 12, 6, 3) == (36, 54, 120)
+    assert cm.cache_step_ring(kv, 120, 6, 6, 3) == (48, 54, 126)
+    assert cm.cache_step_ring(kv, 126, 18, 6, 3) == (18, 54, 144)
+    assert cm.cache_step_ring(kv, 144, 24, 6, 3) is None
+
+
+def test_leaving_the_ring_restores_the_reference_row_order():
+    """Window of 5 frames, one sink frame, chunks of 2, 2, 1 (fills), 2 (ring), then 3 (would straddle) and 1: the same
+    rollout with the shifting cache from the start holds the same rows in the same places afterwards."""
+    outs, caches = [], []
+    for ring in (False, True):
+        torch.manual_seed(0)
+        att = cm.CausalWanSelfAttention(16, 2, 5, 1, True, 1e-6, 0, (2, 3), None,
+                                        cm.AttentionFlags(0, disable_monarch=True, ring_cache=ring),
+                                        OracleOps(compute_dtype=torch.float64)).double().eval()
+        kv = {"k": torch.zeros(1, 30, 2, 8, dtype=torch.float64), "v": torch.zeros(1, 30, 2, 8, dtype=torch.float64),
+              "global_end_index": torch.tensor([0]), "local_end_index": torch.tensor([0])}
+        g = torch.Generator().manual_seed(1)
+        ys, start = [], 0
+        for frames in (2, 2, 1, 2, 3, 1):
+            x = torch.randn(1, frames * 6, 16, generator=g, dtype=torch.float64)
+            with torch.no_grad():
+                ys.append(att(x, (frames, 2, 3), kv, start * 6))
+            if frames == 2 and start >= 5:
+                assert kv.get("_ring", False) == ring
+            start += frames
+        assert not kv.get("_ring", False)
+        outs.append(torch.cat(ys, 1))
+        caches.append((kv["k"].clone(), kv["v"].clone(), int(kv["global_end_index"]), int(kv["local_end_index"])))
+    assert torch.allclose(outs[0], outs[1], atol=1e-12)
+    assert torch.equal(caches[0][0], caches[1][0]) and torch.equal(caches[0][1], caches[1][1])
+    assert caches[0][2:] == caches[1][2:]
