@@ -143,3 +143,105 @@ def test_drawn_case_against_the_oracle(seed):
     if not partial and n_old:
         _grad_close(kc.grad[:, :n_old], kor.grad, dtype)
         _grad_close(vc.grad[:, :n_old], vor.grad, dtype)
+
+
+# ---- the other operators of the path: dense attention (forward, gradients), the q/k prologue, the block's linear layers ----
+
+OTHER = ("dense", "dense_grad", "prologue", "linear")
+
+
+@pytest.mark.parametrize("seed", range(160))
+def test_drawn_case_of_the_other_operators(seed):
+    from oracle import blocks, dense, prologue
+    r = random.Random(10_000 + seed)
+    kind = OTHER[seed % len(OTHER)]
+    if kind in ("dense", "dense_grad"):
+        grad = kind == "dense_grad"
+        B, H, D = r.choice((1, 1, 2)), r.choice((1, 2, 3, 5)), r.choice((64, 128)) if grad else r.choice((32, 64, 128))
+        Lq = r.choice((r.randint(1, 130), r.randint(131, 700), r.randint(701, 2600 if not grad else 1200)))
+        Lk = r.choice((r.randint(1, 70), r.randint(71, 600), r.randint(601, 3000 if not grad else 1500)))
+        dtype = r.choice((torch.bfloat16, torch.float16)) if grad else r.choice((torch.bfloat16, torch.float16, torch.float32))
+        print(dict(kind=kind, B=B, Lq=Lq, Lk=Lk, H=H, D=D, dtype=dtype), flush=True)
+        q0, k0, v0, do = (randn((B, n, H, D), 2000 * seed + i, dtype) for i, n in enumerate((Lq, Lk, Lk, Lq)))
+        if not grad:
+            ref, lse_ref = dense.attention(q0, k0, v0, dtype=torch.float32, return_lse=True)
+            out, lse = sfa.attention.attention(q0.to(DEV), k0.to(DEV), v0.to(DEV), dtype=dtype, return_lse=True)
+            if dtype == torch.float32:
+                assert max_abs(out, ref) < 1e-5
+            else:
+                assert_close_16bit(out, ref, dtype)
+            assert max_abs(lse, lse_ref) < 1e-3
+            return
+        qr, kr, vr = _leaf(q0.double()), _leaf(k0.double()), _leaf(v0.double())
+        dense.attention(qr, kr, vr).backward(do.double())
+        qd, kd, vd = _leaf(q0, DEV), _leaf(k0, DEV), _leaf(v0, DEV)
+        sfa.attention.attention(qd, kd, vd, dtype=dtype).backward(do.to(DEV))
+        tol = 1e-2 if dtype == torch.bfloat16 else 1e-3
+        for got, want in ((qd.grad, qr.grad), (kd.grad, kr.grad), (vd.grad, vr.grad)):
+            got, want = got.float().cpu(), want.float()
+            assert torch.allclose(got, want, atol=tol * max(1.0, want.abs().max().item()), rtol=tol)
+        return
+
+    if kind == "prologue":
+        f_tied, h_reduce, w_reduce = r.choice((1, 1, 3)), r.choice((1, 2, 3)), r.choice((1, 1, 2, 4))
+        h, w = h_reduce * r.randint(1, 12), w_reduce * r.randint(1, 20)
+        F, H, D = f_tied * r.randint(1, 3), r.choice((1, 2, 5, 12)), r.choice((64, 128))
+        B, dtype = r.choice((1, 2)), r.choice((torch.bfloat16, torch.float16, torch.float32))
+        start_frame = r.randint(0, 40)
+        print(dict(kind=kind, tiling=(f_tied, h_reduce, w_reduce, h, w), F=F, B=B, H=H, D=D, dtype=dtype, start=start_frame), flush=True)
+        S, Cd = F * h * w, H * D
+        xq, xk, xv = (randn((B, S, Cd), 3000 * seed + i, dtype) for i in range(3))
+        wq, wk = ((1 + 0.1 * randn((Cd,), 3000 * seed + 3 + i, torch.float32)).to(dtype) for i in range(2))
+        pre = f_tied * h * w * r.randint(0, 2)
+        qr, kr, vr = prologue.qk_prologue(xq, xk, xv, wq, wk, H, (F, h, w), start_frame)
+        kc = torch.zeros(B, pre + S + 7, H, D, dtype=dtype, device=DEV)
+        vc = torch.zeros_like(kc)
+        rope = sfa.prologue.rope_table(D, device=DEV)
+        qo = sfa.prologue.qk_prologue(xq.to(DEV), xk.to(DEV), xv.to(DEV), wq.to(DEV), wk.to(DEV), H, (F, h, w), start_frame,
+                                      rope, kc, vc, pre, f_tied, h_reduce, w_reduce)
+        kref = blocks.to_blocks(kr, f_tied, h_reduce, w_reduce, h, w).reshape(B, S, H, D)
+        vref = blocks.to_blocks(vr, f_tied, h_reduce, w_reduce, h, w).reshape(B, S, H, D)
+        assert torch.equal(vc[:, pre:pre + S].cpu(), vref)
+        assert (kc[:, :pre] == 0).all() and (kc[:, pre + S:] == 0).all() and (vc[:, pre + S:] == 0).all()
+        one_step = {torch.bfloat16: 2 ** -7, torch.float16: 2 ** -10, torch.float32: 2 ** -21}[dtype]
+        for got, ref in ((qo, qr), (kc[:, pre:pre + S], kref)):
+            g, rf = got.float().cpu(), ref.float().cpu()
+            assert ((g - rf).abs() / rf.abs().clamp_min(1.0)).max().item() <= 2 * one_step
+        return
+
+    # linear: out = epilogue(x W^T + b) against fp32 matmul followed by the eager chain's roundings
+    dtype = r.choice((torch.bfloat16, torch.float16))
+    M, N, K = r.choice((r.randint(1, 300), r.randint(301, 2000))), 8 * r.randint(1, 160), 64 * r.randint(1, 24)
+    epi = r.choice(("none", "none", "gelu_tanh", "gate_residual"))
+    tile_rows = r.choice((0, 128, 256))
+    print(dict(kind=kind, M=M, N=N, K=K, dtype=dtype, epilogue=epi, tile_rows=tile_rows), flush=True)
+    x = randn((1, M, K), 4000 * seed, dtype).to(DEV)
+    wt = (randn((N, K), 4000 * seed + 1, dtype) * K ** -0.5).to(dtype).to(DEV)
+    b = randn((N,), 4000 * seed + 2, dtype).to(DEV) if r.random() < 0.7 else None
+    assert sfa.linear.supported(x, wt)
+    y = x.float() @ wt.float().t()
+    y = (y + b.float() if b is not None else y).to(dtype)
+    kw = {}
+    if epi == "gelu_tanh":
+        ref = torch.nn.functional.gelu(y.float(), approximate="tanh").to(dtype)
+        # a product one rounding step away moves the result by |gelu'(y)| steps of y, which in the left tail is many steps
+        # of the tiny result: the steps are measured at |gelu(y)| + |y gelu'(y)| (as tests/test_gpu_linear.py does)
+        yl = y.float().requires_grad_(True)
+        gl = torch.nn.functional.gelu(yl, approximate="tanh")
+        gl.sum().backward()
+        scale = gl.detach().abs() + (yl.detach() * yl.grad).abs()
+    elif epi == "gate_residual":
+        res = randn((1, M, N), 4000 * seed + 3, dtype).to(DEV)
+        gate = randn((1, 1, 1, N), 4000 * seed + 4, dtype).to(DEV)
+        yg = (y.float() * gate.reshape(1, 1, N).float()).to(dtype)
+        ref = (res.float() + yg.float()).to(dtype)
+        scale = res.float().abs() + yg.float().abs()
+        kw = dict(res=res.clone(), gate=gate)
+    else:
+        ref, scale = y, None
+    out = sfa.linear.linear(x, wt, b, epilogue=epi, tile_rows=tile_rows, **kw)
+    unit = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+    err = (out.float() - ref.float()).abs()
+    mag = (ref.float().abs() if scale is None else scale).clamp_min(2.0 ** -6)
+    steps = {"none": 1, "gelu_tanh": 2, "gate_residual": 3}[epi]
+    assert (err <= steps * unit * mag).all(), (err.max().item(), (err / mag).max().item())
