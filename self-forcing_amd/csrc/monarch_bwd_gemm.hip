@@ -570,6 +570,9 @@ int run(const MonarchBwdArgs& g, int n, void* workspace, hipStream_t stream) {
         f1.ws_aj = 1;
         f1.ws_row = (uint32_t)(nf * AJ);
         f1.ws_f = (uint32_t)AJ;
+        f1.cl_unit = f1.ws_unit;         // c sits where its scratch row does: [row][(a, j)]
+        f1.cl_aj = 1;
+        f1.cl_row = 1;
         if (!cx.status) cx.status = launch_monarch_step1(f1, left_dtype<E>(), n, stream);
     } else {
         // 1. S1 = Qk Kk^T per (u, k)

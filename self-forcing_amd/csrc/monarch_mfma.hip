@@ -209,7 +209,7 @@ void monarch_step1_kernel(MonarchArgs p) {
             for (int ds = 0; ds < DS; ++ds) qb[ds] = *(const u32x4*)(qrow + 16 * ds);
 #pragma unroll
             for (int ds = 0; ds < DS; ++ds) asm volatile("" : "+v"(qb[ds]));      // waited for here, before the tile loads below
-            cloff = (uint32_t)(ca * b2 + cj) * p.ws_aj * 4;
+            cloff = (uint32_t)(ca * b2 + cj) * p.cl_aj * 4;
 #pragma unroll
             for (int rb = 0; rb < 4; ++rb) {
                 const int sg = min(wave * 32 + (m & 7) + 8 * rb, cur.ncols - 1);
@@ -270,7 +270,10 @@ void monarch_step1_kernel(MonarchArgs p) {
                 pb[st].w = pack2<E>(s[t][v0 + 6] * inv_l, s[t][v0 + 7] * inv_l);
             }
             // sum_l R log2 R (both halves of a column hold, and store, the same value)
-            *(float*)((char*)p.cl + (size_t)srow * 4 + cloff) = ent * inv_l - (mx + log2f(sum));
+            {
+                const size_t clrow = (size_t)cur.ul * p.cl_unit + (size_t)((uint32_t)cur.k * p.ws_row + (uint32_t)cur.f * fstep) * p.cl_row;
+                *(float*)((char*)p.cl + clrow * 4 + cloff) = ent * inv_l - (mx + log2f(sum));
+            }
             if (WR) {
                 // R[l] for l = 16 st + 0..15: the lower half of the wave holds 0..3 and 8..11, the upper half 4..7 and
                 // 12..15; exchanging the lower half's second pair with the upper half's first leaves 8 consecutive values
@@ -399,7 +402,8 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
     const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj;   // in rows; the rows of one (a, j) are consecutive
     const char* kb = (const char*)p.kbar + blk * (2 * D);
     const char* yb = (const char*)p.y + blk * (2 * D);
-    const char* clp = (const char*)(p.cl + blk);
+    const char* clp = (const char*)(p.cl + (int64_t)ul * p.cl_unit + (int64_t)(a * b2 + j) * p.cl_aj);
+    const uint32_t cl_ld = p.cl_row * 4;                  // bytes between the cl values of consecutive rows
 
     char* const wl = lds_s2 + wave * L::kWave;
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)wl;
@@ -432,7 +436,7 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
             s1_load_lds16(kb, off, dst + (uint32_t)g * 1024);
             s1_load_lds16(yb, off, dst + L::kTile + (uint32_t)g * 1024);
         }
-        s2_load_lds4(clp, (uint32_t)(32 * n + m) * 4, dst + 2 * L::kTile);     // cl of the chunk's 32 rows (twice)
+        s2_load_lds4(clp, (uint32_t)(32 * n + m) * cl_ld, dst + 2 * L::kTile);     // cl of the chunk's 32 rows (twice)
     };
     const uint32_t a_off = (uint32_t)m * L::kPitch + (uint32_t)((hf ^ s1_swz<CPR>(m)) << 4);   // Kbar row m as the logits' A operand
     uint32_t tr[DT][2];            // Y^T as the output's A operand: transposing reads, as in step 1
@@ -595,7 +599,8 @@ __global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
     const int nch = (r_lim + 31) / 32;
     const int64_t blk = (int64_t)ul * p.ws_unit + (int64_t)(a * b2 + j) * p.ws_aj;
     const char* kb = (const char*)p.kbar + blk * (2 * D);
-    const char* clp = (const char*)(p.cl + blk);
+    const char* clp = (const char*)(p.cl + (int64_t)ul * p.cl_unit + (int64_t)(a * b2 + j) * p.cl_aj);
+    const uint32_t cl_ld = p.cl_row * 4;
     char* repb = (char*)p.rep + blk * (2 * D);
     float* wgt = p.wgt + blk;
 
@@ -652,7 +657,7 @@ __global__ __launch_bounds__(256) void monarch_rep_kernel(MonarchArgs p) {
             const uint32_t off = (uint32_t)min(32 * n + r, r_lim - 1) * (2 * D) + (uint32_t)c * 16;
             s1_load_lds16(kb, off, dst + (uint32_t)g * 1024);
         }
-        s2_load_lds4(clp, (uint32_t)(32 * n + m) * 4, dst + L::kTile);
+        s2_load_lds4(clp, (uint32_t)(32 * n + m) * cl_ld, dst + L::kTile);
     };
     const uint32_t b_off = (uint32_t)m * L::kPitch + (uint32_t)((hf ^ s1_swz<CPR>(m)) << 4);   // row m of a 32-row tile as an MFMA operand
     uint32_t tr[DT][2];            // Q^T as the representatives' A operand: transposing reads, as step 2 reads Y^T

@@ -324,6 +324,13 @@ static void init_args(const sfm_monarch_desc* desc, const MonarchPlan& pl, Monar
     // which the rows a step-1 workgroup writes are consecutive instead, measured the same for step 1.)
     a.ws_aj = (uint32_t)pl.r_pad;
     a.ws_row = 1;
+    a.cl_unit = a.ws_unit;
+    a.cl_aj = a.ws_aj;
+    a.cl_row = 1;
+    if (pl.mfma || pl.iter_mfma) {       // row-major cl: a tile's columns are contiguous (see MonarchArgs)
+        a.cl_aj = 1;
+        a.cl_row = (uint32_t)(pl.na * pl.b2);
+    }
     // step 1 takes as many query block-frames per workgroup as fit 256 (a, j) columns
     int a_max = 256 / pl.b2;
     if (a_max < 1) a_max = 1;

@@ -132,7 +132,7 @@ struct MonarchArgs {
     void* out;
     void* kbar;      // [units_per_pass][na][b2][r_pad][D]   16-bit (MFMA path) or float (generic path)
     void* y;         // same shape
-    float* cl;       // [units_per_pass][na][b2][r_pad]      sum_l R log2 R  (log2 units)
+    float* cl;       // [units_per_pass][na][b2][r_pad]      sum_l R log2 R  (log2 units); MFMA kernels: see cl_unit below
     void* rep;       // iterated refinement only: query representatives, same shape and element type as kbar
     float* wgt;      // iterated refinement only: their weights, same shape as cl
     int iter_mode;   // MFMA step 1: 0 = queries from q; 1 = first refinement pass (q, logits / (1 + 1e-6));
@@ -142,6 +142,11 @@ struct MonarchArgs {
     // scratch row index of (unit ul, a, j, r) = ul*ws_unit + (a*b2 + j)*ws_aj + r*ws_row
     uint32_t ws_unit, ws_aj, ws_row;
     uint32_t ws_f;   // MFMA step 1 only: rows between consecutive kv block-frames f of one (unit, a, j, k); 0 = b1 * ws_row
+    // MFMA kernels only: cl of the scratch row above sits at ul*cl_unit + (a*b2 + j)*cl_aj + (r*ws_row)*cl_row.  The forward
+    // keeps cl row-major (cl_aj = 1, cl_row = na*b2): the columns of one K/V tile are then one contiguous run, which step 1
+    // writes as whole cache lines (one float per (a, j)-major row is a partial write of a 32-byte sector each, and 1.2 M of
+    // those per call cost step 1 7 % of its time); step 2 gathers its column with that stride, out of the L2.
+    uint32_t cl_unit, cl_aj, cl_row;
     void* rb;        // MFMA step 1 only, optional: the right factor R, 16 bit, 64 values per scratch row (same row index)
     float* stats;    // MFMA step 2 only, optional: log2-sum-exp of each query row's left-factor logits,
     uint32_t stats_ld;   // at ((b*H + h) * na*b2 + a*b2 + j) * stats_ld + i
