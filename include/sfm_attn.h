@@ -324,8 +324,11 @@ int sfm_probe_mfma_bf16(int32_t iters, void* stream, float* tflops);
  * rows of row_bytes (contiguous) and writes rows_out rows of row_bytes to each of two matrices, row r of item t at row
  * index r * tiles + t (the scatter of step 1's scratch), with non-temporal stores if `nontemporal` != 0.  The caller
  * supplies `workspace` (device memory, 16-byte aligned, >= tiles * (2 rows_in + 2 rows_out) * row_bytes bytes; its
- * contents are read and overwritten).  Runs on `stream`, waits, and returns the mean duration of one pass in
- * microseconds: the floor for this traffic on this machine, which bench.py reports beside step 1's own duration. */
+ * contents are read and overwritten).  A workspace with room for several copies of the input (up to 8 are used:
+ * tiles * (2 rows_in * copies + 2 rows_out) * row_bytes bytes) makes consecutive passes read different copies; with a
+ * single copy below the size of the memory-side cache (256 MB) the reads are served from that cache and cost nothing,
+ * which the operator's own reads in a model are not.  Runs on `stream`, waits, and returns the mean duration of one
+ * pass in microseconds: the floor for this traffic on this machine, which bench.py reports beside step 1's duration. */
 int sfm_probe_tile_traffic(int32_t tiles, int32_t rows_in, int32_t rows_out, int32_t row_bytes, int32_t nontemporal,
                            void* workspace, size_t workspace_bytes, void* stream, float* us);
 

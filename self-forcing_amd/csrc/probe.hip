@@ -161,18 +161,24 @@ extern "C" int sfm_probe_tile_traffic(int32_t tiles, int32_t rows_in, int32_t ro
         set_error("sfm_probe_tile_traffic: hipEventCreate failed");
         return SFM_ERR_HIP;
     }
-    const u32x4* in = (const u32x4*)workspace;
     u32x4* o0 = (u32x4*)((char*)workspace + in_bytes);
     u32x4* o1 = (u32x4*)((char*)workspace + in_bytes + out_bytes);
+    // Consecutive passes read different copies of the input (as many as the workspace holds, at most 8): with a single
+    // copy smaller than the memory-side cache the reads of every pass after the first are served from that cache and the
+    // pass measures the writes only.
+    int copies = (int)((workspace_bytes - 2 * out_bytes) / in_bytes);
+    if (copies > 8) copies = 8;
     const int wgs = tiles < 2 * cu_count() ? tiles : 2 * cu_count();
-    const int reps = 5;
-    auto launch = [&] {
+    const int reps = 8;
+    auto launch = [&](int i) {
+        const int cp = i % copies;                           // copy 0 at the start, the others behind the two outputs
+        const u32x4* in = (const u32x4*)((char*)workspace + (cp ? 2 * out_bytes + (size_t)cp * in_bytes : 0));
         if (nontemporal) hipLaunchKernelGGL(tile_traffic_kernel<true>, dim3(wgs), dim3(320), 0, st, in, o0, o1, tiles, rows_in, rows_out, row_bytes / 16);
         else hipLaunchKernelGGL(tile_traffic_kernel<false>, dim3(wgs), dim3(320), 0, st, in, o0, o1, tiles, rows_in, rows_out, row_bytes / 16);
     };
-    launch();                                                // warm-up
+    launch(0);                                               // warm-up
     (void)hipEventRecord(e0, st);
-    for (int i = 0; i < reps; ++i) launch();
+    for (int i = 0; i < reps; ++i) launch(i + 1);
     (void)hipEventRecord(e1, st);
     hipError_t e = hipEventSynchronize(e1);
     float ms = 0.f;
