@@ -65,9 +65,15 @@ __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
     const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
-    const int q0 = blockIdx.x * (32 * NW) + wave * 32;
+    // the query blocks of one (batch, head) go to one XCD: its K / V rows are fetched from memory once, not once per XCD
     const int nq = p.q_tokens, nk = p.kv_tokens;
+    const int nqb = (nq + 32 * NW - 1) / (32 * NW);
+    const int total = nqb * p.B * p.H;
+    const int item = xcd_item(total);
+    if (item >= total) return;
+    const int unit = item / nqb;
+    const int b = unit / p.H, h = unit % p.H;
+    const int q0 = (item - unit * nqb) * (32 * NW) + wave * 32;
 
     const char* kg = (const char*)(kp + (int64_t)b * p.k_stride[0] + (int64_t)h * p.k_stride[2]);
     const char* vg = (const char*)(vp + (int64_t)b * p.v_stride[0] + (int64_t)h * p.v_stride[2]);
@@ -415,7 +421,8 @@ int launch_dense(const sfm_dense_desc& d, const void* q, const void* k, const vo
                 set_error("hipFuncSetAttribute failed: %s", hipGetErrorString(e));
                 return SFM_ERR_HIP;
             }
-            dim3 grid((d.q_tokens + 32 * nw - 1) / (32 * nw), d.B * d.H);
+            const int total = (d.q_tokens + 32 * nw - 1) / (32 * nw) * d.B * d.H;
+            dim3 grid(xcd_grid(total));
             hipLaunchKernelGGL(kern, grid, dim3(64 * nw), ldsb, stream, d, qq, kk, vv, oo, lse);
             return SFM_OK;
         };

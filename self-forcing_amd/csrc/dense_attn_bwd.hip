@@ -132,8 +132,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
     const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
-    const int i = blockIdx.x * 128 + wave * 32 + m;
+    // the query blocks of one (batch, head) go to one XCD, which then fetches that head's K / V rows once
+    const int nblk = (p.Sq + 127) / 128;
+    const int item = xcd_item(nblk * p.B * p.H);
+    if (item >= nblk * p.B * p.H) return;
+    const int bh = item / nblk, b = bh / p.H, h = bh % p.H;
+    const int i = (item - bh * nblk) * 128 + wave * 32 + m;
     const int ic = min(i, p.Sq - 1);
 
     const char* qrow = p.q + ((int64_t)b * p.qs[0] + (int64_t)ic * p.qs[1] + (int64_t)h * p.qs[2]) * 2 + 16 * hf;
@@ -276,8 +280,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
     const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
-    const int l = p.kv0 + blockIdx.x * 128 + wave * 32 + m;
+    // the key blocks of one (batch, head) go to one XCD, which then fetches that head's q / dO rows once
+    const int nblk = (p.kv1 - p.kv0 + 127) / 128;
+    const int item = xcd_item(nblk * p.B * p.H);
+    if (item >= nblk * p.B * p.H) return;
+    const int bh = item / nblk, b = bh / p.H, h = bh % p.H;
+    const int l = p.kv0 + (item - bh * nblk) * 128 + wave * 32 + m;
     const int lc = min(l, p.kv1 - 1);
 
     const char* krow = p.k + ((int64_t)b * p.ks[0] + (int64_t)lc * p.ks[1] + (int64_t)h * p.ks[2]) * 2 + 16 * hf;
@@ -461,9 +469,9 @@ int launch_t(const DenseBwdArgs& a, hipStream_t stream) {
             return SFM_ERR_HIP;
         }
     }
-    hipLaunchKernelGGL((dense_bwd_dq_kernel<E, D>), dim3((a.Sq + 127) / 128, a.B * a.H), dim3(256), lds_dq, stream, a);
+    hipLaunchKernelGGL((dense_bwd_dq_kernel<E, D>), dim3(xcd_grid((a.Sq + 127) / 128 * a.B * a.H)), dim3(256), lds_dq, stream, a);
     if (a.kv1 > a.kv0)
-        hipLaunchKernelGGL((dense_bwd_dkv_kernel<E, D>), dim3((a.kv1 - a.kv0 + 127) / 128, a.B * a.H), dim3(256), lds_dkv, stream, a);
+        hipLaunchKernelGGL((dense_bwd_dkv_kernel<E, D>), dim3(xcd_grid((a.kv1 - a.kv0 + 127) / 128 * a.B * a.H)), dim3(256), lds_dkv, stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_error("dense backward: launch failed: %s", hipGetErrorString(e));

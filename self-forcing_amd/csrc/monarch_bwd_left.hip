@@ -49,6 +49,7 @@ struct LeftArgs {
     int b1, b2, AJ, nf, RR, causal;
     float scale;
     int64_t slab_rows, slab_dc;   // elements between the dkbar / dy slabs and between the dc slabs of two query-row tiles
+    int nunits, nz;               // units of this launch, 32-row query slices per column
 };
 
 typedef short bl_s16x4 __attribute__((ext_vector_type(4)));
@@ -94,11 +95,17 @@ __global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
 
     const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int ajraw = blockIdx.x * 4 + wave;
+    // work item = (unit, group of 4 columns, slice), slices fastest, one contiguous range of items per XCD: the slices
+    // of a column, which stream the same Kbar / Y rows, meet in one L2
+    const int njg = (p.AJ + 3) / 4;
+    const int item = xcd_item(njg * p.nunits * p.nz);
+    if (item >= njg * p.nunits * p.nz) return;
+    const int zi = item % p.nz, jg = (item / p.nz) % njg;
+    const int ajraw = jg * 4 + wave;
     const bool aj_ok = ajraw < p.AJ;
     const int aj = aj_ok ? ajraw : p.AJ - 1;              // a wave past the end repeats the last column and stores nothing
-    const int u = blockIdx.y;
-    const int i0 = blockIdx.z * 32;                       // first query row of this slice
+    const int u = item / (p.nz * njg);
+    const int i0 = zi * 32;                               // first query row of this slice
     const int RR = p.RR, b1 = p.b1;
     const int64_t uaj = (int64_t)u * p.AJ + aj;
 
@@ -279,9 +286,9 @@ __global__ __launch_bounds__(256) void monarch_bwd_left_kernel(LeftArgs p) {
         tr0 = (uint32_t)(rl * kPitch + cl * 16 + (s16 & 1) * 8);
         tr1 = tr0 + 8 * kPitch;
     }
-    uint16_t* const dkb = p.dkbar + blockIdx.z * p.slab_rows + ((int64_t)u * RR * p.AJ + aj) * D;
-    uint16_t* const dyb = p.dy + blockIdx.z * p.slab_rows + ((int64_t)u * RR * p.AJ + aj) * D;
-    float* const dcp = p.dc + blockIdx.z * p.slab_dc + uaj * RR;
+    uint16_t* const dkb = p.dkbar + zi * p.slab_rows + ((int64_t)u * RR * p.AJ + aj) * D;
+    uint16_t* const dyb = p.dy + zi * p.slab_rows + ((int64_t)u * RR * p.AJ + aj) * D;
+    float* const dcp = p.dc + zi * p.slab_dc + uaj * RR;
     uint16_t* const ds2p = p.ds2 + uaj * b1 * p.ds2_ld;
 
     request(0);
@@ -442,6 +449,7 @@ struct DqaArgs {
     TokMap map;
     int ds2_ld, b1, b2, AJ, RR, H, unit0;
     float scale;
+    int nunits, nz;               // units of this launch, 32-row query slices per column
 };
 
 
@@ -456,11 +464,15 @@ __global__ __launch_bounds__(256) void monarch_bwd_dqa_kernel(DqaArgs p) {
 
     const int tid = threadIdx.x, lane = tid & 63, m = lane & 31, hf = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int ajraw = blockIdx.x * 4 + wave;
+    const int njg = (p.AJ + 3) / 4;                       // work items as in monarch_bwd_left_kernel
+    const int item = xcd_item(njg * p.nunits * p.nz);
+    if (item >= njg * p.nunits * p.nz) return;
+    const int zi = item % p.nz, jg = (item / p.nz) % njg;
+    const int ajraw = jg * 4 + wave;
     const bool aj_ok = ajraw < p.AJ;
     const int aj = aj_ok ? ajraw : p.AJ - 1;              // a wave past the end repeats the last column and stores nothing
-    const int u = blockIdx.y;
-    const int i0 = blockIdx.z * 32;                       // first query row of this slice (b1 > 32: one slice per 32 rows)
+    const int u = item / (p.nz * njg);
+    const int i0 = zi * 32;                               // first query row of this slice (b1 > 32: one slice per 32 rows)
     const int RR = p.RR, b1 = p.b1;
     const int64_t uaj = (int64_t)u * p.AJ + aj;
     const int nch = (RR + 31) / 32;
@@ -595,7 +607,9 @@ int launch_monarch_bwd_left(int dtype, int D, int n, int b1, int b2, int AJ, int
     const int nz = (b1 + 31) / 32;
     a.slab_rows = (int64_t)n * a.RR * AJ * D;             // the caller's dkbar / dy / dc hold nz slabs
     a.slab_dc = (int64_t)n * AJ * a.RR;
-    const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n, (unsigned)nz);
+    a.nunits = n;
+    a.nz = nz;
+    const dim3 grid((unsigned)xcd_grid((AJ + 3) / 4 * n * nz));
     const size_t ldsb = (size_t)4 * (D == 128 ? LeftLds<128>::kPerWave : LeftLds<64>::kPerWave);
     const void* fn = nullptr;
     if (dtype == SFM_BF16) fn = D == 128 ? (const void*)monarch_bwd_left_kernel<BF16, 128> : (const void*)monarch_bwd_left_kernel<BF16, 64>;
@@ -644,7 +658,9 @@ int launch_monarch_bwd_dqa(int dtype, int D, int n, int b1, int b2, int AJ, int 
     a.map = map;
     a.ds2_ld = ds2_ld; a.b1 = b1; a.b2 = b2; a.AJ = AJ; a.RR = nf * b1; a.H = H; a.unit0 = unit0;
     a.scale = scale;
-    const dim3 grid((unsigned)((AJ + 3) / 4), (unsigned)n, (unsigned)((b1 + 31) / 32));
+    a.nunits = n;
+    a.nz = (b1 + 31) / 32;
+    const dim3 grid((unsigned)xcd_grid((AJ + 3) / 4 * n * a.nz));
     const size_t ldsb = (size_t)4 * 2 * 32 * 2 * D;
     if (dtype == SFM_BF16) {
         if (D == 128) hipLaunchKernelGGL((monarch_bwd_dqa_kernel<BF16, 128>), grid, dim3(256), ldsb, stream, a);

@@ -125,6 +125,18 @@ struct TokMap {
     }
 };
 
+// Workgroups of a launch go to the eight XCDs in turn (workgroup i to XCD i % 8) and every XCD has its own L2.  A 1-D
+// grid of xcd_grid(total) workgroups that takes its work item from xcd_item(total) gives each XCD one contiguous range
+// of items, so that items which read the same rows (the query blocks of one head, say) meet in one L2.  Items >= total
+// have nothing to do.
+__host__ __device__ __forceinline__ int xcd_grid(int total) { return (total + 7) / 8 * 8; }
+#if defined(__HIPCC__)
+__device__ __forceinline__ int xcd_item(int total) {
+    const int per_xcd = (total + 7) / 8;
+    return (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+}
+#endif
+
 struct MonarchArgs {
     const void* q;
     const void* k;
