@@ -53,3 +53,32 @@ def monarch_fwd_exact_workspace(q, k, v, tiling, heads_per_pass, num_iters=1, on
     torch.cuda.synchronize()
     assert bool((buf[n:] == 0xA5).all()), "bytes behind the workspace were overwritten"
     return out
+
+
+def monarch_bwd_exact_workspace(q, k, v, dout, tiling, heads_per_pass=0, cbf=0):
+    """sfm_monarch_bwd through the C ABI with a workspace of exactly sfm_monarch_bwd_workspace_bytes(heads_per_pass) and
+    64 KiB of canary bytes behind it; returns (dq, dk, dv) after checking that the canary is untouched."""
+    import ctypes as C
+
+    import self_forcing_amd as sfa
+    from self_forcing_amd import lib as L
+
+    f_tied, h_reduce, w_reduce, h, w = tiling
+    dq = torch.empty(q.shape, dtype=torch.float32, device=q.device)
+    dk, dv = torch.empty_like(k), torch.empty_like(v)
+    bd = L.MonarchBwdDesc()
+    bd.fwd = sfa.monarch_attn._desc(q, k, v, dout, f_tied, h_reduce, w_reduce, h, w, q.shape[-1] ** -0.5, 0, cbf)
+    bd.dq_stride = L.strides3(dq)
+    bd.dkv_stride = L.strides3(dk)
+    per_frame = f_tied * (h // h_reduce) * (w // w_reduce)
+    bd.kv_grad_frame_start, bd.kv_grad_frame_end = 0, k.shape[1] // per_frame
+    n = C.c_size_t(0)
+    L.check(L.load().sfm_monarch_bwd_workspace_bytes(C.byref(bd), heads_per_pass, C.byref(n)))
+    pad = 64 * 1024
+    buf = torch.full((n.value + pad,), 0xA5, dtype=torch.uint8, device=q.device)
+    stream = C.c_void_p(torch.cuda.current_stream(q.device).cuda_stream)
+    L.check(L.load().sfm_monarch_bwd(C.byref(bd), q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), dq.data_ptr(),
+                                     dk.data_ptr(), dv.data_ptr(), buf.data_ptr(), n.value, stream))
+    torch.cuda.synchronize()
+    assert bool((buf[n.value:] == 0xA5).all()), "bytes behind the workspace were overwritten"
+    return dq, dk, dv

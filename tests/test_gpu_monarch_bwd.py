@@ -310,3 +310,22 @@ def test_three_frames_tied_480p_blocks_on_the_fused_kernels(saved):
     _close(dq, qr.grad, dtype)
     _close(dk, kr.grad, dtype)
     _close(dv, vr.grad, dtype)
+
+
+@pytest.mark.parametrize("h,w,Fq,Fk,H,hpp", [
+    (4, 52, 3, 5, 3, 0),        # one slab: every fused part, all heads in one pass
+    (40, 12, 2, 3, 3, 2),       # b1 = 40: two query-row slices (two slabs of partial sums), a shorter last pass
+    (90, 8, 1, 2, 2, 1),        # three slices, one head per pass
+    (5, 6, 2, 3, 2, 0),         # b2 = 6: the right factor on the library chain, whose scratch is laid out differently
+])
+def test_backward_stays_inside_an_exactly_sized_workspace(h, w, Fq, Fk, H, hpp):
+    """sfm_monarch_bwd with a workspace of exactly the queried size and canary bytes behind it; the gradients equal the
+    autograd path's, which sizes its own scratch."""
+    from gpu_util import monarch_bwd_exact_workspace
+    dtype, D = torch.bfloat16, 64
+    q0, do = (randn((1, Fq * h * w, H, D), 400 + i, dtype).to(DEV) for i in range(2))
+    k0, v0 = (randn((1, Fk * h * w, H, D), 402 + i, dtype).to(DEV) for i in range(2))
+    dq, dk, dv = monarch_bwd_exact_workspace(q0, k0, v0, do, (1, 1, 1, h, w), hpp)
+    want = mattn._monarch_bwd(q0, k0, v0, do, (1, 1, 1, h, w), D ** -0.5, 0, 0)
+    for got, ref in zip((dq, dk, dv), want):
+        assert torch.equal(got, ref)
