@@ -354,13 +354,15 @@ void monarch_step1_kernel(MonarchArgs p) {
 // ------------------------------------------------------------------------------------------------
 // step 2
 // ------------------------------------------------------------------------------------------------
-// Per wave: two buffers of [Kbar chunk | Y chunk | cl values], a chunk being 32 scratch rows of 2 D bytes, row-major
-// with the 16-byte pieces XOR-swizzled per row as in step 1.
+// Per wave: [Kbar chunk | Y chunk | cl values, two buffers of 256 bytes], a chunk being 32 scratch rows of 2 D bytes,
+// row-major with the 16-byte pieces XOR-swizzled per row as in step 1.  One buffer per matrix: the next chunk's Kbar rows
+// are requested as soon as the logits have read the current ones, its Y rows as soon as the output products have, which
+// keeps a chunk in flight with 17 KB of LDS per wave instead of 33 KB, so that two workgroups share a compute unit
+// (two waves per SIMD, and the 1872 waves of the 480p chunk shape in one round instead of two).
 template <int D>
 struct S2Lds {
     static constexpr int kPitch = 2 * D, kTile = 32 * kPitch;
-    static constexpr int kBuf = 2 * kTile + 256;
-    static constexpr int kWave = 2 * kBuf;
+    static constexpr int kWave = 2 * kTile + 512;
     static __host__ __device__ constexpr size_t bytes() { return 4 * (size_t)kWave; }
 };
 
@@ -369,9 +371,9 @@ __device__ __forceinline__ void s2_load_lds4(const char* base, uint32_t off, uin
 }
 
 // The four waves of a workgroup share nothing: each streams the rows of its own (a, j) through its own part of LDS
-// (global_load_lds_dwordx4, 1 KB contiguous per instruction, one chunk ahead of the one being contracted) and
-// synchronises with its own loads only (vector memory operations complete in order, so waiting until one chunk's
-// worth of them is outstanding means the chunk before has landed).
+// (global_load_lds_dwordx4, 1 KB contiguous per instruction, requested as soon as the buffer's last reader is done) and
+// synchronises with its own loads only (vector memory operations complete in order, so waiting until only the loads
+// issued after a tile's are outstanding means that tile has landed).
 template <class E, int D>
 __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
     using L = S2Lds<D>;
@@ -424,20 +426,6 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
         }
     }
 
-    // chunk n into buffer `buf`: CPR + 1 loads per lane.  Rows past the valid range may hold anything: the last valid
-    // row is read instead (the rows' weights are exactly zero).
-    auto issue = [&](int n, int buf) {
-        const uint32_t dst = lds0 + (uint32_t)buf * L::kBuf;
-#pragma unroll
-        for (int g = 0; g < CPR / 2; ++g) {
-            const int P = g * 64 + lane;
-            const int r = P / CPR, c = (P % CPR) ^ s1_swz<CPR>(r);
-            const uint32_t off = (uint32_t)min(32 * n + r, r_lim - 1) * (2 * D) + (uint32_t)c * 16;
-            s1_load_lds16(kb, off, dst + (uint32_t)g * 1024);
-            s1_load_lds16(yb, off, dst + L::kTile + (uint32_t)g * 1024);
-        }
-        s2_load_lds4(clp, (uint32_t)(32 * n + m) * cl_ld, dst + 2 * L::kTile);     // cl of the chunk's 32 rows (twice)
-    };
     const uint32_t a_off = (uint32_t)m * L::kPitch + (uint32_t)((hf ^ s1_swz<CPR>(m)) << 4);   // Kbar row m as the logits' A operand
     uint32_t tr[DT][2];            // Y^T as the output's A operand: transposing reads, as in step 1
     {
@@ -460,17 +448,34 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
     for (int dt = 0; dt < DT; ++dt) oacc[dt] = kZero;
     float mrun = -INFINITY, lrun = 0.f;
 
-    issue(0, 0);
-    for (int n = 0; n < nch; ++n) {
-        if (n + 1 < nch) {
-            issue(n + 1, (n + 1) & 1);
-            if (D == 128) asm volatile("s_waitcnt vmcnt(17)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
-        } else {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    auto issue_k = [&](int n) {
+#pragma unroll
+        for (int g = 0; g < CPR / 2; ++g) {
+            const int P = g * 64 + lane;
+            const int r = P / CPR, c = (P % CPR) ^ s1_swz<CPR>(r);
+            const uint32_t off = (uint32_t)min(32 * n + r, r_lim - 1) * (2 * D) + (uint32_t)c * 16;
+            s1_load_lds16(kb, off, lds0 + (uint32_t)g * 1024);
         }
-        const char* kt = wl + (n & 1) * L::kBuf;
-        const char* yt = kt + L::kTile;
+        s2_load_lds4(clp, (uint32_t)(32 * n + m) * cl_ld, lds0 + 2 * L::kTile + (uint32_t)(n & 1) * 256);   // lanes >= 32 repeat
+    };
+    auto issue_y = [&](int n) {
+#pragma unroll
+        for (int g = 0; g < CPR / 2; ++g) {
+            const int P = g * 64 + lane;
+            const int r = P / CPR, c = (P % CPR) ^ s1_swz<CPR>(r);
+            const uint32_t off = (uint32_t)min(32 * n + r, r_lim - 1) * (2 * D) + (uint32_t)c * 16;
+            s1_load_lds16(yb, off, lds0 + L::kTile + (uint32_t)g * 1024);
+        }
+    };
+    issue_k(0);
+    issue_y(0);
+    for (int n = 0; n < nch; ++n) {
+        // Kbar and cl of chunk n have landed when only the Y loads issued after them are outstanding
+        if (D == 128) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        const char* kt = wl;
+        const char* yt = wl + L::kTile;
+        const char* clt = wl + 2 * L::kTile + (n & 1) * 256;
 
         f32x16 s;
 #pragma unroll
@@ -480,7 +485,9 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
         }
         f32x4 cc[4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) cc[g] = *(const f32x4*)(kt + 2 * L::kTile + (8 * g + 4 * hf) * 4);
+        for (int g = 0; g < 4; ++g) cc[g] = *(const f32x4*)(clt + (8 * g + 4 * hf) * 4);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // the Kbar tile has been read: the next chunk's may land on it
+        if (n + 1 < nch) issue_k(n + 1);
 
         float mx = -INFINITY;
 #pragma unroll
@@ -510,6 +517,13 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
             pb[st].z = pack2<E>(s[8 * st + 4], s[8 * st + 5]);
             pb[st].w = pack2<E>(s[8 * st + 6], s[8 * st + 7]);
         }
+        // Y of chunk n has landed when only the Kbar / cl loads of chunk n + 1 are outstanding
+        if (n + 1 < nch) {
+            if (D == 128) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
@@ -522,6 +536,8 @@ __global__ __launch_bounds__(256) void monarch_step2_kernel(MonarchArgs p) {
                 oacc[dt] = E::mfma32(ay, pb[st], oacc[dt]);
             }
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // the Y tile has been read
+        if (n + 1 < nch) issue_y(n + 1);
     }
 
     // epilogue: O[i, d] = O^T / l, turned through the wave's LDS (the operand buffers are dead: every load has landed)
